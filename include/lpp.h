@@ -1,0 +1,272 @@
+/*
+ * lpp.h -- C ABI of liblpp_hip.so: the MI355X (gfx950) implementation of the
+ * Lighter++ batch-1 decode path.
+ *
+ * Everything here is plain C: pointers, sizes and scalars, no C++ or HIP types.
+ * Pointers named d_* are DEVICE pointers owned by the caller unless stated.
+ * Every function returns an lpp_status (0 = LPP_OK); nothing aborts the
+ * process.  lpp_last_error() describes the most recent failure on the calling
+ * thread.  Launches are asynchronous on the library's current stream
+ * (lpp_set_stream) and ordered only by stream order, exactly like the
+ * reference's default-stream launches.
+ *
+ * Section A replaces, one for one, the twelve host wrappers declared in the
+ * reference's src/kernels.cuh:24-36 (the operator surface src/model.cpp calls).
+ * Section B replaces the model-level functions of src/model.h:117-164.
+ * Section C is plumbing the reference gets from the CUDA runtime directly.
+ */
+#ifndef LPP_H
+#define LPP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int lpp_status;
+enum {
+    LPP_OK = 0,
+    LPP_ERR_INVALID_ARG = 1, /* null pointer, non-positive size, shape the kernels cannot take */
+    LPP_ERR_HIP = 2,         /* a HIP runtime call failed; see lpp_last_error()                */
+    LPP_ERR_OOM = 3,         /* device or host allocation failed                               */
+    LPP_ERR_STATE = 4,       /* call order violated (e.g. forward before weights are loaded)   */
+    LPP_ERR_UNSUPPORTED = 5  /* valid in the reference, not provided here (e.g. INT4 weights)  */
+};
+
+/* binary16 storage; stands where the reference's signatures say __half. */
+typedef uint16_t lpp_half;
+
+/* Values of the reference's WeightPrecision (src/model.h:8-12). */
+enum { LPP_WEIGHT_FP32 = 0, LPP_WEIGHT_FP16 = 1, LPP_WEIGHT_INT4 = 2 };
+
+/* ===================================================================== */
+/* A. Operator entry points (src/kernels.cuh:24-36)                       */
+/* ===================================================================== */
+
+/* kernels.cuh:24 cuda_convert_f32_to_f16 (matmul.cu:150-161): dst[i] = RN(src[i]). */
+lpp_status lpp_convert_f32_to_f16(lpp_half *d_dst, const float *d_src, int n);
+
+/* kernels.cuh:26 cuda_gemv (matmul.cu:134-147): out[n] = W[n][d] . x[d], W
+ * row-major.  precision LPP_WEIGHT_FP16 reads binary16 weights, anything else
+ * fp32 (the reference's default: branch).  x stays fp32 and accumulation is
+ * fp32; d_workspace is accepted for signature compatibility and never touched. */
+lpp_status lpp_gemv(float *d_out, const float *d_x, const void *d_w, void *d_workspace,
+                    int n, int d, int precision);
+
+/* kernels.cuh:27 cuda_rmsnorm (RMSNorm.cu:11-71): out = x * w / sqrt(mean(x^2) + 1e-5).
+ * d_out may alias d_x. */
+lpp_status lpp_rmsnorm(float *d_out, const float *d_x, const float *d_w, int n);
+
+/* kernels.cuh:28 cuda_rope (rope.cu:7-38): rotate adjacent pairs (2i, 2i+1) of q,
+ * and of k while 2i < kv_dim, by angle pos / base^((2i mod head_size)/head_size).
+ * The cos/sin values are computed on the host with the C library and cached
+ * on the device, so they match a CPU run on the same machine bit for bit. */
+lpp_status lpp_rope(float *d_q, float *d_k, int pos, int dim, int kv_dim, int head_size,
+                    float rope_base);
+
+/* kernels.cuh:29 cuda_swiglu (swiglu.cu:6-33): hb = h1 * sigmoid(h1) * h3; hb may
+ * alias h1 or h3.  Every element is processed (no size %% 4 tail is dropped). */
+lpp_status lpp_swiglu(float *d_hb, const float *d_h1, const float *d_h3, int size);
+
+/* kernels.cuh:30 cuda_softmax_multihead (softmax.cu:5-125): for each of n_heads
+ * rows of stride att_stride, softmax over the first seq_len entries.  d_out may
+ * alias d_x. */
+lpp_status lpp_softmax_multihead(float *d_out, const float *d_x, int n_heads, int seq_len,
+                                 int att_stride);
+
+/* kernels.cuh:31 cuda_scale_multihead (scale.cu:6-21): att[h][t] *= scale, t < seq_len. */
+lpp_status lpp_scale_multihead(float *d_att, float scale, int n_heads, int seq_len,
+                               int att_stride);
+
+/* kernels.cuh:32 cuda_aggregation_multihead (aggregation.cu:6-31):
+ * out[h][i] = sum_{t<seq_len} att[h][t] * V[h/gqa_factor][t][i].  d_v is already
+ * offset to the layer; att_stride is both the att row stride and the cache's
+ * positions-per-head, as in the reference. */
+lpp_status lpp_aggregation_multihead(float *d_out, const lpp_half *d_v, const float *d_att,
+                                     int n_heads, int seq_len, int head_size, int gqa_factor,
+                                     int att_stride);
+
+/* kernels.cuh:33 cuda_residual_add (residual.cu:5-31): out = a + b; out may alias a or b. */
+lpp_status lpp_residual_add(float *d_out, const float *d_a, const float *d_b, int n);
+
+/* kernels.cuh:34 cuda_scatter_kv (scatter_kv.cu:6-26):
+ * cache[layer][h][pos][i] = RN16(k or v[h*head_size + i]), cache shape
+ * [layers][n_kv_heads][seq_len][head_size].  Offsets are computed in 64 bits. */
+lpp_status lpp_scatter_kv(lpp_half *d_key_cache, lpp_half *d_value_cache, const float *d_k,
+                          const float *d_v, int layer, int pos, int n_kv_heads, int head_size,
+                          int seq_len);
+
+/* kernels.cuh:35 cuda_multihead_gemv (multihead_gemv.cu:6-68):
+ * out[h][t] = q_h . K[layer][h/(n_heads/n_kv_heads)][t], t in [0,pos]; d_k_cache is
+ * the cache BASE; out row stride is seq_len; unscaled. */
+lpp_status lpp_multihead_gemv(float *d_out, const float *d_q, const lpp_half *d_k_cache,
+                              int layer, int pos, int n_heads, int n_kv_heads, int head_size,
+                              int seq_len);
+
+/* kernels.cuh:36 cuda_sample (sample.cu:6-214), following the CPU sampler's
+ * semantics (model.cpp:256-303): repetition penalty applied once per occurrence
+ * in history order; temperature 0 returns the lowest index of the maximum;
+ * otherwise logits / temperature, softmax, and the first index whose cumulative
+ * probability exceeds r (vocab_size-1 if none).  r is the uniform draw the
+ * reference's wrapper takes from rand()/RAND_MAX (sample.cu:211); here the caller
+ * supplies it.  topp and d_rng_state are accepted and ignored, as in the
+ * reference.  d_logits is overwritten (penalised and scaled logits, then
+ * probabilities); the 4-byte result lands in d_sampled_token[0]. */
+lpp_status lpp_sample(float *d_logits, int vocab_size, float temperature, float topp,
+                      float penalty, const int *d_history, int history_len,
+                      int *d_sampled_token, unsigned int *d_rng_state, float r);
+
+/* ===================================================================== */
+/* B. Model-level entry points (src/model.h:21-164, src/model.cpp)        */
+/* ===================================================================== */
+
+/* Same fields, order and meaning as Config (src/model.h:21-31). */
+typedef struct lpp_config {
+    int dim;
+    int hidden_dim;
+    int n_layers;
+    int n_heads;
+    int n_kv_heads;
+    int vocab_size;
+    int seq_len;
+    float rope_base;
+    int weight_precision; /* LPP_WEIGHT_FP32 or LPP_WEIGHT_FP16 */
+} lpp_config;
+
+/* Tensor names of transformerWeights (src/model.h:34-55); per-layer tensors are
+ * stacked [n_layers][rows][cols] exactly as the reference's loaders lay them out. */
+enum {
+    LPP_T_TOKEN_EMBEDDING = 0, /* fp32 [vocab][dim]                        */
+    LPP_T_RMS_ATT = 1,         /* fp32 [L][dim]                            */
+    LPP_T_WQ = 2,              /* [L][dim][dim]         weight_precision   */
+    LPP_T_WK = 3,              /* [L][kv_dim][dim]                         */
+    LPP_T_WV = 4,              /* [L][kv_dim][dim]                         */
+    LPP_T_WO = 5,              /* [L][dim][dim]                            */
+    LPP_T_RMS_FFN = 6,         /* fp32 [L][dim]                            */
+    LPP_T_W1 = 7,              /* [L][hidden][dim]  gate                   */
+    LPP_T_W2 = 8,              /* [L][dim][hidden]  down                   */
+    LPP_T_W3 = 9,              /* [L][hidden][dim]  up                     */
+    LPP_T_RMS_FINAL = 10,      /* fp32 [dim]                               */
+    LPP_T_WCLS = 11,           /* [vocab][dim]                             */
+    LPP_T_COUNT = 12
+};
+
+/* Run-state buffers of RunState (src/model.h:96-114), for inspection. */
+enum {
+    LPP_B_X = 0, LPP_B_XB = 1, LPP_B_XB2 = 2, LPP_B_HB = 3, LPP_B_HE = 4, LPP_B_Q = 5,
+    LPP_B_K = 6, LPP_B_V = 7, LPP_B_ATT = 8, LPP_B_LOGITS = 9,
+    LPP_B_KEY_CACHE = 10,  /* binary16 [L][n_kv_heads][seq_len][head_size] */
+    LPP_B_VALUE_CACHE = 11,
+    LPP_B_COUNT = 12
+};
+
+/* How lpp_forward schedules a token. */
+enum {
+    LPP_PATH_OPS = 0,   /* the twelve section-A operators in the reference's call order
+                           (model.cpp:133-160, 216-226, 357-366)                        */
+    LPP_PATH_FUSED = 1, /* fused kernels, one HIP graph per token                        */
+    LPP_PATH_PERSISTENT = 2 /* one persistent kernel per token                           */
+};
+
+typedef struct lpp_model lpp_model;
+
+/* malloc_run_state (model.cpp:18-81) plus device storage for the weights:
+ * allocates, zero-fills the KV cache, keeps everything resident in HBM. */
+lpp_status lpp_model_create(lpp_model **out, const lpp_config *cfg);
+/* free_run_state (model.cpp:83-118) + free_weights_cuda (loader.cpp:181-194). */
+lpp_status lpp_model_destroy(lpp_model *m);
+
+/* Size in bytes the named tensor occupies for this model. */
+lpp_status lpp_model_tensor_bytes(const lpp_model *m, int tensor, size_t *bytes);
+/* Copy host data into (part of) a weight tensor; the upload half of
+ * checkpoint_init_weights / gguf_init_weights (loader.cpp:73-131, 543-637). */
+lpp_status lpp_model_upload(lpp_model *m, int tensor, size_t byte_offset, const void *host_src,
+                            size_t bytes);
+/* loader.cpp:619-632: classifier shares the embedding; for FP16 models this makes
+ * the binary16 copy on the device with lpp_convert_f32_to_f16. */
+lpp_status lpp_model_tie_classifier(lpp_model *m);
+/* Device pointer of a weight tensor / run-state buffer (caller must not free). */
+lpp_status lpp_model_tensor_ptr(lpp_model *m, int tensor, void **d_ptr);
+lpp_status lpp_model_buffer_ptr(lpp_model *m, int buffer, void **d_ptr, size_t *bytes);
+
+lpp_status lpp_model_set_path(lpp_model *m, int path);
+/* Forget the KV cache contents (zero-fill, as malloc_run_state leaves it). */
+lpp_status lpp_model_reset(lpp_model *m);
+
+/* attention (model.cpp:121-160) and transformer_block (:205-226), operator path. */
+lpp_status lpp_attention(lpp_model *m, int layer, int pos);
+lpp_status lpp_transformer_block(lpp_model *m, int layer, int pos);
+
+/* forward (model.cpp:342-371): embed token, run every layer at position pos, final
+ * norm, classifier, sample; returns the sampled id in *next_token after the 4-byte
+ * device-to-host copy (the only synchronisation).  r is the uniform draw for the
+ * sampler (ignored when temperature == 0).  The logits of this step remain
+ * readable through LPP_B_LOGITS until the next call (raw, before the sampler
+ * touches them, on the fused paths; sampler-mutated on LPP_PATH_OPS, as in the
+ * reference). */
+lpp_status lpp_forward(lpp_model *m, int token, int pos, float temperature, float topp,
+                       float penalty, const int *history, int history_len, float r,
+                       int *next_token);
+
+/* Timing filled by lpp_generate. */
+typedef struct lpp_gen_stats {
+    double wall_seconds;   /* steady_clock around the generation loop, D2H per token included */
+    double device_ms;      /* HIP events on the launch stream around the same loop           */
+    double kernel_ms_sum;  /* sum of per-token event pairs around the dominant kernel        */
+    int    kernel_launches;
+    int    tokens;
+} lpp_gen_stats;
+
+/* Generation loop of src/main.cpp:158-223 without text: starting from
+ * first_token at start_pos, run n_steps forwards, feeding each sampled token
+ * back and keeping the sliding penalty window (capacity history_cap; initial
+ * contents history[0..*history_len)).  uniforms[n_steps] supplies r per step.
+ * out_tokens[n_steps] receives the sampled ids.  No EOS stop. */
+lpp_status lpp_generate(lpp_model *m, int first_token, int start_pos, int n_steps,
+                        float temperature, float topp, float penalty, int *history,
+                        int *history_len, int history_cap, const float *uniforms,
+                        int *out_tokens, lpp_gen_stats *stats);
+
+/* ===================================================================== */
+/* C. Runtime plumbing                                                    */
+/* ===================================================================== */
+
+const char *lpp_last_error(void);
+const char *lpp_version(void);
+lpp_status lpp_device_count(int *count);
+/* Select the device and create the library's stream; idempotent. */
+lpp_status lpp_init(int device);
+/* Launch on a caller-owned hipStream_t (passed as void*); NULL restores the
+ * library's own stream. */
+lpp_status lpp_set_stream(void *hip_stream);
+lpp_status lpp_get_stream(void **hip_stream);
+lpp_status lpp_synchronize(void);
+lpp_status lpp_malloc(void **d_ptr, size_t bytes);
+lpp_status lpp_free(void *d_ptr);
+lpp_status lpp_memset(void *d_ptr, int value, size_t bytes);
+lpp_status lpp_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes);
+lpp_status lpp_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes);
+lpp_status lpp_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes);
+/* Device facts used by the benchmark report. */
+lpp_status lpp_device_info(char *name, size_t name_cap, int *compute_units, size_t *hbm_bytes);
+
+/* Deterministic synthetic tensors (host side): element i of a stream named by
+ * seed is N(0, std) from a counter-based generator (splitmix64 -> Box-Muller in
+ * double), so any slice can be produced independently.  _f16 rounds to nearest
+ * even binary16. */
+lpp_status lpp_synth_normal_f32(float *h_dst, size_t n, uint64_t seed, uint64_t first_index,
+                                float std);
+lpp_status lpp_synth_normal_f16(lpp_half *h_dst, size_t n, uint64_t seed, uint64_t first_index,
+                                float std);
+lpp_status lpp_synth_uniform_f32(float *h_dst, size_t n, uint64_t seed, uint64_t first_index);
+lpp_status lpp_synth_token_ids(int *h_dst, size_t n, uint64_t seed, int vocab_size);
+/* Exact widening / RN narrowing on the host (loader.cpp:346-379 and its inverse). */
+lpp_status lpp_f16_to_f32_host(float *h_dst, const lpp_half *h_src, size_t n);
+lpp_status lpp_f32_to_f16_host(lpp_half *h_dst, const float *h_src, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LPP_H */

@@ -1,0 +1,647 @@
+// decode_phases.hpp -- the per-token schedule of forward() (reference
+// src/model.cpp:342-371 -> transformer_block :205-226 -> attention :121-160) cut
+// into phases.  Between two phases every workgroup needs results of all others
+// (a full activation vector); inside a phase workgroups are independent.
+//
+//   qkv      rmsnorm(x)        -> q,k,v GEMV -> RoPE -> q buffer, K/V cache  (fuses :216,:133-141)
+//   attend   scores, softmax, value aggregation over the cache -> xb          (fuses :146-157)
+//   oproj    Wo.xb + x -> x                                                   (fuses :160,:218)
+//   gateup   rmsnorm(x)        -> W1,W3 GEMV -> SwiGLU -> hb                  (fuses :221-224)
+//   down     W2.hb + x -> x                                                   (fuses :225-226)
+//   lmhead   rmsnorm(x)        -> classifier GEMV -> logits                   (fuses :357-358)
+//   sample   four short steps over vocabulary chunks + one bookkeeping step   (:366-370)
+//
+// Each phase is a __device__ function of (workgroup index, workgroup count), so
+// the same code runs as one launch per phase (a HIP graph of kernels) or inside
+// one persistent kernel with grid barriers in between.  GEMV phases issue their
+// first weight loads BEFORE calling the `pre` hook that waits for the previous
+// phase and stages the activations in LDS: weights never depend on activations,
+// so HBM keeps streaming across the phase boundary.
+#pragma once
+
+#include "lpp_device.hpp"
+#include "lpp_model.hpp"
+#include "sampler.hpp"
+
+namespace lpp {
+namespace ph {
+
+using namespace dev;
+
+struct DecodeArgs {
+    int dim, hidden, n_layers, n_heads, n_kv_heads, head_size, kv_dim, vocab, seq_len, gqa;
+    int max_splits;
+    // weights (stacked per layer), see lpp_model
+    const float* emb;
+    const float* rms_att;
+    const char* wq;
+    const char* wk;
+    const char* wv;
+    const char* wo;
+    const float* rms_ffn;
+    const char* w1;
+    const char* w2;
+    const char* w3;
+    const float* rms_final;
+    const char* wcls;
+    // run state
+    float* x;
+    float* xb;
+    float* q;
+    float* k;
+    float* v;
+    float* hb;
+    float* logits;
+    float* work;           // sampler working copy of the logits
+    uint16_t* key_cache;
+    uint16_t* value_cache;
+    float* att_partial;    // [n_heads][max_splits][head_size + 2]
+    unsigned* att_count;   // [n_kv_heads] arrival counters of the split combine
+    const float2* rope;    // [seq_len][head_size/2]
+    StepParams* step;
+    int* history;          // ring of step->history_cap entries
+    const float* uniforms; // per-step draws, or null: use step->r
+    int* out_tokens;       // per-step results, or null
+    int* sampled;          // [1]
+    smp::SampleScratch sample_scratch;
+};
+
+// ---------------------------------------------------------------------------
+// Activation staging
+// ---------------------------------------------------------------------------
+
+// xs[0..n) = src, zero padded to a multiple of 8.
+__device__ __forceinline__ void stage_plain(float* xs, const float* src, int n) {
+    const int n_pad = (n + 7) & ~7;
+    for (int i = threadIdx.x; i < n_pad; i += blockDim.x) xs[i] = (i < n) ? src[i] : 0.0f;
+    __syncthreads();
+}
+
+// xs = rmsnorm(src) * gain, ops.cpp:20-32: (x * s) * w with s = 1/sqrtf(mean + 1e-5f).
+__device__ __forceinline__ void stage_rmsnorm(float* xs, const float* src, const float* gain, int n) {
+#pragma clang fp contract(off)
+    __shared__ float scratch[16];
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = src[i];
+        xs[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    ss /= static_cast<float>(n);
+    ss += 1e-5f;
+    const float scale = 1.0f / sqrtf(ss);
+    const int n_pad = (n + 7) & ~7;
+    for (int i = threadIdx.x; i < n_pad; i += blockDim.x) xs[i] = (i < n) ? xs[i] * scale * gain[i] : 0.0f;
+    __syncthreads();
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined row-tile GEMV
+// ---------------------------------------------------------------------------
+
+template <bool kF16, int kRows, int kUnroll>
+struct Tile {
+    static constexpr int kPer = WTraits<kF16>::kPerLoad;
+    static constexpr int kChunk = kWave * kPer;
+    uintx4 w[kUnroll][kRows];
+
+    __device__ __forceinline__ void load(const char* const (&rows)[kRows], int cg, int d) {
+        const int lane = lane_id();
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int col = (cg * kUnroll + u) * kChunk + lane * kPer;
+            const bool live = col < d;
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                if (live && rows[r] != nullptr)
+                    w[u][r] = load16_stream(rows[r] + static_cast<size_t>(col) * WTraits<kF16>::kBytes);
+                else
+                    w[u][r] = uintx4{0u, 0u, 0u, 0u};
+            }
+        }
+    }
+
+    __device__ __forceinline__ void fma(const float* xs, int cg, int d, float (&acc)[kRows]) const {
+        const int lane = lane_id();
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int col = (cg * kUnroll + u) * kChunk + lane * kPer;
+            if (col < d) {
+                if constexpr (kF16) {
+                    const floatx4 xa = *reinterpret_cast<const floatx4*>(xs + col);
+                    const floatx4 xb = *reinterpret_cast<const floatx4*>(xs + col + 4);
+#pragma unroll
+                    for (int r = 0; r < kRows; ++r) acc[r] = dot8(w[u][r], xa, xb, acc[r]);
+                } else {
+                    const floatx4 xa = *reinterpret_cast<const floatx4*>(xs + col);
+#pragma unroll
+                    for (int r = 0; r < kRows; ++r) acc[r] = dot4(w[u][r], xa, acc[r]);
+                }
+            }
+        }
+    }
+};
+
+// One wavefront walks tiles wave_g, wave_g + waves_total, ...; a tile is kRows
+// rows given by row_ptr(tile, r) (null = no such row) and is consumed in groups
+// of kUnroll 1-KiB chunks.  While group g is multiplied, group g+1 (possibly of
+// the next tile) is already in flight.  pre() runs once, after the first loads
+// have been issued and before anything reads xs; every wavefront of the
+// workgroup calls it, with or without work.  epi(tile, sums) receives
+// wave-uniform dot products.
+template <bool kF16, int kRows, int kUnroll, class RowFn, class EpiFn, class PreFn>
+__device__ __forceinline__ void gemv_phase(int ntiles, int d, const float* xs, int wave_g, int waves_total,
+                                           RowFn row_ptr, EpiFn epi, PreFn pre) {
+    using T = Tile<kF16, kRows, kUnroll>;
+    const int ncg = (d + T::kChunk * kUnroll - 1) / (T::kChunk * kUnroll);
+    T a, b;
+    int tile = wave_g, cg = 0;
+    bool have = tile < ntiles && ncg > 0;
+    const char* rows[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) rows[r] = have ? row_ptr(tile, r) : nullptr;
+    if (have) a.load(rows, 0, d);
+    pre();
+    float acc[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) acc[r] = 0.0f;
+
+#define LPP_GEMV_STEP(CUR, NXT)                                                   \
+    {                                                                             \
+        int ntile = tile, ncgi = cg + 1;                                          \
+        if (ncgi == ncg) {                                                        \
+            ncgi = 0;                                                             \
+            ntile = tile + waves_total;                                           \
+        }                                                                         \
+        const bool nhave = ntile < ntiles;                                        \
+        const char* nrows[kRows];                                                 \
+        _Pragma("unroll") for (int r = 0; r < kRows; ++r) nrows[r] = rows[r];     \
+        if (nhave) {                                                              \
+            if (ncgi == 0) {                                                      \
+                _Pragma("unroll") for (int r = 0; r < kRows; ++r) nrows[r] = row_ptr(ntile, r); \
+            }                                                                     \
+            NXT.load(nrows, ncgi, d);                                             \
+        }                                                                         \
+        CUR.fma(xs, cg, d, acc);                                                  \
+        if (ncgi == 0) {                                                          \
+            float sums[kRows];                                                    \
+            _Pragma("unroll") for (int r = 0; r < kRows; ++r) {                   \
+                sums[r] = wave_sum(acc[r]);                                       \
+                acc[r] = 0.0f;                                                    \
+            }                                                                     \
+            epi(tile, sums);                                                      \
+        }                                                                         \
+        tile = ntile;                                                             \
+        cg = ncgi;                                                                \
+        have = nhave;                                                             \
+        _Pragma("unroll") for (int r = 0; r < kRows; ++r) rows[r] = nrows[r];     \
+    }
+    while (have) {
+        LPP_GEMV_STEP(a, b)
+        if (!have) break;
+        LPP_GEMV_STEP(b, a)
+    }
+#undef LPP_GEMV_STEP
+}
+
+__device__ __forceinline__ const char* row_at(const char* base, size_t layer_rows, int layer, int row, int d,
+                                              int wbytes) {
+    return base + (static_cast<size_t>(layer) * layer_rows + static_cast<size_t>(row)) * d * wbytes;
+}
+
+// Input of layer 0 is the embedding row of the current token (model.cpp:345-349);
+// later layers read x.
+__device__ __forceinline__ const float* layer_input(const DecodeArgs& a, int layer) {
+    return layer == 0 ? a.emb + static_cast<size_t>(a.step->token) * a.dim : a.x;
+}
+
+// ---------------------------------------------------------------------------
+// Phase: rmsnorm -> QKV -> RoPE -> q buffer and K/V cache
+// ---------------------------------------------------------------------------
+template <bool kF16, int kRows, class PreFn>
+__device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg, int nwg, float* xs, PreFn pre) {
+#pragma clang fp contract(off)
+    static_assert(kRows % 2 == 0, "RoPE pairs must stay inside a tile");
+    const int wbytes = kF16 ? 2 : 4;
+    const int waves_per_wg = static_cast<int>(blockDim.x) / kWave;
+    const int wave_g = wg * waves_per_wg + wave_index();
+    const int total_rows = a.dim + 2 * a.kv_dim;
+    const int ntiles = (total_rows + kRows - 1) / kRows;
+    const int dim = a.dim, kv_dim = a.kv_dim;
+
+    auto row_ptr = [&](int tile, int r) -> const char* {
+        const int g = tile * kRows + r;
+        if (g < dim) return row_at(a.wq, dim, layer, g, dim, wbytes);
+        if (g < dim + kv_dim) return row_at(a.wk, kv_dim, layer, g - dim, dim, wbytes);
+        if (g < total_rows) return row_at(a.wv, kv_dim, layer, g - dim - kv_dim, dim, wbytes);
+        return nullptr;
+    };
+    auto prologue = [&]() {
+        pre();
+        stage_rmsnorm(xs, layer_input(a, layer), a.rms_att + static_cast<size_t>(layer) * dim, dim);
+    };
+    auto epilogue = [&](int tile, float (&sums)[kRows]) {
+        if (lane_id() != 0) return;
+        const int pos = a.step->pos;
+        const int hs = a.head_size;
+        const float2* cs_row = a.rope + static_cast<size_t>(pos) * (hs / 2);
+#pragma unroll
+        for (int r = 0; r < kRows; r += 2) {
+            const int g = tile * kRows + r;
+            if (g >= total_rows) break;
+            float e0 = sums[r], e1 = sums[r + 1];
+            if (g < dim + kv_dim) {
+                // ops.cpp:36-52 on the pair (i, i+1); i is the index inside q or k.
+                const int i = (g < dim) ? g : g - dim;
+                const float2 cs = cs_row[(i % hs) >> 1];
+                const float r0 = e0 * cs.x - e1 * cs.y;
+                const float r1 = e0 * cs.y + e1 * cs.x;
+                e0 = r0;
+                e1 = r1;
+            }
+            if (g < dim) {
+                a.q[g] = e0;
+                a.q[g + 1] = e1;
+            } else {
+                // model.cpp:171-176 / scatter_kv.cu:15-18.
+                const bool is_k = g < dim + kv_dim;
+                const int i = is_k ? g - dim : g - dim - kv_dim;
+                const int head = i / hs, within = i - head * hs;
+                const size_t dst = static_cast<size_t>(layer) * kv_dim * a.seq_len +
+                                   static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(pos) * hs + within;
+                float* plain = is_k ? a.k : a.v;
+                uint16_t* cache = is_k ? a.key_cache : a.value_cache;
+                plain[i] = e0;
+                plain[i + 1] = e1;
+                cache[dst] = f32_to_f16_bits(e0);
+                cache[dst + 1] = f32_to_f16_bits(e1);
+            }
+        }
+    };
+    gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
+}
+
+// ---------------------------------------------------------------------------
+// Phase: out = W . xs + residual   (O projection and down projection)
+// ---------------------------------------------------------------------------
+template <bool kF16, int kRows, class PreFn>
+__device__ __forceinline__ void phase_proj_residual(const char* w_layer, int n, int d, const float* src,
+                                                    const float* residual, float* out, int wg, int nwg,
+                                                    float* xs, PreFn pre) {
+    const int wbytes = kF16 ? 2 : 4;
+    const int waves_per_wg = static_cast<int>(blockDim.x) / kWave;
+    const int wave_g = wg * waves_per_wg + wave_index();
+    const int ntiles = (n + kRows - 1) / kRows;
+    auto row_ptr = [&](int tile, int r) -> const char* {
+        const int g = tile * kRows + r;
+        return g < n ? w_layer + static_cast<size_t>(g) * d * wbytes : nullptr;
+    };
+    auto prologue = [&]() {
+        pre();
+        stage_plain(xs, src, d);
+    };
+    auto epilogue = [&](int tile, float (&sums)[kRows]) {
+        const int lane = lane_id();
+        if (lane >= kRows) return;
+        const int g = tile * kRows + lane;
+        if (g >= n) return;
+        float v = sums[0];
+#pragma unroll
+        for (int r = 1; r < kRows; ++r)
+            if (lane == r) v = sums[r];
+        out[g] = residual[g] + v;  // model.cpp:232,239: x[i] += xb2[i]
+    };
+    gemv_phase<kF16, kRows, 4>(ntiles, d, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
+}
+
+// ---------------------------------------------------------------------------
+// Phase: rmsnorm -> gate/up -> SwiGLU -> hb
+// ---------------------------------------------------------------------------
+template <bool kF16, int kPairRows, class PreFn>
+__device__ __forceinline__ void phase_gateup(const DecodeArgs& a, int layer, int wg, int nwg, float* xs, PreFn pre) {
+#pragma clang fp contract(off)
+    constexpr int kRows = 2 * kPairRows;
+    const int wbytes = kF16 ? 2 : 4;
+    const int waves_per_wg = static_cast<int>(blockDim.x) / kWave;
+    const int wave_g = wg * waves_per_wg + wave_index();
+    const int hidden = a.hidden, dim = a.dim;
+    const int ntiles = (hidden + kPairRows - 1) / kPairRows;
+    auto row_ptr = [&](int tile, int r) -> const char* {
+        const int g = tile * kPairRows + (r % kPairRows);
+        if (g >= hidden) return nullptr;
+        return row_at(r < kPairRows ? a.w1 : a.w3, hidden, layer, g, dim, wbytes);
+    };
+    auto prologue = [&]() {
+        pre();
+        stage_rmsnorm(xs, a.x, a.rms_ffn + static_cast<size_t>(layer) * dim, dim);
+    };
+    auto epilogue = [&](int tile, float (&sums)[kRows]) {
+        const int lane = lane_id();
+        if (lane >= kPairRows) return;
+        const int g = tile * kPairRows + lane;
+        if (g >= hidden) return;
+        float gate = sums[0], up = sums[kPairRows];
+#pragma unroll
+        for (int r = 1; r < kPairRows; ++r)
+            if (lane == r) {
+                gate = sums[r];
+                up = sums[kPairRows + r];
+            }
+        // ops.cpp:80-85
+        const float sigma = 1.0f / (1.0f + expf(-gate));
+        a.hb[g] = (gate * sigma) * up;
+    };
+    gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
+}
+
+// ---------------------------------------------------------------------------
+// Phase: final rmsnorm -> classifier -> logits
+// ---------------------------------------------------------------------------
+template <bool kF16, int kRows, class PreFn>
+__device__ __forceinline__ void phase_lmhead(const DecodeArgs& a, int wg, int nwg, float* xs, PreFn pre) {
+    const int wbytes = kF16 ? 2 : 4;
+    const int waves_per_wg = static_cast<int>(blockDim.x) / kWave;
+    const int wave_g = wg * waves_per_wg + wave_index();
+    const int vocab = a.vocab, dim = a.dim;
+    const int ntiles = (vocab + kRows - 1) / kRows;
+    auto row_ptr = [&](int tile, int r) -> const char* {
+        const int g = tile * kRows + r;
+        return g < vocab ? a.wcls + static_cast<size_t>(g) * dim * wbytes : nullptr;
+    };
+    auto prologue = [&]() {
+        pre();
+        stage_rmsnorm(xs, a.x, a.rms_final, dim);
+    };
+    auto epilogue = [&](int tile, float (&sums)[kRows]) {
+        const int lane = lane_id();
+        if (lane >= kRows) return;
+        const int g = tile * kRows + lane;
+        if (g >= vocab) return;
+        float v = sums[0];
+#pragma unroll
+        for (int r = 1; r < kRows; ++r)
+            if (lane == r) v = sums[r];
+        a.logits[g] = v;
+    };
+    gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
+}
+
+// ---------------------------------------------------------------------------
+// Phase: attention over the cache (split context)
+// ---------------------------------------------------------------------------
+
+// Number of context splits in use at this position: about 64 positions each.
+__device__ __forceinline__ int active_splits(int npos, int max_splits) {
+    int s = (npos + 63) / 64;
+    return s < 1 ? 1 : (s > max_splits ? max_splits : s);
+}
+
+template <int kGroup>
+__device__ __forceinline__ float group_sum(float v) {
+    if constexpr (kGroup >= 2) v += dpp_move<kDppXor1>(v);
+    if constexpr (kGroup >= 4) v += dpp_move<kDppXor2>(v);
+    if constexpr (kGroup >= 8) v += dpp_move<kDppHalfMirror>(v);
+    if constexpr (kGroup >= 16) v += dpp_move<kDppMirror>(v);
+    return v;
+}
+
+// Device-coherent read of a value another workgroup published before a fence.
+__device__ __forceinline__ float coherent_load(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr int kAttBlock = 512;   // positions per softmax sub-block
+constexpr int kMaxGqa = 8;       // query heads per KV head held in registers
+
+// LDS floats the attention phase needs.
+__host__ __device__ inline int attention_lds_floats(int gqa, int head_size, int nthreads) {
+    const int hs_pad = (head_size + 7) & ~7;
+    return gqa * hs_pad              // q
+           + gqa * kAttBlock         // scores / probabilities of one sub-block
+           + 3 * gqa                 // running max, running sum, correction
+           + (nthreads / kWave) * gqa * hs_pad;  // cross-wave reduction
+}
+
+// One work item: KV head `kvh`, context split `split` of `nsplits`.  kGroup lanes
+// cover one position (8 binary16 each).  Sub-blocks of kAttBlock positions:
+// scores -> LDS, per-head max/exp/sum by one wavefront per head, then V
+// accumulation with the running-max correction (the sum the CPU forms at
+// model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped).  The partial
+// (max, sum, unnormalised output) goes to att_partial; the last split to arrive
+// for this KV head combines all splits into xb.
+template <int kGroup>
+__device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int split, int nsplits, int npos,
+                               float* lds) {
+    const int hs = a.head_size, gqa = a.gqa;
+    const int hs_pad = kGroup * 8;
+    const int nthreads = static_cast<int>(blockDim.x);
+    const int nwaves = nthreads / kWave;
+    const int ngroups = nthreads / kGroup;
+    const int tid = static_cast<int>(threadIdx.x);
+    const int sub = tid % kGroup, grp = tid / kGroup;
+    const int wave = tid / kWave;
+
+    float* qs = lds;                          // [gqa][hs_pad]
+    float* sc = qs + gqa * hs_pad;            // [gqa][kAttBlock]
+    float* run_max = sc + gqa * kAttBlock;    // [gqa]
+    float* run_sum = run_max + gqa;           // [gqa]
+    float* corr = run_sum + gqa;              // [gqa]
+    float* red = corr + gqa;                  // [nwaves][gqa][hs_pad]
+
+    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
+    for (int i = tid; i < gqa * hs_pad; i += nthreads) {
+        const int qh = i / hs_pad, e = i - qh * hs_pad;
+        qs[i] = (e < hs) ? a.q[static_cast<size_t>(kvh * gqa + qh) * hs + e] : 0.0f;
+    }
+    if (tid < gqa) {
+        run_max[tid] = -INFINITY;
+        run_sum[tid] = 0.0f;
+    }
+    const int chunk = (npos + nsplits - 1) / nsplits;
+    const int t_begin = split * chunk;
+    const int t_end = min(npos, t_begin + chunk);
+    const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
+    const uint16_t* kbase = a.key_cache + head_base;
+    const uint16_t* vbase = a.value_cache + head_base;
+
+    float acc[kMaxGqa][8];
+#pragma unroll
+    for (int qh = 0; qh < kMaxGqa; ++qh)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[qh][e] = 0.0f;
+    __syncthreads();
+
+    for (int b0 = t_begin; b0 < t_end; b0 += kAttBlock) {
+        const int b1 = min(t_end, b0 + kAttBlock);
+        // scores of this sub-block
+        for (int t = b0 + grp; t < b1; t += ngroups) {
+            uintx4 kb = uintx4{0u, 0u, 0u, 0u};
+            if (sub * 8 < hs) kb = load16(kbase + static_cast<size_t>(t) * hs + sub * 8);
+#pragma unroll
+            for (int qh = 0; qh < kMaxGqa; ++qh) {
+                if (qh < gqa) {
+                    const float* qv = qs + qh * hs_pad + sub * 8;
+                    const floatx4 xa = *reinterpret_cast<const floatx4*>(qv);
+                    const floatx4 xb = *reinterpret_cast<const floatx4*>(qv + 4);
+                    const float s = group_sum<kGroup>(dot8(kb, xa, xb, 0.0f));
+                    if (sub == 0) sc[qh * kAttBlock + (t - b0)] = s * scale;
+                }
+            }
+        }
+        __syncthreads();
+        // per head: new running max, probabilities, running sum, correction
+        for (int qh = wave; qh < gqa; qh += nwaves) {
+            float* row = sc + qh * kAttBlock;
+            const int n = b1 - b0;
+            float m = -INFINITY;
+            for (int i = lane_id(); i < n; i += kWave) m = fmaxf(m, row[i]);
+            m = wave_max(m);
+            const float m_old = run_max[qh];
+            const float m_new = fmaxf(m_old, m);
+            float l = 0.0f;
+            for (int i = lane_id(); i < n; i += kWave) {
+                const float p = expf(row[i] - m_new);
+                row[i] = p;
+                l += p;
+            }
+            l = wave_sum(l);
+            if (lane_id() == 0) {
+                const float c = (m_old == -INFINITY) ? 0.0f : expf(m_old - m_new);
+                corr[qh] = c;
+                run_sum[qh] = run_sum[qh] * c + l;
+                run_max[qh] = m_new;
+            }
+        }
+        __syncthreads();
+        // value accumulation
+#pragma unroll
+        for (int qh = 0; qh < kMaxGqa; ++qh) {
+            if (qh < gqa) {
+                const float c = corr[qh];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[qh][e] *= c;
+            }
+        }
+        if (sub * 8 < hs) {
+            for (int t = b0 + grp; t < b1; t += ngroups) {
+                const half8_t vv = as_half8(load16(vbase + static_cast<size_t>(t) * hs + sub * 8));
+#pragma unroll
+                for (int qh = 0; qh < kMaxGqa; ++qh) {
+                    if (qh < gqa) {
+                        const float p = sc[qh * kAttBlock + (t - b0)];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc[qh][e] = fmaf(static_cast<float>(vv[e]), p, acc[qh][e]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // Reduce the per-group partial outputs: across the groups of a wavefront by
+    // lane exchange, across wavefronts through LDS in wave order.
+#pragma unroll
+    for (int qh = 0; qh < kMaxGqa; ++qh) {
+        if (qh < gqa) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float v = acc[qh][e];
+#pragma unroll
+                for (int off = kGroup; off < kWave; off <<= 1) v += __shfl_xor(v, off);
+                acc[qh][e] = v;
+            }
+            if (lane_id() < kGroup) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) red[(wave * gqa + qh) * hs_pad + sub * 8 + e] = acc[qh][e];
+            }
+        }
+    }
+    __syncthreads();
+    const int stride = hs + 2;
+    for (int i = tid; i < gqa * hs; i += nthreads) {
+        const int qh = i / hs, e = i - qh * hs;
+        float o = 0.0f;
+        for (int w = 0; w < nwaves; ++w) o += red[(w * gqa + qh) * hs_pad + e];
+        float* part = a.att_partial + (static_cast<size_t>(kvh * gqa + qh) * a.max_splits + split) * stride;
+        part[e] = o;
+        if (e == 0) {
+            part[hs] = run_max[qh];
+            part[hs + 1] = run_sum[qh];
+        }
+    }
+
+    // Last split to arrive combines.
+    __shared__ int is_last;
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned ticket = atomicAdd(&a.att_count[kvh], 1u);
+        is_last = (ticket == static_cast<unsigned>(nsplits - 1)) ? 1 : 0;
+        if (is_last) a.att_count[kvh] = 0u;  // ready for the next layer
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    for (int i = tid; i < gqa * hs; i += nthreads) {
+        const int qh = i / hs, e = i - qh * hs;
+        const float* base = a.att_partial + static_cast<size_t>(kvh * gqa + qh) * a.max_splits * stride;
+        float top = -INFINITY;
+        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, coherent_load(base + s * stride + hs));
+        float o = 0.0f, l = 0.0f;
+        for (int s = 0; s < nsplits; ++s) {
+            const float ms = coherent_load(base + s * stride + hs);
+            const float wgt = (ms == -INFINITY) ? 0.0f : expf(ms - top);
+            o += coherent_load(base + s * stride + e) * wgt;
+            l += coherent_load(base + s * stride + hs + 1) * wgt;
+        }
+        a.xb[static_cast<size_t>(kvh * gqa + qh) * hs + e] = o / l;
+    }
+}
+
+template <class PreFn>
+__device__ __forceinline__ void phase_attention(const DecodeArgs& a, int layer, int wg, int nwg, float* lds,
+                                                PreFn pre) {
+    pre();
+    const int npos = a.step->pos + 1;
+    const int nsplits = active_splits(npos, a.max_splits);
+    const int items = a.n_kv_heads * nsplits;
+    const int hs = a.head_size;
+    for (int item = wg; item < items; item += nwg) {
+        const int kvh = item / nsplits, split = item - kvh * nsplits;
+        if (hs <= 8) attention_item<1>(a, layer, kvh, split, nsplits, npos, lds);
+        else if (hs <= 16) attention_item<2>(a, layer, kvh, split, nsplits, npos, lds);
+        else if (hs <= 32) attention_item<4>(a, layer, kvh, split, nsplits, npos, lds);
+        else if (hs <= 64) attention_item<8>(a, layer, kvh, split, nsplits, npos, lds);
+        else attention_item<16>(a, layer, kvh, split, nsplits, npos, lds);
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Sampler steps (see sampler.hpp) and the end-of-token bookkeeping
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ float step_uniform(const DecodeArgs& a) {
+    return a.uniforms ? a.uniforms[a.step->step_index] : a.step->r;
+}
+
+// After the sampler: publish the token, feed it back as the next input, advance
+// the position and the penalty window (src/main.cpp:200-208; the window is kept
+// as a ring because the penalty does not depend on the order of its entries).
+__device__ __forceinline__ void finish_token(const DecodeArgs& a, int token) {
+    StepParams* sp = a.step;
+    a.sampled[0] = token;
+    if (a.out_tokens) a.out_tokens[sp->step_index] = token;
+    if (sp->history_cap > 0) {
+        a.history[sp->history_next] = token;
+        sp->history_next = (sp->history_next + 1) % sp->history_cap;
+        if (sp->history_len < sp->history_cap) sp->history_len += 1;
+    }
+    sp->token = token;
+    sp->pos += 1;
+    sp->step_index += 1;
+}
+
+}  // namespace ph
+}  // namespace lpp

@@ -1,0 +1,98 @@
+// lpp_model.hpp -- the model object behind section B of lpp.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "lpp_internal.hpp"
+
+// Everything forward() touches, resident in HBM.  Field names follow
+// transformerWeights and RunState (reference src/model.h:34-115).
+namespace lpp {
+struct StepParams;
+}
+
+struct lpp_model {
+    lpp_config cfg{};
+    int kv_dim = 0;
+    int head_size = 0;
+    int gqa = 0;
+    int path = LPP_PATH_OPS;
+
+    // Weights, stacked per layer: [L][rows][cols].  Matrices are binary16 or fp32
+    // according to cfg.weight_precision; embedding and norm gains are fp32.
+    void* w[LPP_T_COUNT] = {};
+    size_t w_bytes[LPP_T_COUNT] = {};
+    bool w_loaded[LPP_T_COUNT] = {};
+
+    // Run state (model.h:96-114).
+    float* x = nullptr;
+    float* xb = nullptr;
+    float* xb2 = nullptr;
+    float* hb = nullptr;
+    float* he = nullptr;
+    float* q = nullptr;
+    float* k = nullptr;
+    float* v = nullptr;
+    float* att = nullptr;
+    float* logits = nullptr;
+    uint16_t* key_cache = nullptr;    // [L][n_kv_heads][seq_len][head_size]
+    uint16_t* value_cache = nullptr;
+    void* workspace_f16 = nullptr;    // kept for the operator signature; unused
+    int* sampled_token = nullptr;     // [1]
+    int* history = nullptr;           // [seq_len]
+
+    // Fused paths: per-token scalars live on the device so that a recorded
+    // graph can be replayed without touching its nodes.
+    struct lpp::StepParams* step = nullptr;       // device
+    struct lpp::StepParams* step_host = nullptr;  // pinned host mirror
+    int* pinned_tokens = nullptr;            // pinned host landing area for sampled ids
+    int pinned_tokens_cap = 0;
+    float* att_partial = nullptr;            // split-context attention partials
+    float* work_logits = nullptr;            // sampler working copy of the logits
+    unsigned* sync_words = nullptr;          // arrival counters (attention combine, grid barrier)
+    float* sample_scratch = nullptr;         // 4 x kMaxChunks words
+    float* gen_uniforms = nullptr;           // device copy of the per-step draws
+    int* gen_tokens = nullptr;               // device per-step results
+    int gen_cap = 0;
+    const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
+    int max_splits = 1;
+    bool fused_ok = false;                   // shape supported by the fused kernels
+    char fused_why[160] = "";
+
+    hipGraphExec_t graph_exec[2] = {nullptr, nullptr};  // [0] without, [1] with uniforms/out arrays
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+    hipEvent_t ev_tok[2] = {nullptr, nullptr};
+};
+
+namespace lpp {
+
+// Per-token scalars the fused kernels read from device memory, so that a
+// recorded graph can be replayed without touching its nodes.
+struct StepParams {
+    int token;         // input token id; replaced by the sampled id at the end of the step
+    int pos;           // position of this token; advanced at the end of the step
+    int history_len;   // valid entries in the device penalty window
+    int history_cap;   // capacity of the window (0: no window kept)
+    int history_next;  // ring slot the next sampled id goes to
+    int step_index;    // index into uniforms[] / out_tokens[]
+    float temperature;
+    float penalty;
+    float r;           // uniform draw when no uniforms[] array is attached
+    unsigned epoch;    // grid-barrier generation base of the persistent kernel
+    int error;         // set by a kernel that gave up (bounded barrier wait)
+    int reserved;
+};
+
+size_t tensor_bytes(const lpp_config& c, int tensor);
+
+// Implemented in fused_decode.hip.
+lpp_status fused_prepare(lpp_model* m);
+lpp_status fused_release(lpp_model* m);
+// forward() and the generation loop on LPP_PATH_FUSED / LPP_PATH_PERSISTENT.
+lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, float penalty,
+                         const int* history, int history_len, float r, int* next_token);
+lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_steps, float temperature,
+                          float penalty, int* history, int* history_len, int history_cap,
+                          const float* uniforms, int* out_tokens, lpp_gen_stats* stats);
+
+}  // namespace lpp

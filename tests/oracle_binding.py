@@ -1,0 +1,247 @@
+"""ctypes view of the CPU oracle (oracle/liblpp_oracle.so) and, where it was
+built, of the compiled reference (oracle/_ref/liblpp_ref.so).  Test-side only."""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent.parent
+ORACLE_DIR = ROOT / "oracle"
+ORACLE_SO = ORACLE_DIR / "liblpp_oracle.so"
+REF_SO = ORACLE_DIR / "_ref" / "liblpp_ref.so"
+
+_f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+_u16p = np.ctypeslib.ndpointer(dtype=np.uint16, flags="C_CONTIGUOUS")
+
+
+class OrcConfig(C.Structure):
+    _fields_ = [("dim", C.c_int), ("hidden_dim", C.c_int), ("n_layers", C.c_int), ("n_heads", C.c_int),
+                ("n_kv_heads", C.c_int), ("vocab_size", C.c_int), ("seq_len", C.c_int), ("rope_base", C.c_float)]
+
+
+class OrcWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in
+                ("token_embedding_table", "rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", "w2",
+                 "w3", "rms_final_weight", "w_cls")] + [("w_is_f16", C.c_int)]
+
+
+class OrcState(C.Structure):
+    _fields_ = [(n, C.POINTER(C.c_float)) for n in
+                ("x", "xb", "xb2", "hb", "he", "q", "k", "v", "att", "logits", "key_cache", "value_cache")] + \
+               [("kv_round_f16", C.c_int)]
+
+
+_oracle = None
+_ref = None
+
+
+def build_oracle() -> None:
+    subprocess.run(["make", "-C", str(ORACLE_DIR), "liblpp_oracle.so"], check=True, capture_output=True)
+
+
+def oracle() -> C.CDLL:
+    global _oracle
+    if _oracle is not None:
+        return _oracle
+    if not ORACLE_SO.exists():
+        build_oracle()
+    lib = C.CDLL(str(ORACLE_SO))
+    lib.orc_naive_matmul.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int]
+    lib.orc_matmul_f16w.argtypes = [_f32p, _f32p, _u16p, C.c_int, C.c_int]
+    lib.orc_rmsnorm.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    lib.orc_rope.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]
+    lib.orc_softmax.argtypes = [_f32p, C.c_int]
+    lib.orc_swiglu.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    lib.orc_f16_to_f32.argtypes = [C.c_uint16]
+    lib.orc_f16_to_f32.restype = C.c_float
+    lib.orc_f32_to_f16_rn.argtypes = [C.c_float]
+    lib.orc_f32_to_f16_rn.restype = C.c_uint16
+    lib.orc_state_alloc.argtypes = [C.POINTER(OrcState), C.POINTER(OrcConfig)]
+    lib.orc_state_free.argtypes = [C.POINTER(OrcState)]
+    lib.orc_attention.argtypes = [C.POINTER(OrcState), C.POINTER(OrcWeights), C.POINTER(OrcConfig), C.c_int, C.c_int]
+    lib.orc_transformer_block.argtypes = lib.orc_attention.argtypes
+    lib.orc_forward_logits.argtypes = [C.c_int, C.c_int, C.POINTER(OrcState), C.POINTER(OrcWeights),
+                                       C.POINTER(OrcConfig)]
+    lib.orc_sample.argtypes = [_f32p, C.c_int, C.c_float, C.c_float, C.c_float, C.c_void_p, C.c_int, C.c_float]
+    lib.orc_sample.restype = C.c_int
+    lib.orc_sample_cdf.argtypes = [_f32p, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_int, C.c_float,
+                                   C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    lib.orc_sample_cdf.restype = C.c_int
+    lib.orc_forward.argtypes = [C.c_int, C.c_int, C.POINTER(OrcState), C.POINTER(OrcWeights), C.POINTER(OrcConfig),
+                                C.c_float, C.c_float, C.c_float, C.c_void_p, C.c_int, C.c_float]
+    lib.orc_forward.restype = C.c_int
+    lib.orc_history_push.argtypes = [_i32p, C.POINTER(C.c_int), C.c_int, C.c_int]
+    _oracle = lib
+    return lib
+
+
+def have_ref() -> bool:
+    return REF_SO.exists()
+
+
+def ref() -> C.CDLL:
+    global _ref
+    if _ref is not None:
+        return _ref
+    lib = C.CDLL(str(REF_SO))
+    lib.ref_naive_matmul.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int]
+    lib.ref_rmsnorm.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    lib.ref_rope.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]
+    lib.ref_softmax.argtypes = [_f32p, C.c_int]
+    lib.ref_swiglu.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    lib.ref_srand.argtypes = [C.c_uint]
+    lib.ref_next_uniform.restype = C.c_float
+    lib.ref_sample.argtypes = [_f32p, C.c_int, C.c_float, C.c_float, C.c_float, C.c_void_p, C.c_int]
+    lib.ref_sample.restype = C.c_int
+    lib.ref_model_create.argtypes = [C.c_int] * 7 + [C.c_float] + [C.c_void_p] * 12
+    lib.ref_model_create.restype = C.c_void_p
+    lib.ref_model_destroy.argtypes = [C.c_void_p]
+    lib.ref_forward.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_void_p, C.c_int]
+    lib.ref_forward.restype = C.c_int
+    lib.ref_attention.argtypes = [C.c_void_p, C.c_int, C.c_int]
+    lib.ref_transformer_block.argtypes = [C.c_void_p, C.c_int, C.c_int]
+    lib.ref_state_buffer.argtypes = [C.c_void_p, C.c_int]
+    lib.ref_state_buffer.restype = C.POINTER(C.c_float)
+    _ref = lib
+    return lib
+
+
+WEIGHT_FIELDS = ["token_embedding_table", "rms_att_weight", "wq", "wk", "wv", "wo", "rms_ffn_weight", "w1", "w2",
+                 "w3", "rms_final_weight", "w_cls"]
+STATE_FIELDS = ["x", "xb", "xb2", "hb", "he", "q", "k", "v", "att", "logits", "key_cache", "value_cache"]
+
+
+class OracleModel:
+    """The oracle's forward() over host weight arrays.
+
+    weights: dict tensor-id (0..11, the order of WEIGHT_FIELDS) -> numpy array;
+    matrices are float32, or uint16 binary16 bit patterns when fp16=True."""
+
+    def __init__(self, shape, weights: dict, fp16: bool, kv_round_f16: bool = False):
+        self.lib = oracle()
+        self.shape = shape
+        self.cfg = OrcConfig(shape.dim, shape.hidden_dim, shape.n_layers, shape.n_heads, shape.n_kv_heads,
+                             shape.vocab_size, shape.seq_len, shape.rope_base)
+        self._keep = {t: np.ascontiguousarray(a) for t, a in weights.items()}
+        self.w = OrcWeights()
+        for t, name in enumerate(WEIGHT_FIELDS):
+            setattr(self.w, name, self._keep[t].ctypes.data)
+        self.w.w_is_f16 = 1 if fp16 else 0
+        self.s = OrcState()
+        if self.lib.orc_state_alloc(C.byref(self.s), C.byref(self.cfg)) != 0:
+            raise MemoryError("orc_state_alloc failed")
+        self.s.kv_round_f16 = 1 if kv_round_f16 else 0
+
+    def close(self):
+        if self.s.x:
+            self.lib.orc_state_free(C.byref(self.s))
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def sizes(self):
+        p = self.shape
+        kv_dim = p.dim * p.n_kv_heads // p.n_heads
+        cache = p.n_layers * p.seq_len * kv_dim
+        return {"x": p.dim, "xb": p.dim, "xb2": p.dim, "hb": p.hidden_dim, "he": p.hidden_dim, "q": p.dim,
+                "k": kv_dim, "v": kv_dim, "att": p.n_heads * p.seq_len, "logits": p.vocab_size,
+                "key_cache": cache, "value_cache": cache}
+
+    def buf(self, name: str) -> np.ndarray:
+        """Live numpy view of a state buffer."""
+        n = self.sizes()[name]
+        return np.ctypeslib.as_array(getattr(self.s, name), shape=(n,))
+
+    def forward_logits(self, token: int, pos: int) -> np.ndarray:
+        self.lib.orc_forward_logits(token, pos, C.byref(self.s), C.byref(self.w), C.byref(self.cfg))
+        return self.buf("logits").copy()
+
+    def transformer_block(self, layer: int, pos: int):
+        self.lib.orc_transformer_block(C.byref(self.s), C.byref(self.w), C.byref(self.cfg), layer, pos)
+
+    def attention(self, layer: int, pos: int):
+        self.lib.orc_attention(C.byref(self.s), C.byref(self.w), C.byref(self.cfg), layer, pos)
+
+    def forward(self, token, pos, temperature=0.0, topp=1.0, penalty=1.0, history=None, r=0.0) -> int:
+        if history is not None and len(history) > 0:
+            h = np.ascontiguousarray(history, dtype=np.int32)
+            hp, hl = h.ctypes.data, int(h.size)
+        else:
+            hp, hl = None, 0
+        return self.lib.orc_forward(token, pos, C.byref(self.s), C.byref(self.w), C.byref(self.cfg), temperature,
+                                    topp, penalty, hp, hl, r)
+
+
+def orc_sample(logits: np.ndarray, temperature, topp, penalty, history, r) -> tuple:
+    """Runs the oracle sampler on a copy; returns (token, mutated logits)."""
+    lg = np.ascontiguousarray(logits, dtype=np.float32).copy()
+    if history is not None and len(history) > 0:
+        h = np.ascontiguousarray(history, dtype=np.int32)
+        hp, hl = h.ctypes.data, int(h.size)
+    else:
+        hp, hl = None, 0
+    tok = oracle().orc_sample(lg, lg.size, temperature, topp, penalty, hp, hl, r)
+    return tok, lg
+
+
+def orc_sample_cdf(logits: np.ndarray, temperature, penalty, history, r) -> tuple:
+    """(token, cdf just below the token's bucket, cdf at its upper edge)."""
+    lg = np.ascontiguousarray(logits, dtype=np.float32).copy()
+    if history is not None and len(history) > 0:
+        h = np.ascontiguousarray(history, dtype=np.int32)
+        hp, hl = h.ctypes.data, int(h.size)
+    else:
+        hp, hl = None, 0
+    lo, hi = C.c_float(), C.c_float()
+    tok = oracle().orc_sample_cdf(lg, lg.size, temperature, penalty, hp, hl, r, C.byref(lo), C.byref(hi))
+    return tok, lo.value, hi.value
+
+
+class RefModel:
+    """forward() of the compiled reference over fp32 host weights (tensor ids as above)."""
+
+    def __init__(self, shape, weights_f32: dict):
+        self.lib = ref()
+        self.shape = shape
+        self._keep = {t: np.ascontiguousarray(a, dtype=np.float32) for t, a in weights_f32.items()}
+        ptrs = [self._keep[t].ctypes.data for t in range(12)]
+        self.h = self.lib.ref_model_create(shape.dim, shape.hidden_dim, shape.n_layers, shape.n_heads,
+                                           shape.n_kv_heads, shape.vocab_size, shape.seq_len, shape.rope_base, *ptrs)
+        if not self.h:
+            raise MemoryError("ref_model_create failed")
+
+    def close(self):
+        if self.h:
+            self.lib.ref_model_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def buf(self, name: str) -> np.ndarray:
+        p = self.shape
+        kv_dim = p.dim * p.n_kv_heads // p.n_heads
+        cache = p.n_layers * p.seq_len * kv_dim
+        sizes = {"x": p.dim, "xb": p.dim, "xb2": p.dim, "hb": p.hidden_dim, "he": p.hidden_dim, "q": p.dim,
+                 "k": kv_dim, "v": kv_dim, "att": p.n_heads * p.seq_len, "logits": p.vocab_size,
+                 "key_cache": cache, "value_cache": cache}
+        ptr = self.lib.ref_state_buffer(self.h, STATE_FIELDS.index(name))
+        return np.ctypeslib.as_array(ptr, shape=(sizes[name],))
+
+    def forward(self, token, pos, temperature=0.0, topp=1.0, penalty=1.0, history=None) -> int:
+        if history is not None and len(history) > 0:
+            h = np.ascontiguousarray(history, dtype=np.int32)
+            hp, hl = h.ctypes.data, int(h.size)
+        else:
+            hp, hl = None, 0
+        return self.lib.ref_forward(self.h, token, pos, temperature, topp, penalty, hp, hl)

@@ -1,0 +1,260 @@
+"""Parity of the decode loop (include/lpp.h section B: forward / generate, the
+counterpart of the reference's src/model.cpp:342-371 and src/main.cpp:158-223)
+against the CPU oracle on identical seeded weights, for every scheduling path
+of the library, on a real MI355X.
+
+Bars (from the task statement):
+  * logits: max |gpu - cpu| / max |cpu| <= 2e-3 per step (fp32 accumulation);
+  * greedy token sequences agree on >= 99 % of steps;
+  * a sampled token may differ only where the uniform draw sits closer than the
+    logits tolerance to a bucket edge of the CPU CDF;
+  * KV-cache scatter: slot index logic and binary16 rounding bit-exact.
+The oracle rounds K/V through binary16 on store (kv_round_f16), which is what the
+GPU operator API does by contract (kernels.cuh:34); a second check bounds the
+distance to the pure-fp32-cache CPU path as well.
+"""
+import numpy as np
+import pytest
+
+import oracle_binding as ob
+from lighterpp_amd import CONFIGS, Model, Shape, capi
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+LOGIT_TOL = 2e-3
+
+PATHS = [capi.PATH_OPS, capi.PATH_FUSED]
+PATH_IDS = ["ops", "fused"]
+
+SMALL_SHAPES = {
+    # name: Shape
+    "mha_fp32_c1like": Shape(288, 768, 3, 6, 6, 1000, 64, 10000.0, fp16=False, tied=True),
+    "gqa4_fp16": Shape(256, 512, 3, 8, 2, 2048, 160, 500000.0, fp16=True, tied=True),
+    "gqa8_fp16_untied": Shape(512, 1408, 2, 8, 1, 1500, 96, 10000.0, fp16=True, tied=False),
+    "hs128_fp16": Shape(512, 1024, 2, 4, 2, 777, 48, 500000.0, fp16=True, tied=False),
+}
+
+
+def build(shape: Shape, seed: int, kv_round=True):
+    m = Model(shape)
+    w = m.load_synthetic(seed, keep=True)
+    o = ob.OracleModel(shape, w, fp16=shape.fp16, kv_round_f16=kv_round)
+    return m, o
+
+
+def rel_err(got, want):
+    return float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
+
+
+@pytest.mark.parametrize("path", PATHS, ids=PATH_IDS)
+@pytest.mark.parametrize("name", list(SMALL_SHAPES))
+def test_greedy_decode_matches_oracle(name, path):
+    shape = SMALL_SHAPES[name]
+    m, o = build(shape, 21)
+    m.set_path(path)
+    prompt = capi.synth_token_ids(8, 5, shape.vocab_size)
+    steps = min(48, shape.seq_len)
+    tok_g = tok_c = int(prompt[0])
+    agree, worst = 0, 0.0
+    for pos in range(steps):
+        # teacher-force the oracle's token into both, so one early flip cannot cascade
+        nxt_g = m.forward(tok_c, pos, 0.0)
+        want = o.forward_logits(tok_c, pos)
+        got = m.buffer(capi.B_LOGITS)
+        worst = max(worst, rel_err(got, want))
+        nxt_c = int(np.argmax(want))
+        agree += int(nxt_g == nxt_c)
+        tok_c = int(prompt[pos + 1]) if pos + 1 < len(prompt) else nxt_c
+    assert worst <= LOGIT_TOL, f"max relative logit error {worst}"
+    assert agree >= int(np.ceil(0.99 * steps)), f"greedy agreement {agree}/{steps}"
+    # cache contents: same slots, same binary16 values up to the rounding of a k that differs in the last bits
+    kc = m.buffer(capi.B_KEY_CACHE).view(np.float16).astype(F)
+    vc = m.buffer(capi.B_VALUE_CACHE).view(np.float16).astype(F)
+    assert np.allclose(kc, o.buf("key_cache"), rtol=2e-3, atol=2e-3 * np.abs(o.buf("key_cache")).max())
+    assert np.allclose(vc, o.buf("value_cache"), rtol=2e-3, atol=2e-3 * np.abs(o.buf("value_cache")).max())
+    hs, nkv = shape.head_size, shape.n_kv_heads
+    kc4 = kc.reshape(shape.n_layers, nkv, shape.seq_len, hs)
+    assert np.all(kc4[:, :, steps:, :] == 0), "slots beyond the decoded positions were written"
+    m.close()
+    o.close()
+
+
+@pytest.mark.parametrize("path", PATHS, ids=PATH_IDS)
+def test_kv_scatter_index_and_rounding_bit_exact(path):
+    """After a step at position p the cache slice [layer][h][p][:] of the LAST layer
+    must hold exactly RN16 of that layer's k / v vectors (model.cpp:171-176), which
+    the run state still contains."""
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m = Model(shape)
+    m.load_synthetic(33)
+    m.set_path(path)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    tok = 3
+    for pos in [0, 1, 2, 77]:
+        tok = m.forward(tok, pos, 0.0)
+        k = m.buffer(capi.B_K).reshape(nkv, hs)
+        v = m.buffer(capi.B_V).reshape(nkv, hs)
+        kc = m.buffer(capi.B_KEY_CACHE).reshape(L, nkv, shape.seq_len, hs)
+        vc = m.buffer(capi.B_VALUE_CACHE).reshape(L, nkv, shape.seq_len, hs)
+        assert np.array_equal(kc[L - 1, :, pos, :], k.astype(np.float16).view(np.uint16))
+        assert np.array_equal(vc[L - 1, :, pos, :], v.astype(np.float16).view(np.uint16))
+    written = {0, 1, 2, 77}
+    kc = m.buffer(capi.B_KEY_CACHE).reshape(L, nkv, shape.seq_len, hs)
+    for p in range(shape.seq_len):
+        if p not in written:
+            assert not kc[:, :, p, :].any()
+    m.close()
+
+
+def test_distance_to_fp32_cache_cpu_path():
+    """Against the reference CPU semantics proper (fp32 KV cache): the binary16
+    cache the GPU API prescribes must still leave logits inside the tolerance."""
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m, o = build(shape, 9, kv_round=False)
+    m.set_path(capi.PATH_FUSED)
+    tok = 11
+    worst = 0.0
+    for pos in range(40):
+        m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        worst = max(worst, rel_err(m.buffer(capi.B_LOGITS), want))
+        tok = int(np.argmax(want))
+    assert worst <= LOGIT_TOL, worst
+    m.close()
+    o.close()
+
+
+@pytest.mark.parametrize("path", PATHS, ids=PATH_IDS)
+def test_generate_sampled_matches_oracle(path):
+    """Generation loop with the fused sampler: temperature 0.8, penalty 1.1,
+    64-entry sliding window, pre-drawn uniforms (config-3 settings, small shape)."""
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m, o = build(shape, 17)
+    m.set_path(path)
+    steps = 100
+    draws = capi.synth_uniform_f32(steps, 99)
+    first = 42
+    toks, hist_after, stats = m.generate(first, 0, steps, temperature=0.8, penalty=1.1, history=[first],
+                                         history_cap=64, uniforms=draws)
+    assert stats.tokens == steps
+    # replay on the oracle, feeding the GPU's tokens so that one allowed flip does not cascade
+    hist = [first]
+    tok = first
+    flips = 0
+    for i in range(steps):
+        o.forward_logits(tok, i)
+        want, lo, hi = ob.orc_sample_cdf(o.buf("logits"), 0.8, 1.1, hist, float(draws[i]))
+        if toks[i] != want:
+            flips += 1
+            gap = min(abs(float(draws[i]) - lo), abs(float(draws[i]) - hi))
+            assert gap < LOGIT_TOL, f"step {i}: token {toks[i]} vs {want}, CDF gap {gap}"
+        tok = int(toks[i])
+        hist = (hist + [tok])[-64:]
+    assert flips <= 2
+    assert hist_after == hist  # the window comes back oldest-first, like main.cpp:203-208 keeps it
+    m.close()
+    o.close()
+
+
+def test_generate_paths_agree_and_window_wraps():
+    """Fused generate == operator-path generate token for token (greedy, penalty on,
+    window of 5 so that it wraps many times)."""
+    shape = SMALL_SHAPES["gqa8_fp16_untied"]
+    m = Model(shape)
+    m.load_synthetic(4)
+    out = {}
+    for path in PATHS:
+        m.set_path(path)
+        m.reset()
+        out[path] = m.generate(7, 0, 60, temperature=0.0, penalty=1.3, history=[7], history_cap=5)
+    a, b = out[capi.PATH_OPS], out[capi.PATH_FUSED]
+    assert np.mean(a[0] == b[0]) >= 0.99
+    if np.array_equal(a[0], b[0]):
+        assert a[1] == b[1] and len(a[1]) == 5
+    m.close()
+
+
+def test_forward_then_generate_continuation():
+    """Prefill by single forwards (main.cpp:163-179), then generate from the next
+    position; positions and cache carry over."""
+    shape = SMALL_SHAPES["mha_fp32_c1like"]
+    m, o = build(shape, 2)
+    m.set_path(capi.PATH_FUSED)
+    prompt = capi.synth_token_ids(8, 1, shape.vocab_size)
+    for pos in range(7):
+        m.forward(int(prompt[pos]), pos, 0.0)
+        o.forward_logits(int(prompt[pos]), pos)
+    toks, _, _ = m.generate(int(prompt[7]), 7, 40, temperature=0.0)
+    tok = int(prompt[7])
+    agree = 0
+    for i in range(40):
+        want = int(np.argmax(o.forward_logits(tok, 7 + i)))
+        agree += int(want == toks[i])
+        tok = int(toks[i])
+    assert agree >= 39
+    m.close()
+    o.close()
+
+
+def test_long_context_attention_matches_oracle():
+    """Config-4 style: cache pre-filled with binary16 N(0,1) up to a long position,
+    then decode there; the split-context attention must agree with the CPU loop."""
+    shape = Shape(256, 512, 2, 8, 2, 1000, 4400, 500000.0, fp16=True, tied=True)
+    m, o = build(shape, 8)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    start = 4300
+    n = L * nkv * shape.seq_len * hs
+    kfill = capi.synth_normal_f16(n, 501, 1.0).reshape(L, nkv, shape.seq_len, hs)
+    vfill = capi.synth_normal_f16(n, 502, 1.0).reshape(L, nkv, shape.seq_len, hs)
+    kfill[:, :, start:, :] = 0
+    vfill[:, :, start:, :] = 0
+    o.buf("key_cache")[:] = capi.f16_to_f32(kfill.reshape(-1))
+    o.buf("value_cache")[:] = capi.f16_to_f32(vfill.reshape(-1))
+    for path in PATHS:
+        m.write_buffer(capi.B_KEY_CACHE, kfill)
+        m.write_buffer(capi.B_VALUE_CACHE, vfill)
+        m.set_path(path)
+        tok = 5
+        for pos in range(start, start + 6):
+            m.forward(tok, pos, 0.0)
+            want = o.forward_logits(tok, pos)
+            assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL
+            tok = int(np.argmax(want))
+    m.close()
+    o.close()
+
+
+def test_model_argument_errors():
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m = Model(shape)
+    with pytest.raises(capi.LppError) as e:
+        m.forward(1, 0)
+    assert e.value.status == capi.LPP_ERR_STATE  # weights not uploaded
+    m.load_synthetic(1)
+    for bad in [dict(token=-1, pos=0), dict(token=shape.vocab_size, pos=0), dict(token=0, pos=shape.seq_len)]:
+        with pytest.raises(capi.LppError) as e:
+            m.forward(bad["token"], bad["pos"])
+        assert e.value.status == capi.LPP_ERR_INVALID_ARG
+    with pytest.raises(capi.LppError):
+        m.generate(0, shape.seq_len - 3, 10)
+    m.close()
+
+
+@pytest.mark.parametrize("cfg,steps,start", [("c1_llama2c_15m_fp32", 24, 0), ("c3_llama32_1b_fp16", 6, 0)])
+def test_benchmark_shapes_first_steps(cfg, steps, start):
+    """The real benchmark shapes for a handful of steps (the oracle needs about a
+    second per token at the 1B shape)."""
+    shape = CONFIGS[cfg]
+    m, o = build(shape, 1234)
+    m.set_path(capi.PATH_FUSED)
+    tok = int(capi.synth_token_ids(1, 77, shape.vocab_size)[0])
+    agree = 0
+    for pos in range(start, start + steps):
+        nxt = m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL
+        agree += int(nxt == int(np.argmax(want)))
+        tok = int(np.argmax(want))
+    assert agree == steps
+    m.close()
+    o.close()
