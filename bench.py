@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Batch-1 decode benchmark of liblpp_hip.so on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--path fused|ops|persistent]
+
+A step is one decoded token: forward() over every layer, classifier and the
+fused sampler, on synthetic seeded weights of the named shape, with weights and
+KV cache resident in HBM before the clock starts.  The timed region is the
+generation loop of the reference's main.cpp (one forward per token, the 4-byte
+token copy per token included).  Prints ONE JSON line.
+
+Besides the throughput the line carries
+  roofline     the dominant kernel's achieved HBM rate (algorithmic bytes per
+               launch / mean launch duration from HIP events on the launch
+               stream) against MI355X's 8 TB/s,
+  cpu_baseline the reference CPU path (oracle/_ref, the reference's own
+               ops.cpp + model.cpp compiled for the host; falls back to the
+               restated oracle) timed on a bounded sample of the same workload
+               on the host cores of this machine,
+  parity       logits of the first decoded positions against the CPU oracle.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "decode tok/s at batch 1 + % of 8 TB/s HBM roofline, Llama-3.2-1B-shape fp16"
+
+# Workload of each configuration: (prompt tokens, default decode steps, start position, sampler settings)
+WORKLOADS = {
+    "c1_llama2c_15m_fp32": dict(prompt=8, steps=248, start=0, temperature=0.0, penalty=1.0, history_cap=0),
+    "c2_tinyllama_1b_fp16": dict(prompt=16, steps=512, start=0, temperature=0.0, penalty=1.0, history_cap=0),
+    "c3_llama32_1b_fp16": dict(prompt=1, steps=512, start=0, temperature=0.8, penalty=1.1, history_cap=64),
+    "c4_llama32_1b_longctx_fp16": dict(prompt=1, steps=256, start=8192, temperature=0.0, penalty=1.0,
+                                       history_cap=0),
+    "c5_llama3_8b_fp16": dict(prompt=32, steps=1024, start=0, temperature=0.0, penalty=1.0, history_cap=0),
+}
+SEED = 20251
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def prefill_cache(model, shape, upto: int) -> None:
+    """Config 4: K/V of positions [0, upto) filled with binary16 N(0, 1)."""
+    from lighterpp_amd import capi
+    hs, nkv, L, seq = shape.head_size, shape.n_kv_heads, shape.n_layers, shape.seq_len
+    for which, buf in ((0, capi.B_KEY_CACHE), (1, capi.B_VALUE_CACHE)):
+        for layer in range(L):
+            for h in range(nkv):
+                a = capi.synth_normal_f16(upto * hs, SEED * 7 + which, 1.0, first_index=(layer * nkv + h) * seq * hs)
+                model.write_buffer(buf, a, byte_offset=((layer * nkv + h) * seq * hs) * 2)
+
+
+def cpu_baseline(shape, weights, wl, first_token, start, budget_s: float):
+    """Times the CPU path on a bounded sample of the workload.  Prefers the compiled
+    reference; otherwise the restated oracle."""
+    import oracle_binding as ob
+    from lighterpp_amd import capi
+    cores = os.cpu_count() or 1
+    if start != 0:
+        return dict(value=None, unit="tok/s", cores=1, kind="port",
+                    sample="skipped: a pre-filled cache at this size does not fit the CPU path's time bound")
+    kind = "reference" if ob.have_ref() else "port"
+    t_build = time.time()
+    if kind == "reference":
+        w32 = {t: (capi.f16_to_f32(a) if a.dtype == np.uint16 else np.ascontiguousarray(a, np.float32))
+               for t, a in weights.items()}
+        cpu = ob.RefModel(shape, w32)
+        step = lambda tok, pos, hist: cpu.forward(tok, pos, wl["temperature"], 1.0, wl["penalty"], hist)
+    else:
+        cpu = ob.OracleModel(shape, weights, fp16=shape.fp16)
+        step = lambda tok, pos, hist: cpu.forward(tok, pos, wl["temperature"], 1.0, wl["penalty"], hist, 0.5)
+    log(f"cpu baseline ({kind}) ready in {time.time() - t_build:.1f}s")
+    tok, hist, n = first_token, [first_token], 0
+    t0 = time.perf_counter()
+    while True:
+        tok = step(tok, n, hist if wl["history_cap"] else None)
+        if wl["history_cap"]:
+            hist = (hist + [tok])[-wl["history_cap"]:]
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or n >= 256 or n >= shape.seq_len:
+            break
+    cpu.close()
+    return dict(value=round(n / el, 4), unit="tok/s", cores=1, host_cores=cores, kind=kind,
+                sample=f"{n} decode steps from position 0 of the same workload, single thread, {el:.1f}s")
+
+
+def parity_check(model, shape, weights, first_token, n_steps: int):
+    """Teacher-forced logits comparison against the oracle on the first positions."""
+    import oracle_binding as ob
+    from lighterpp_amd import capi
+    o = ob.OracleModel(shape, weights, fp16=shape.fp16, kv_round_f16=True)
+    model.reset()
+    tok, worst, agree = first_token, 0.0, 0
+    for pos in range(n_steps):
+        nxt = model.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        got = model.buffer(capi.B_LOGITS)
+        worst = max(worst, float(np.max(np.abs(got - want)) / np.max(np.abs(want))))
+        agree += int(nxt == int(np.argmax(want)))
+        tok = int(np.argmax(want))
+    o.close()
+    return dict(steps=n_steps, max_rel_logit_err=worst, greedy_agreement=agree / n_steps, tolerance=2e-3,
+                checker="oracle (CPU restatement, binary16 KV store)")
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", default="c3_llama32_1b_fp16", choices=list(WORKLOADS))
+    ap.add_argument("--path", default="fused", choices=["ops", "fused", "persistent"])
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time bound of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--parity-steps", type=int, default=3)
+    ap.add_argument("--profile-reps", type=int, default=20)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (batch-1 decode has no multi-GPU path here); "
+              "run with --gpus 1", file=sys.stderr)
+        return 2
+
+    from lighterpp_amd import CONFIGS, Model, capi
+    lib = capi.load()
+    if capi.device_count() < 1:
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 3
+    capi.check(lib.lpp_init(0))
+    name = ctypes.create_string_buffer(128)
+    cus, hbm = ctypes.c_int(), ctypes.c_size_t()
+    capi.check(lib.lpp_device_info(name, 128, ctypes.byref(cus), ctypes.byref(hbm)))
+
+    shape = CONFIGS[args.config]
+    wl = dict(WORKLOADS[args.config])
+    steps = args.steps if args.steps is not None else wl["steps"]
+    start = wl["start"] + wl["prompt"] - 1
+    steps = min(steps, shape.seq_len - start)
+    path = {"ops": capi.PATH_OPS, "fused": capi.PATH_FUSED, "persistent": capi.PATH_PERSISTENT}[args.path]
+
+    t0 = time.time()
+    model = Model(shape)
+    need_host = args.cpu_seconds > 0 or args.parity_steps > 0
+    weights = model.load_synthetic(SEED, keep=need_host)
+    log(f"{args.config}: weights resident in HBM after {time.time() - t0:.1f}s "
+        f"({shape.matrix_params() / 1e6:.1f} M matrix params)")
+    model.set_path(path)
+    prompt = capi.synth_token_ids(max(wl["prompt"], 1), SEED + 1, shape.vocab_size)
+    uniforms = capi.synth_uniform_f32(max(steps, args.warmup, 1), SEED + 2)
+    temperature, penalty, cap = wl["temperature"], wl["penalty"], wl["history_cap"]
+
+    def run(n_steps: int):
+        """Prompt by single forwards (untimed, main.cpp:163-179), then the timed loop."""
+        model.reset()
+        if wl["start"] > 0:
+            prefill_cache(model, shape, wl["start"])
+        hist = []
+        for i in range(wl["prompt"] - 1):
+            hist = (hist + [int(prompt[i])])[-cap:] if cap else []
+            model.forward(int(prompt[i]), wl["start"] + i, temperature, 1.0, penalty, hist or None, 0.5)
+        first = int(prompt[wl["prompt"] - 1])
+        hist = (hist + [first])[-cap:] if cap else []
+        return model.generate(first, start, n_steps, temperature=temperature, penalty=penalty, history=hist,
+                              history_cap=cap, uniforms=uniforms if temperature != 0.0 else None)
+
+    if args.warmup > 0:
+        run(min(args.warmup, steps))
+    capi.synchronize()
+    t_wall = time.perf_counter()
+    tokens, _, stats = run(steps)
+    capi.synchronize()
+    wall_outer = time.perf_counter() - t_wall  # includes reset/prompt; the figure reported is the loop itself
+    sec = stats.wall_seconds
+    tok_s = steps / sec
+    avg_bytes = float(np.mean([shape.bytes_per_token(p) for p in range(start, start + steps)]))
+    log(f"{steps} tokens in {sec * 1e3:.1f} ms -> {tok_s:.1f} tok/s, {avg_bytes * tok_s / 1e9:.0f} GB/s algorithmic "
+        f"(outer {wall_outer:.2f}s)")
+
+    # dominant kernel, timed live with HIP events on the launch stream
+    roofline = None
+    kernels = []
+    if path != capi.PATH_OPS:
+        mid = start + steps // 2
+        prof = model.profile_kernels(min(mid, shape.seq_len - 1), args.profile_reps)
+        per_token_ms = sum(n * ms for (_, n, ms, _) in prof)
+        kernels = [dict(kernel=k, launches_per_token=n, avg_us=round(ms * 1e3, 3),
+                        algorithmic_mb=round(b / 1e6, 3), gbs=round(b / (ms * 1e-3) / 1e9, 1) if ms > 0 else None)
+                   for (k, n, ms, b) in prof]
+        dom = max(prof, key=lambda p: p[1] * p[2])
+        achieved = dom[3] / (dom[2] * 1e-3) / 1e9
+        roofline = dict(bound="hbm", kernel=dom[0], achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                        frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                        bytes_per_launch=dom[3], avg_launch_us=round(dom[2] * 1e3, 3),
+                        sum_of_kernel_times_ms_per_token=round(per_token_ms, 4))
+
+    parity = None
+    if args.parity_steps > 0:
+        parity = parity_check(model, shape, weights, int(prompt[0]), args.parity_steps)
+        log(f"parity: {parity}")
+    cpu = None
+    if args.cpu_seconds > 0:
+        model.close()
+        cpu = cpu_baseline(shape, weights, wl, int(prompt[wl['prompt'] - 1]), wl["start"], args.cpu_seconds)
+        log(f"cpu baseline: {cpu}")
+
+    out = {
+        "metric": METRIC,
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec / steps * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32 accumulate over f16 weights" if shape.fp16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": args.config, "path": args.path, "dim": shape.dim, "hidden_dim": shape.hidden_dim,
+                   "n_layers": shape.n_layers, "n_heads": shape.n_heads, "n_kv_heads": shape.n_kv_heads,
+                   "vocab_size": shape.vocab_size, "start_pos": start, "temperature": temperature,
+                   "penalty": penalty, "history_window": cap, "weights": "N(0,0.02) seeded, norm gains 1"},
+        "hbm": {"algorithmic_bytes_per_token": round(avg_bytes), "achieved_gbs": round(avg_bytes * tok_s / 1e9, 1),
+                "peak_gbs": HBM_PEAK_GBS, "frac_of_peak": round(avg_bytes * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+                "device_ms_per_token": round(stats.device_ms / steps, 5)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "parity": parity,
+        "kernels": kernels,
+        "device": {"name": name.value.decode(), "compute_units": cus.value},
+        "first_tokens": tokens[:8].tolist(),
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

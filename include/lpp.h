@@ -229,6 +229,20 @@ lpp_status lpp_generate(lpp_model *m, int first_token, int start_pos, int n_step
                         int *history_len, int history_cap, const float *uniforms,
                         int *out_tokens, lpp_gen_stats *stats);
 
+/* Per-kernel timing of the fused path, measured with HIP events on the launch
+ * stream: each kernel class is recorded n_layers times (one launch per layer,
+ * so every launch streams different weights) into a graph that is replayed
+ * `reps` times between two events.  avg_ms is the mean duration of one launch,
+ * bytes the algorithmic HBM bytes of one launch at position `pos`. */
+typedef struct lpp_kernel_time {
+    char name[32];
+    int launches_per_token;
+    double avg_ms;
+    double bytes_per_launch;
+} lpp_kernel_time;
+lpp_status lpp_profile_kernels(lpp_model *m, int pos, int reps, lpp_kernel_time *out, int capacity,
+                               int *count);
+
 /* ===================================================================== */
 /* C. Runtime plumbing                                                    */
 /* ===================================================================== */

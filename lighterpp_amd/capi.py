@@ -47,6 +47,11 @@ class LppGenStats(C.Structure):
                 ("kernel_launches", C.c_int), ("tokens", C.c_int)]
 
 
+class LppKernelTime(C.Structure):
+    _fields_ = [("name", C.c_char * 32), ("launches_per_token", C.c_int), ("avg_ms", C.c_double),
+                ("bytes_per_launch", C.c_double)]
+
+
 class LppError(RuntimeError):
     def __init__(self, status: int, message: str):
         super().__init__(f"lpp status {status}: {message}")
@@ -84,6 +89,7 @@ SIGNATURES = {
     "lpp_transformer_block": (_i, [_vp, _i, _i]),
     "lpp_forward": (_i, [_vp, _i, _i, _f, _f, _f, _vp, _i, _f, _ip]),
     "lpp_generate": (_i, [_vp, _i, _i, _i, _f, _f, _f, _vp, _ip, _i, _vp, _vp, C.POINTER(LppGenStats)]),
+    "lpp_profile_kernels": (_i, [_vp, _i, _i, C.POINTER(LppKernelTime), _i, _ip]),
     # C. runtime
     "lpp_last_error": (C.c_char_p, []),
     "lpp_version": (C.c_char_p, []),

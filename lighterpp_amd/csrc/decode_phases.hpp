@@ -391,9 +391,10 @@ __device__ __forceinline__ void phase_lmhead(const DecodeArgs& a, int wg, int nw
 // Phase: attention over the cache (split context)
 // ---------------------------------------------------------------------------
 
-// Number of context splits in use at this position: about 64 positions each.
+// Number of context splits in use at this position: about 256 positions each
+// (shorter pieces do not repay the cross-workgroup combine).
 __device__ __forceinline__ int active_splits(int npos, int max_splits) {
-    int s = (npos + 63) / 64;
+    int s = (npos + 255) / 256;
     return s < 1 ? 1 : (s > max_splits ? max_splits : s);
 }
 
@@ -404,11 +405,6 @@ __device__ __forceinline__ float group_sum(float v) {
     if constexpr (kGroup >= 8) v += dpp_move<kDppHalfMirror>(v);
     if constexpr (kGroup >= 16) v += dpp_move<kDppMirror>(v);
     return v;
-}
-
-// Device-coherent read of a value another workgroup published before a fence.
-__device__ __forceinline__ float coherent_load(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 constexpr int kAttBlock = 512;   // positions per softmax sub-block
@@ -559,6 +555,16 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
     }
     __syncthreads();
     const int stride = hs + 2;
+    if (nsplits == 1) {
+        // Whole context in this workgroup: normalise and finish (model.cpp:190-198).
+        for (int i = tid; i < gqa * hs; i += nthreads) {
+            const int qh = i / hs, e = i - qh * hs;
+            float o = 0.0f;
+            for (int w = 0; w < nwaves; ++w) o += red[(w * gqa + qh) * hs_pad + e];
+            a.xb[static_cast<size_t>(kvh * gqa + qh) * hs + e] = o / run_sum[qh];
+        }
+        return;
+    }
     for (int i = tid; i < gqa * hs; i += nthreads) {
         const int qh = i / hs, e = i - qh * hs;
         float o = 0.0f;
@@ -571,9 +577,11 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
         }
     }
 
-    // Last split to arrive combines.
+    // The last split to arrive for this KV head combines all of them.  Writers
+    // publish with a release fence before taking a ticket; the combiner acquires
+    // after seeing the last ticket, then reads the partials with ordinary loads.
     __shared__ int is_last;
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     if (tid == 0) {
         const unsigned ticket = atomicAdd(&a.att_count[kvh], 1u);
@@ -582,18 +590,18 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
     }
     __syncthreads();
     if (!is_last) return;
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     for (int i = tid; i < gqa * hs; i += nthreads) {
         const int qh = i / hs, e = i - qh * hs;
         const float* base = a.att_partial + static_cast<size_t>(kvh * gqa + qh) * a.max_splits * stride;
         float top = -INFINITY;
-        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, coherent_load(base + s * stride + hs));
+        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, base[s * stride + hs]);
         float o = 0.0f, l = 0.0f;
         for (int s = 0; s < nsplits; ++s) {
-            const float ms = coherent_load(base + s * stride + hs);
+            const float ms = base[s * stride + hs];
             const float wgt = (ms == -INFINITY) ? 0.0f : expf(ms - top);
-            o += coherent_load(base + s * stride + e) * wgt;
-            l += coherent_load(base + s * stride + hs + 1) * wgt;
+            o += base[s * stride + e] * wgt;
+            l += base[s * stride + hs + 1] * wgt;
         }
         a.xb[static_cast<size_t>(kvh * gqa + qh) * hs + e] = o / l;
     }
@@ -629,18 +637,23 @@ __device__ __forceinline__ float step_uniform(const DecodeArgs& a) {
 // After the sampler: publish the token, feed it back as the next input, advance
 // the position and the penalty window (src/main.cpp:200-208; the window is kept
 // as a ring because the penalty does not depend on the order of its entries).
-__device__ __forceinline__ void finish_token(const DecodeArgs& a, int token) {
+// out_tokens may be pinned host memory: the 4-byte result is stored with system
+// scope so the host sees it without a copy command.
+__device__ __forceinline__ void finish_token(const DecodeArgs& a, int token, unsigned epoch_advance) {
     StepParams* sp = a.step;
+    sp->epoch += epoch_advance;
     a.sampled[0] = token;
-    if (a.out_tokens) a.out_tokens[sp->step_index] = token;
+    if (sp->freeze) return;
     if (sp->history_cap > 0) {
         a.history[sp->history_next] = token;
         sp->history_next = (sp->history_next + 1) % sp->history_cap;
         if (sp->history_len < sp->history_cap) sp->history_len += 1;
     }
+    const int index = sp->step_index;
     sp->token = token;
     sp->pos += 1;
-    sp->step_index += 1;
+    sp->step_index = index + 1;
+    if (a.out_tokens) __hip_atomic_store(a.out_tokens + index, token, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 }  // namespace ph

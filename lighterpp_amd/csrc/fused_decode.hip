@@ -1,10 +1,20 @@
-// fused_decode.hip -- LPP_PATH_FUSED: one token of forward() (reference
-// src/model.cpp:342-371) as 5 launches per layer + classifier + sampler steps,
-// recorded once into a HIP graph and replayed per token.  All per-token
-// scalars (token, position, penalty window, uniform draw) live in device
-// memory, so the graph is never patched; the sampled id is fed back on the
-// device, and the host only collects 4 bytes per token.
+// fused_decode.hip -- the two fast schedules of forward() (reference
+// src/model.cpp:342-371) built from the phases of decode_phases.hpp:
+//
+//   LPP_PATH_FUSED       one launch per phase (5 per layer + classifier + sampler
+//                        steps), recorded once into a HIP graph, replayed per token;
+//   LPP_PATH_PERSISTENT  one kernel per token that walks all phases itself, with
+//                        a grid barrier between phases.  A workgroup requests the
+//                        first weights of the next phase before it waits at the
+//                        barrier, so HBM keeps streaming while the grid
+//                        synchronises.
+//
+// All per-token scalars (token, position, penalty window, uniform draw) live in
+// device memory, so neither schedule is patched between tokens; the sampled id is
+// fed back on the device and written straight into pinned host memory, 4 bytes
+// per token.
 #include <chrono>
+#include <cstdio>
 #include <cstring>
 #include <vector>
 
@@ -15,12 +25,18 @@ namespace {
 
 using namespace ph;
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;            // graph path
 constexpr int kWavesPerWg = kThreads / dev::kWave;
+constexpr int kPersistThreads = 512;     // persistent path: 8 wavefronts per workgroup
+constexpr int kNoToken = -1;             // sentinel in the pinned token array
 
 struct NoWait {
     __device__ __forceinline__ void operator()() const {}
 };
+
+// ---------------------------------------------------------------------------
+// One launch per phase
+// ---------------------------------------------------------------------------
 
 template <bool kF16>
 __global__ __launch_bounds__(kThreads) void k_qkv(DecodeArgs a, int layer) {
@@ -62,39 +78,151 @@ __global__ __launch_bounds__(kThreads) void k_lmhead(DecodeArgs a) {
     phase_lmhead<kF16, 4>(a, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
-// Sampler steps; one workgroup per vocabulary chunk.
-__global__ __launch_bounds__(smp::kSampleThreads) void k_sample_scale(DecodeArgs a, int chunk) {
+// Sampler steps; chunk c of the vocabulary is handled by workgroup c.
+__device__ __forceinline__ void sample_step_scale(const DecodeArgs& a, int chunk, int c) {
     const StepParams* sp = a.step;
-    smp::scale_max_chunk(a.logits, a.work, a.vocab, chunk, blockIdx.x, sp->temperature, sp->penalty,
+    smp::scale_max_chunk(a.logits, a.work, a.vocab, chunk, c, sp->temperature, sp->penalty,
                          sp->history_len > 0 ? a.history : nullptr, sp->history_len, a.sample_scratch);
 }
-
-__global__ __launch_bounds__(smp::kSampleThreads) void k_sample_exp(DecodeArgs a, int chunk, int nchunks) {
+// Greedy (model.cpp:272-283) finishes here in chunk 0; otherwise exponentials.
+__device__ __forceinline__ void sample_step_exp(const DecodeArgs& a, int chunk, int nchunks, int c) {
     if (a.step->temperature == 0.0f) {
-        // model.cpp:272-283: greedy; one workgroup finishes the token.
-        if (blockIdx.x == 0) {
+        if (c == 0) {
             const int tok = smp::argmax_over_chunks(nchunks, a.sample_scratch);
             if (threadIdx.x == 0) a.sampled[0] = tok;
         }
         return;
     }
-    smp::exp_sum_chunk(a.work, a.vocab, chunk, nchunks, blockIdx.x, a.sample_scratch);
+    smp::exp_sum_chunk(a.work, a.vocab, chunk, nchunks, c, a.sample_scratch);
+}
+__device__ __forceinline__ void sample_step_norm(const DecodeArgs& a, int chunk, int nchunks, int c) {
+    if (a.step->temperature == 0.0f) return;
+    smp::normalise_chunk(a.work, a.vocab, chunk, nchunks, c, a.sample_scratch);
+    if (c == 0 && threadIdx.x == 0) a.sampled[0] = a.vocab - 1;  // model.cpp:302
+}
+__device__ __forceinline__ void sample_step_search(const DecodeArgs& a, int chunk, int c) {
+    if (a.step->temperature == 0.0f) return;
+    smp::cdf_search_chunk(a.work, a.vocab, chunk, c, step_uniform(a), a.sample_scratch, a.sampled);
 }
 
+__global__ __launch_bounds__(smp::kSampleThreads) void k_sample_scale(DecodeArgs a, int chunk) {
+    sample_step_scale(a, chunk, blockIdx.x);
+}
+__global__ __launch_bounds__(smp::kSampleThreads) void k_sample_exp(DecodeArgs a, int chunk, int nchunks) {
+    sample_step_exp(a, chunk, nchunks, blockIdx.x);
+}
 __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_norm(DecodeArgs a, int chunk, int nchunks) {
-    if (a.step->temperature == 0.0f) return;
-    smp::normalise_chunk(a.work, a.vocab, chunk, nchunks, blockIdx.x, a.sample_scratch);
-    if (blockIdx.x == 0 && threadIdx.x == 0) a.sampled[0] = a.vocab - 1;  // model.cpp:302
+    sample_step_norm(a, chunk, nchunks, blockIdx.x);
 }
-
 __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_search(DecodeArgs a, int chunk) {
-    if (a.step->temperature == 0.0f) return;
-    smp::cdf_search_chunk(a.work, a.vocab, chunk, blockIdx.x, step_uniform(a), a.sample_scratch, a.sampled);
+    sample_step_search(a, chunk, blockIdx.x);
+}
+__global__ void k_finish(DecodeArgs a) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) finish_token(a, a.sampled[0], 0u);
 }
 
-__global__ void k_finish(DecodeArgs a) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) finish_token(a, a.sampled[0]);
+// ---------------------------------------------------------------------------
+// One kernel per token
+// ---------------------------------------------------------------------------
+
+// Grid barrier over a monotonically increasing arrival counter.  Barrier number
+// i of the token whose generation base is `base` is complete when the counter
+// has reached (base + i + 1) * nwg; the counter is never reset, comparisons are
+// wrap-safe.  The wait is bounded: after spin_limit polls the workgroup records
+// an error, raises the shared abort flag and every later wait returns at once,
+// so the grid always drains.
+struct GridSync {
+    unsigned* counter;
+    unsigned* abort_flag;
+    StepParams* step;
+    unsigned base;
+    unsigned nwg;
+    unsigned spin_limit;
+    unsigned index;
+
+    __device__ __forceinline__ void arrive() {
+        __syncthreads();  // every wavefront of the workgroup has issued its stores
+        if (threadIdx.x == 0) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+
+    __device__ __forceinline__ void wait() {
+        if (threadIdx.x == 0) {
+            const unsigned target = (base + index + 1u) * nwg;
+            unsigned spins = 0;
+            while (static_cast<int>(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+                if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
+                if (++spins > spin_limit) {
+                    __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    step->error = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+        }
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        ++index;
+    }
+};
+
+// Barriers per token: 5 per layer + classifier + 4 sampler steps.
+__host__ __device__ inline unsigned barriers_per_token(int n_layers) {
+    return static_cast<unsigned>(n_layers) * 5u + 5u;
 }
+
+template <bool kF16>
+__global__ __launch_bounds__(kPersistThreads) void k_decode_token(DecodeArgs a, unsigned* counter, unsigned* abort_flag,
+                                                                  unsigned spin_limit) {
+    extern __shared__ __align__(16) float lds[];
+    const int wg = blockIdx.x, nwg = gridDim.x;
+    GridSync gs{counter, abort_flag, a.step, a.step->epoch, static_cast<unsigned>(nwg), spin_limit, 0u};
+    auto wait = [&]() { gs.wait(); };
+    const int wbytes = kF16 ? 2 : 4;
+
+    for (int layer = 0; layer < a.n_layers; ++layer) {
+        if (layer == 0) phase_qkv<kF16, 2>(a, layer, wg, nwg, lds, NoWait{});  // previous token ended at a kernel boundary
+        else phase_qkv<kF16, 2>(a, layer, wg, nwg, lds, wait);
+        gs.arrive();
+        phase_attention(a, layer, wg, nwg, lds, wait);
+        gs.arrive();
+        phase_proj_residual<kF16, 2>(a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes, a.dim, a.dim, a.xb,
+                                     layer_input(a, layer), a.x, wg, nwg, lds, wait);
+        gs.arrive();
+        phase_gateup<kF16, 2>(a, layer, wg, nwg, lds, wait);
+        gs.arrive();
+        phase_proj_residual<kF16, 1>(a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden,
+                                     a.hb, a.x, a.x, wg, nwg, lds, wait);
+        gs.arrive();
+    }
+    phase_lmhead<kF16, 4>(a, wg, nwg, lds, wait);
+    gs.arrive();
+
+    const int chunk = smp::chunk_size_for(a.vocab);
+    const int nchunks = (a.vocab + chunk - 1) / chunk;
+    gs.wait();
+    for (int c = wg; c < nchunks; c += nwg) sample_step_scale(a, chunk, c);
+    gs.arrive();
+    gs.wait();
+    for (int c = wg; c < nchunks; c += nwg) sample_step_exp(a, chunk, nchunks, c);
+    gs.arrive();
+    gs.wait();
+    for (int c = wg; c < nchunks; c += nwg) sample_step_norm(a, chunk, nchunks, c);
+    gs.arrive();
+    gs.wait();
+    for (int c = wg; c < nchunks; c += nwg) sample_step_search(a, chunk, c);
+    gs.arrive();
+    if (wg == 0) {
+        gs.wait();
+        if (threadIdx.x == 0) finish_token(a, a.sampled[0], barriers_per_token(a.n_layers));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
 
 DecodeArgs make_args(const lpp_model* m, bool with_arrays) {
     DecodeArgs a{};
@@ -138,7 +266,7 @@ DecodeArgs make_args(const lpp_model* m, bool with_arrays) {
     a.step = m->step;
     a.history = m->history;
     a.uniforms = with_arrays ? m->gen_uniforms : nullptr;
-    a.out_tokens = with_arrays ? m->gen_tokens : nullptr;
+    a.out_tokens = with_arrays ? m->pinned_tokens_dev : nullptr;
     a.sampled = m->sampled_token;
     float* sc = m->sample_scratch;
     a.sample_scratch = smp::SampleScratch{sc, reinterpret_cast<int*>(sc + smp::kMaxChunks),
@@ -153,42 +281,47 @@ int blocks_for_tiles(int ntiles) {
     return blocks < 1 ? 1 : blocks;
 }
 
-// Enqueue every launch of one token on `s`.
+struct Launch {
+    size_t lds_dim, lds_hidden, lds_att;
+    int qkv_blocks, o_blocks, gu_blocks, down_blocks, lm_blocks, att_blocks, chunk, nchunks;
+};
+
+Launch launch_plan(const lpp_model* m) {
+    const lpp_config& c = m->cfg;
+    Launch p;
+    p.lds_dim = static_cast<size_t>((c.dim + 7) & ~7) * 4;
+    p.lds_hidden = static_cast<size_t>((c.hidden_dim + 7) & ~7) * 4;
+    p.lds_att = static_cast<size_t>(attention_lds_floats(m->gqa, m->head_size, kThreads)) * 4;
+    p.qkv_blocks = blocks_for_tiles((c.dim + 2 * m->kv_dim + 1) / 2);
+    p.o_blocks = blocks_for_tiles((c.dim + 1) / 2);
+    p.gu_blocks = blocks_for_tiles((c.hidden_dim + 1) / 2);
+    p.down_blocks = blocks_for_tiles(c.dim);
+    p.lm_blocks = blocks_for_tiles((c.vocab_size + 3) / 4);
+    p.att_blocks = c.n_kv_heads * m->max_splits;
+    p.chunk = smp::chunk_size_for(c.vocab_size);
+    p.nchunks = (c.vocab_size + p.chunk - 1) / p.chunk;
+    return p;
+}
+
+// Enqueue every launch of one token on `s` (graph path).
 template <bool kF16>
 lpp_status enqueue_token(const lpp_model* m, const DecodeArgs& a, hipStream_t s) {
-    const lpp_config& c = m->cfg;
-    const size_t lds_dim = static_cast<size_t>((c.dim + 7) & ~7) * 4;
-    const size_t lds_hidden = static_cast<size_t>((c.hidden_dim + 7) & ~7) * 4;
-    const size_t lds_att = static_cast<size_t>(attention_lds_floats(m->gqa, m->head_size, kThreads)) * 4;
-    const int qkv_tiles = (c.dim + 2 * m->kv_dim + 1) / 2;
-    const int o_tiles = (c.dim + 1) / 2;
-    const int gu_tiles = (c.hidden_dim + 1) / 2;
-    const int down_tiles = c.dim;
-    const int lm_tiles = (c.vocab_size + 3) / 4;
-    const int att_blocks = c.n_kv_heads * m->max_splits;
-    for (int layer = 0; layer < c.n_layers; ++layer) {
-        hipLaunchKernelGGL((k_qkv<kF16>), dim3(blocks_for_tiles(qkv_tiles)), dim3(kThreads), lds_dim, s, a, layer);
-        hipLaunchKernelGGL(k_attention, dim3(att_blocks), dim3(kThreads), lds_att, s, a, layer);
-        hipLaunchKernelGGL((k_oproj<kF16>), dim3(blocks_for_tiles(o_tiles)), dim3(kThreads), lds_dim, s, a, layer);
-        hipLaunchKernelGGL((k_gateup<kF16>), dim3(blocks_for_tiles(gu_tiles)), dim3(kThreads), lds_dim, s, a, layer);
-        hipLaunchKernelGGL((k_down<kF16>), dim3(blocks_for_tiles(down_tiles)), dim3(kThreads), lds_hidden, s, a,
-                           layer);
+    const Launch p = launch_plan(m);
+    for (int layer = 0; layer < m->cfg.n_layers; ++layer) {
+        hipLaunchKernelGGL((k_qkv<kF16>), dim3(p.qkv_blocks), dim3(kThreads), p.lds_dim, s, a, layer);
+        hipLaunchKernelGGL(k_attention, dim3(p.att_blocks), dim3(kThreads), p.lds_att, s, a, layer);
+        hipLaunchKernelGGL((k_oproj<kF16>), dim3(p.o_blocks), dim3(kThreads), p.lds_dim, s, a, layer);
+        hipLaunchKernelGGL((k_gateup<kF16>), dim3(p.gu_blocks), dim3(kThreads), p.lds_dim, s, a, layer);
+        hipLaunchKernelGGL((k_down<kF16>), dim3(p.down_blocks), dim3(kThreads), p.lds_hidden, s, a, layer);
     }
-    hipLaunchKernelGGL((k_lmhead<kF16>), dim3(blocks_for_tiles(lm_tiles)), dim3(kThreads), lds_dim, s, a);
-    const int chunk = smp::chunk_size_for(c.vocab_size);
-    const int nchunks = (c.vocab_size + chunk - 1) / chunk;
-    hipLaunchKernelGGL(k_sample_scale, dim3(nchunks), dim3(smp::kSampleThreads), 0, s, a, chunk);
-    hipLaunchKernelGGL(k_sample_exp, dim3(nchunks), dim3(smp::kSampleThreads), 0, s, a, chunk, nchunks);
-    hipLaunchKernelGGL(k_sample_norm, dim3(nchunks), dim3(smp::kSampleThreads), 0, s, a, chunk, nchunks);
-    hipLaunchKernelGGL(k_sample_search, dim3(nchunks), dim3(smp::kSampleThreads), 0, s, a, chunk);
+    hipLaunchKernelGGL((k_lmhead<kF16>), dim3(p.lm_blocks), dim3(kThreads), p.lds_dim, s, a);
+    hipLaunchKernelGGL(k_sample_scale, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk);
+    hipLaunchKernelGGL(k_sample_exp, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk, p.nchunks);
+    hipLaunchKernelGGL(k_sample_norm, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk, p.nchunks);
+    hipLaunchKernelGGL(k_sample_search, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk);
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(64), 0, s, a);
     LPP_CHECK_LAUNCH("fused token");
     return LPP_OK;
-}
-
-lpp_status enqueue_token_any(const lpp_model* m, const DecodeArgs& a, hipStream_t s) {
-    return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? enqueue_token<true>(m, a, s)
-                                                      : enqueue_token<false>(m, a, s);
 }
 
 // Record the token into a graph once per (model, with_arrays) and keep the
@@ -201,7 +334,8 @@ lpp_status token_graph(lpp_model* m, bool with_arrays, hipGraphExec_t* exec) {
         const DecodeArgs a = make_args(m, with_arrays);
         hipGraph_t graph = nullptr;
         LPP_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
-        lpp_status st = enqueue_token_any(m, a, s);
+        lpp_status st = m->cfg.weight_precision == LPP_WEIGHT_FP16 ? enqueue_token<true>(m, a, s)
+                                                                     : enqueue_token<false>(m, a, s);
         hipError_t e = hipStreamEndCapture(s, &graph);
         if (st != LPP_OK) {
             if (graph) (void)hipGraphDestroy(graph);
@@ -223,10 +357,49 @@ void drop_graphs(lpp_model* m) {
     }
 }
 
+// Persistent path: grid = one workgroup per compute unit, all co-resident.
+size_t persistent_lds_bytes(const lpp_model* m) {
+    const lpp_config& c = m->cfg;
+    size_t floats = static_cast<size_t>((c.dim + 7) & ~7);
+    const size_t hidden = static_cast<size_t>((c.hidden_dim + 7) & ~7);
+    if (hidden > floats) floats = hidden;
+    const size_t att = static_cast<size_t>(attention_lds_floats(m->gqa, m->head_size, kPersistThreads));
+    if (att > floats) floats = att;
+    return floats * 4;
+}
+
+template <bool kF16>
+lpp_status persistent_launch(lpp_model* m, const DecodeArgs& a, hipStream_t s) {
+    if (m->persist_grid == 0) {
+        int per_cu = 0;
+        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode_token<kF16>, kPersistThreads,
+                                                              persistent_lds_bytes(m)));
+        if (per_cu < 1)
+            return fail(LPP_ERR_UNSUPPORTED, "persistent decode kernel does not fit a compute unit (LDS %zu bytes)",
+                        persistent_lds_bytes(m));
+        m->persist_grid = compute_units();
+    }
+    hipLaunchKernelGGL((k_decode_token<kF16>), dim3(m->persist_grid), dim3(kPersistThreads), persistent_lds_bytes(m), s,
+                       a, m->sync_words + 64, m->sync_words + 65, m->spin_limit);
+    LPP_CHECK_LAUNCH("k_decode_token");
+    return LPP_OK;
+}
+
+// One token on the model's current path.
+lpp_status launch_token(lpp_model* m, bool with_arrays, hipStream_t s) {
+    if (m->path == LPP_PATH_PERSISTENT) {
+        const DecodeArgs a = make_args(m, with_arrays);
+        return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? persistent_launch<true>(m, a, s)
+                                                          : persistent_launch<false>(m, a, s);
+    }
+    hipGraphExec_t exec = nullptr;
+    LPP_TRY(token_graph(m, with_arrays, &exec));
+    LPP_HIP(hipGraphLaunch(exec, s));
+    return LPP_OK;
+}
+
 lpp_status require_fused(const lpp_model* m) {
     if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused decode path unavailable for this shape: %s", m->fused_why);
-    if (m->path == LPP_PATH_PERSISTENT)
-        return fail(LPP_ERR_UNSUPPORTED, "LPP_PATH_PERSISTENT is not built into this library");
     return LPP_OK;
 }
 
@@ -237,22 +410,37 @@ lpp_status ensure_gen_capacity(lpp_model* m, int n_steps) {
     LPP_HIP(hipStreamSynchronize(stream()));
     drop_graphs(m);  // the recorded kernels hold the old array addresses
     lpp_free(m->gen_uniforms);
-    lpp_free(m->gen_tokens);
     m->gen_uniforms = nullptr;
-    m->gen_tokens = nullptr;
+    if (m->pinned_tokens) (void)hipHostFree(m->pinned_tokens);
+    m->pinned_tokens = nullptr;
+    m->pinned_tokens_dev = nullptr;
     m->gen_cap = 0;
     void* p = nullptr;
     LPP_TRY(lpp_malloc(&p, static_cast<size_t>(want) * sizeof(float)));
     m->gen_uniforms = static_cast<float*>(p);
-    LPP_TRY(lpp_malloc(&p, static_cast<size_t>(want) * sizeof(int)));
-    m->gen_tokens = static_cast<int*>(p);
-    if (m->pinned_tokens) (void)hipHostFree(m->pinned_tokens);
-    m->pinned_tokens = nullptr;
     if (hipHostMalloc(reinterpret_cast<void**>(&m->pinned_tokens), static_cast<size_t>(want) * sizeof(int),
-                      hipHostMallocDefault) != hipSuccess)
+                      hipHostMallocMapped) != hipSuccess)
         return fail(LPP_ERR_OOM, "pinned token buffer allocation failed");
-    m->pinned_tokens_cap = want;
+    LPP_HIP(hipHostGetDevicePointer(reinterpret_cast<void**>(&m->pinned_tokens_dev), m->pinned_tokens, 0));
     m->gen_cap = want;
+    return LPP_OK;
+}
+
+// Wait until the kernels have delivered token i to pinned host memory.
+lpp_status await_token(lpp_model* m, int i, hipStream_t s) {
+    volatile int* slot = m->pinned_tokens + i;
+    unsigned polls = 0;
+    while (*slot == kNoToken) {
+        if ((++polls & 0xfffu) == 0u) {
+            // Nothing arrived for a while: make sure the stream is still making progress.
+            const hipError_t q = hipStreamQuery(s);
+            if (q == hipSuccess) {
+                if (*slot != kNoToken) break;
+                return fail(LPP_ERR_HIP, "decode finished without delivering token %d", i);
+            }
+            if (q != hipErrorNotReady) return fail(LPP_ERR_HIP, "stream failed: %s", hipGetErrorString(q));
+        }
+    }
     return LPP_OK;
 }
 
@@ -271,11 +459,12 @@ lpp_status fused_prepare(lpp_model* m) {
     else if (c.dim % per != 0 || c.hidden_dim % per != 0) reject("dim and hidden_dim must fill whole 16-byte weight loads");
     else if (c.hidden_dim > 16384 || c.dim > 16384) reject("activation vector does not fit the 64 KiB LDS stage");
 
-    // About 64 positions per split once the context is long; at most 32 splits.
-    int splits = c.seq_len / 64;
+    // About 256 positions per split once the context is long; at most 32 splits.
+    int splits = c.seq_len / 256;
     if (splits < 1) splits = 1;
     if (splits > 32) splits = 32;
     m->max_splits = splits;
+    m->spin_limit = 1u << 20;
 
     void* p = nullptr;
     LPP_TRY(lpp_malloc(&p, sizeof(StepParams)));
@@ -289,13 +478,13 @@ lpp_status fused_prepare(lpp_model* m) {
     m->att_partial = static_cast<float*>(p);
     LPP_TRY(lpp_malloc(&p, static_cast<size_t>(c.vocab_size) * sizeof(float)));
     m->work_logits = static_cast<float*>(p);
-    LPP_TRY(lpp_malloc(&p, 256 * sizeof(unsigned)));
+    // words 0..63: attention split counters per KV head; 64: grid-barrier arrivals; 65: abort flag
+    LPP_REQUIRE(c.n_kv_heads <= 64 || !m->fused_ok, "more than 64 KV heads");
+    LPP_TRY(lpp_malloc(&p, 128 * sizeof(unsigned)));
     m->sync_words = static_cast<unsigned*>(p);
-    LPP_TRY(lpp_memset(m->sync_words, 0, 256 * sizeof(unsigned)));
+    LPP_TRY(lpp_memset(m->sync_words, 0, 128 * sizeof(unsigned)));
     LPP_TRY(lpp_malloc(&p, 4 * smp::kMaxChunks * sizeof(float)));
     m->sample_scratch = static_cast<float*>(p);
-    for (auto& e : m->ev_tok)
-        if (hipEventCreate(&e) != hipSuccess) return fail(LPP_ERR_HIP, "hipEventCreate failed");
     return LPP_OK;
 }
 
@@ -309,9 +498,18 @@ lpp_status fused_release(lpp_model* m) {
     lpp_free(m->sync_words);
     lpp_free(m->sample_scratch);
     lpp_free(m->gen_uniforms);
-    lpp_free(m->gen_tokens);
-    for (auto& e : m->ev_tok)
-        if (e) (void)hipEventDestroy(e);
+    return LPP_OK;
+}
+
+// Bring the device-side step record (and the persistent kernel's barrier state)
+// to a known start.
+static lpp_status begin_run(lpp_model* m, const StepParams& init, hipStream_t s) {
+    StepParams& sp = *m->step_host;
+    sp = init;
+    sp.epoch = 0;
+    sp.error = 0;
+    LPP_HIP(hipMemcpyAsync(m->step, &sp, sizeof sp, hipMemcpyHostToDevice, s));
+    if (m->path == LPP_PATH_PERSISTENT) LPP_TRY(lpp_memset(m->sync_words + 64, 0, 2 * sizeof(unsigned)));
     return LPP_OK;
 }
 
@@ -323,8 +521,7 @@ lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, fl
     if (use_history)
         LPP_REQUIRE(history_len <= m->cfg.seq_len, "lpp_forward: history_len %d exceeds seq_len %d", history_len,
                     m->cfg.seq_len);
-    StepParams& sp = *m->step_host;
-    std::memset(&sp, 0, sizeof sp);
+    StepParams sp{};
     sp.token = token;
     sp.pos = pos;
     sp.history_len = use_history ? history_len : 0;
@@ -332,15 +529,17 @@ lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, fl
     sp.temperature = temperature;
     sp.penalty = penalty;
     sp.r = r;
-    LPP_HIP(hipMemcpyAsync(m->step, &sp, sizeof sp, hipMemcpyHostToDevice, s));
+    LPP_TRY(begin_run(m, sp, s));
     if (use_history)
         LPP_HIP(hipMemcpyAsync(m->history, history, static_cast<size_t>(history_len) * sizeof(int),
                                hipMemcpyHostToDevice, s));
-    hipGraphExec_t exec = nullptr;
-    LPP_TRY(token_graph(m, false, &exec));
-    LPP_HIP(hipGraphLaunch(exec, s));
+    LPP_TRY(launch_token(m, false, s));
     LPP_HIP(hipMemcpyAsync(next_token, m->sampled_token, sizeof(int), hipMemcpyDeviceToHost, s));
     LPP_HIP(hipStreamSynchronize(s));
+    if (m->path == LPP_PATH_PERSISTENT) {
+        LPP_HIP(hipMemcpy(m->step_host, m->step, sizeof(StepParams), hipMemcpyDeviceToHost));
+        if (m->step_host->error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up at a grid barrier");
+    }
     return LPP_OK;
 }
 
@@ -351,8 +550,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     if (n_steps == 0) return LPP_OK;
     hipStream_t s = stream();
     LPP_TRY(ensure_gen_capacity(m, n_steps));
-    StepParams& sp = *m->step_host;
-    std::memset(&sp, 0, sizeof sp);
+    StepParams sp{};
     sp.token = first_token;
     sp.pos = start_pos;
     sp.history_len = *history_len;
@@ -360,7 +558,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     sp.history_next = (history_cap > 0) ? (*history_len % history_cap) : 0;
     sp.temperature = temperature;
     sp.penalty = penalty;
-    LPP_HIP(hipMemcpyAsync(m->step, &sp, sizeof sp, hipMemcpyHostToDevice, s));
+    LPP_TRY(begin_run(m, sp, s));
     if (*history_len > 0)
         LPP_HIP(hipMemcpyAsync(m->history, history, static_cast<size_t>(*history_len) * sizeof(int),
                                hipMemcpyHostToDevice, s));
@@ -369,37 +567,41 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
                                hipMemcpyHostToDevice, s));
     else
         LPP_TRY(lpp_memset(m->gen_uniforms, 0, static_cast<size_t>(n_steps) * sizeof(float)));
-    hipGraphExec_t exec = nullptr;
-    LPP_TRY(token_graph(m, true, &exec));
+    for (int i = 0; i < n_steps; ++i) m->pinned_tokens[i] = kNoToken;
+    if (m->path != LPP_PATH_PERSISTENT) {
+        hipGraphExec_t exec = nullptr;
+        LPP_TRY(token_graph(m, true, &exec));  // record outside the timed loop
+    }
     LPP_HIP(hipStreamSynchronize(s));
 
-    // main.cpp:196-223: one forward per token.  Token i+1 is launched before the
-    // host waits for the 4 bytes of token i, so the device never idles on the host.
+    // main.cpp:196-223: one forward per token.  The device feeds each sampled id
+    // back by itself and writes it to pinned host memory; token i+1 is launched
+    // before the host waits for the 4 bytes of token i, so the device never idles
+    // on the host.
     LPP_HIP(hipEventRecord(m->ev_a, s));
     const auto t0 = std::chrono::steady_clock::now();
     for (int i = 0; i < n_steps; ++i) {
-        LPP_HIP(hipGraphLaunch(exec, s));
-        LPP_HIP(hipMemcpyAsync(m->pinned_tokens + i, m->gen_tokens + i, sizeof(int), hipMemcpyDeviceToHost, s));
-        LPP_HIP(hipEventRecord(m->ev_tok[i & 1], s));
+        LPP_TRY(launch_token(m, true, s));
         if (i > 0) {
-            LPP_HIP(hipEventSynchronize(m->ev_tok[(i - 1) & 1]));
+            LPP_TRY(await_token(m, i - 1, s));
             out_tokens[i - 1] = m->pinned_tokens[i - 1];
         }
     }
-    LPP_HIP(hipEventSynchronize(m->ev_tok[(n_steps - 1) & 1]));
+    LPP_TRY(await_token(m, n_steps - 1, s));
     out_tokens[n_steps - 1] = m->pinned_tokens[n_steps - 1];
     const auto t1 = std::chrono::steady_clock::now();
     LPP_HIP(hipEventRecord(m->ev_b, s));
     LPP_HIP(hipEventSynchronize(m->ev_b));
 
     // Hand the penalty window back in the reference's order (oldest first).
-    LPP_HIP(hipMemcpy(&sp, m->step, sizeof sp, hipMemcpyDeviceToHost));
-    if (sp.error != 0) return fail(LPP_ERR_HIP, "decode kernel reported error %d", sp.error);
+    StepParams done{};
+    LPP_HIP(hipMemcpy(&done, m->step, sizeof done, hipMemcpyDeviceToHost));
+    if (done.error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up at a grid barrier");
     if (history_cap > 0) {
         std::vector<int> ring(static_cast<size_t>(history_cap));
         LPP_HIP(hipMemcpy(ring.data(), m->history, ring.size() * sizeof(int), hipMemcpyDeviceToHost));
-        const int len = sp.history_len;
-        const int oldest = (len < history_cap) ? 0 : sp.history_next;
+        const int len = done.history_len;
+        const int oldest = (len < history_cap) ? 0 : done.history_next;
         for (int i = 0; i < len; ++i) history[i] = ring[static_cast<size_t>((oldest + i) % history_cap)];
         *history_len = len;
     }
@@ -409,8 +611,137 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
         stats->wall_seconds = std::chrono::duration<double>(t1 - t0).count();
         stats->device_ms = ms;
         stats->tokens = n_steps;
+        stats->kernel_launches = (m->path == LPP_PATH_PERSISTENT) ? n_steps : 0;
     }
     return LPP_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Per-kernel timing (lpp_profile_kernels)
+// ---------------------------------------------------------------------------
+namespace {
+
+template <class EnqueueFn>
+lpp_status time_class(lpp_model* m, int launches_in_graph, int reps, EnqueueFn enqueue, double* avg_ms) {
+    hipStream_t s = stream();
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    LPP_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    enqueue(s);
+    hipError_t e = hipStreamEndCapture(s, &graph);
+    if (e != hipSuccess) return fail(LPP_ERR_HIP, "profile capture failed: %s", hipGetErrorString(e));
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail(LPP_ERR_HIP, "profile instantiate failed: %s", hipGetErrorString(e));
+    LPP_HIP(hipGraphLaunch(exec, s));  // warm-up
+    LPP_HIP(hipStreamSynchronize(s));
+    LPP_HIP(hipEventRecord(m->ev_a, s));
+    for (int r = 0; r < reps; ++r) LPP_HIP(hipGraphLaunch(exec, s));
+    LPP_HIP(hipEventRecord(m->ev_b, s));
+    LPP_HIP(hipEventSynchronize(m->ev_b));
+    float ms = 0.0f;
+    LPP_HIP(hipEventElapsedTime(&ms, m->ev_a, m->ev_b));
+    (void)hipGraphExecDestroy(exec);
+    *avg_ms = static_cast<double>(ms) / (static_cast<double>(reps) * launches_in_graph);
+    return LPP_OK;
+}
+
+template <bool kF16>
+lpp_status profile_impl(lpp_model* m, int pos, int reps, lpp_kernel_time* out, int capacity, int* count) {
+    const lpp_config& c = m->cfg;
+    const DecodeArgs a = make_args(m, false);
+    const Launch p = launch_plan(m);
+    const int L = c.n_layers;
+    const double wb = kF16 ? 2.0 : 4.0;
+    const double dim = c.dim, hidden = c.hidden_dim, kv = m->kv_dim, vocab = c.vocab_size;
+    int n = 0;
+    auto add = [&](const char* name, int per_token, double ms, double bytes) {
+        if (n < capacity) {
+            std::snprintf(out[n].name, sizeof out[n].name, "%s", name);
+            out[n].launches_per_token = per_token;
+            out[n].avg_ms = ms;
+            out[n].bytes_per_launch = bytes;
+        }
+        ++n;
+    };
+    // Algorithmic bytes of one token at this position (what Shape.bytes_per_token counts).
+    const double token_bytes = wb * (L * (2 * dim * dim + 2 * kv * dim + 3 * hidden * dim) + vocab * dim) +
+                               4 * (2 * L + 1) * dim + 4 * dim + 4.0 * kv * L * (pos + 1) + 4.0 * kv * L;
+    double ms = 0.0;
+    if (m->path == LPP_PATH_PERSISTENT) {
+        // The whole token is one launch; a fresh step record per replay keeps pos fixed.
+        hipStream_t s = stream();
+        LPP_HIP(hipEventRecord(m->ev_a, s));
+        for (int r = 0; r < reps; ++r) {
+            LPP_TRY(persistent_launch<kF16>(m, a, s));
+        }
+        LPP_HIP(hipEventRecord(m->ev_b, s));
+        LPP_HIP(hipEventSynchronize(m->ev_b));
+        float total = 0.0f;
+        LPP_HIP(hipEventElapsedTime(&total, m->ev_a, m->ev_b));
+        add("k_decode_token", 1, static_cast<double>(total) / reps, token_bytes);
+        *count = n < capacity ? n : capacity;
+        return LPP_OK;
+    }
+    LPP_TRY(time_class(m, L, reps, [&](hipStream_t s) {
+        for (int l = 0; l < L; ++l)
+            hipLaunchKernelGGL((k_qkv<kF16>), dim3(p.qkv_blocks), dim3(kThreads), p.lds_dim, s, a, l);
+    }, &ms));
+    add("k_qkv", L, ms, (dim + 2 * kv) * dim * wb + 8 * dim + 4 * kv);
+    LPP_TRY(time_class(m, L, reps, [&](hipStream_t s) {
+        for (int l = 0; l < L; ++l)
+            hipLaunchKernelGGL(k_attention, dim3(p.att_blocks), dim3(kThreads), p.lds_att, s, a, l);
+    }, &ms));
+    add("k_attention", L, ms, 4.0 * kv * (pos + 1));
+    LPP_TRY(time_class(m, L, reps, [&](hipStream_t s) {
+        for (int l = 0; l < L; ++l)
+            hipLaunchKernelGGL((k_oproj<kF16>), dim3(p.o_blocks), dim3(kThreads), p.lds_dim, s, a, l);
+    }, &ms));
+    add("k_oproj", L, ms, dim * dim * wb);
+    LPP_TRY(time_class(m, L, reps, [&](hipStream_t s) {
+        for (int l = 0; l < L; ++l)
+            hipLaunchKernelGGL((k_gateup<kF16>), dim3(p.gu_blocks), dim3(kThreads), p.lds_dim, s, a, l);
+    }, &ms));
+    add("k_gateup", L, ms, 2 * hidden * dim * wb);
+    LPP_TRY(time_class(m, L, reps, [&](hipStream_t s) {
+        for (int l = 0; l < L; ++l)
+            hipLaunchKernelGGL((k_down<kF16>), dim3(p.down_blocks), dim3(kThreads), p.lds_hidden, s, a, l);
+    }, &ms));
+    add("k_down", L, ms, dim * hidden * wb);
+    LPP_TRY(time_class(m, 1, reps, [&](hipStream_t s) {
+        hipLaunchKernelGGL((k_lmhead<kF16>), dim3(p.lm_blocks), dim3(kThreads), p.lds_dim, s, a);
+    }, &ms));
+    add("k_lmhead", 1, ms, vocab * dim * wb);
+    LPP_TRY(time_class(m, 4, reps, [&](hipStream_t s) {
+        hipLaunchKernelGGL(k_sample_scale, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk);
+        hipLaunchKernelGGL(k_sample_exp, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk, p.nchunks);
+        hipLaunchKernelGGL(k_sample_norm, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk, p.nchunks);
+        hipLaunchKernelGGL(k_sample_search, dim3(p.nchunks), dim3(smp::kSampleThreads), 0, s, a, p.chunk);
+    }, &ms));
+    add("k_sample_*", 4, ms, 0.0);
+    *count = n < capacity ? n : capacity;
+    return LPP_OK;
+}
+
+}  // namespace
 }  // namespace lpp
+
+extern "C" lpp_status lpp_profile_kernels(lpp_model* m, int pos, int reps, lpp_kernel_time* out, int capacity,
+                                          int* count) {
+    using namespace lpp;
+    LPP_REQUIRE(m && out && count && capacity > 0 && reps > 0, "lpp_profile_kernels: bad argument");
+    LPP_REQUIRE(pos >= 0 && pos < m->cfg.seq_len, "lpp_profile_kernels: pos %d outside [0, %d)", pos, m->cfg.seq_len);
+    if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
+    for (int t = 0; t < LPP_T_COUNT; ++t)
+        if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
+    StepParams sp{};
+    sp.pos = pos;
+    sp.temperature = 0.8f;
+    sp.penalty = 1.0f;
+    sp.r = 0.5f;
+    sp.freeze = 1;  // replays must not advance the position
+    LPP_TRY(begin_run(m, sp, stream()));
+    LPP_HIP(hipStreamSynchronize(stream()));
+    return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? profile_impl<true>(m, pos, reps, out, capacity, count)
+                                                      : profile_impl<false>(m, pos, reps, out, capacity, count);
+}

@@ -46,14 +46,15 @@ struct lpp_model {
     struct lpp::StepParams* step = nullptr;       // device
     struct lpp::StepParams* step_host = nullptr;  // pinned host mirror
     int* pinned_tokens = nullptr;            // pinned host landing area for sampled ids
-    int pinned_tokens_cap = 0;
+    int* pinned_tokens_dev = nullptr;        // the same memory as the device addresses it
     float* att_partial = nullptr;            // split-context attention partials
     float* work_logits = nullptr;            // sampler working copy of the logits
     unsigned* sync_words = nullptr;          // arrival counters (attention combine, grid barrier)
     float* sample_scratch = nullptr;         // 4 x kMaxChunks words
     float* gen_uniforms = nullptr;           // device copy of the per-step draws
-    int* gen_tokens = nullptr;               // device per-step results
     int gen_cap = 0;
+    int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
+    unsigned spin_limit = 1u << 20;          // polls a grid-barrier wait may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
     int max_splits = 1;
     bool fused_ok = false;                   // shape supported by the fused kernels
@@ -61,7 +62,6 @@ struct lpp_model {
 
     hipGraphExec_t graph_exec[2] = {nullptr, nullptr};  // [0] without, [1] with uniforms/out arrays
     hipEvent_t ev_a = nullptr, ev_b = nullptr;
-    hipEvent_t ev_tok[2] = {nullptr, nullptr};
 };
 
 namespace lpp {
@@ -80,7 +80,7 @@ struct StepParams {
     float r;           // uniform draw when no uniforms[] array is attached
     unsigned epoch;    // grid-barrier generation base of the persistent kernel
     int error;         // set by a kernel that gave up (bounded barrier wait)
-    int reserved;
+    int freeze;        // nonzero: a step leaves token/position/window as they are (timing replays)
 };
 
 size_t tensor_bytes(const lpp_config& c, int tensor);

@@ -182,6 +182,14 @@ class Model:
                                          C.c_void_p(out.ctypes.data), C.byref(stats)))
         return out, hist[:hlen.value].tolist(), stats
 
+    def profile_kernels(self, pos: int, reps: int = 20) -> list:
+        """[(name, launches_per_token, avg_ms, bytes_per_launch)] for the fused path."""
+        arr = (capi.LppKernelTime * 16)()
+        n = C.c_int(0)
+        capi.check(self.lib.lpp_profile_kernels(self.handle, pos, reps, arr, 16, C.byref(n)))
+        return [(arr[i].name.decode(), arr[i].launches_per_token, arr[i].avg_ms, arr[i].bytes_per_launch)
+                for i in range(n.value)]
+
     # ---- inspection ----
     def buffer(self, b: int, dtype=None) -> np.ndarray:
         p, n = C.c_void_p(), C.c_size_t()

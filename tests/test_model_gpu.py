@@ -23,8 +23,8 @@ pytestmark = pytest.mark.gpu
 F = np.float32
 LOGIT_TOL = 2e-3
 
-PATHS = [capi.PATH_OPS, capi.PATH_FUSED]
-PATH_IDS = ["ops", "fused"]
+PATHS = [capi.PATH_OPS, capi.PATH_FUSED, capi.PATH_PERSISTENT]
+PATH_IDS = ["ops", "fused", "persistent"]
 
 SMALL_SHAPES = {
     # name: Shape
@@ -167,10 +167,12 @@ def test_generate_paths_agree_and_window_wraps():
         m.set_path(path)
         m.reset()
         out[path] = m.generate(7, 0, 60, temperature=0.0, penalty=1.3, history=[7], history_cap=5)
-    a, b = out[capi.PATH_OPS], out[capi.PATH_FUSED]
-    assert np.mean(a[0] == b[0]) >= 0.99
-    if np.array_equal(a[0], b[0]):
-        assert a[1] == b[1] and len(a[1]) == 5
+    a = out[capi.PATH_OPS]
+    for path in PATHS[1:]:
+        b = out[path]
+        assert np.mean(a[0] == b[0]) >= 0.99
+        if np.array_equal(a[0], b[0]):
+            assert a[1] == b[1] and len(a[1]) == 5
     m.close()
 
 
