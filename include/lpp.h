@@ -243,6 +243,12 @@ typedef struct lpp_kernel_time {
 lpp_status lpp_profile_kernels(lpp_model *m, int pos, int reps, lpp_kernel_time *out, int capacity,
                                int *count);
 
+/* Timeline of one token on LPP_PATH_PERSISTENT at position `pos`: for grid barrier
+ * i, out[2i] is when workgroup 0 arrived and out[2i+1] when it was released, in
+ * 10 ns ticks from the kernel's start.  Barrier order per layer: qkv, attention,
+ * o-projection, gate/up, down; then classifier and four sampler steps. */
+lpp_status lpp_trace_token(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count);
+
 /* ===================================================================== */
 /* C. Runtime plumbing                                                    */
 /* ===================================================================== */

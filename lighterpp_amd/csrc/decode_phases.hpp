@@ -17,6 +17,11 @@
 // first weight loads BEFORE calling the `pre` hook that waits for the previous
 // phase and stages the activations in LDS: weights never depend on activations,
 // so HBM keeps streaming across the phase boundary.
+//
+// kCoh = true is the persistent kernel: whatever one phase hands to the next
+// (q, k, v, x, xb, hb, logits, sampler tables) is written and read with
+// device-coherent accesses (dev::Mem<true>), because producer and consumer may
+// sit on different XCDs and no cache-wide fence is issued at the barriers.
 #pragma once
 
 #include "lpp_device.hpp"
@@ -61,38 +66,57 @@ struct DecodeArgs {
     StepParams* step;
     int* history;          // ring of step->history_cap entries
     const float* uniforms; // per-step draws, or null: use step->r
-    int* out_tokens;       // per-step results, or null
+    int* out_tokens;       // per-step results (may be pinned host memory), or null
     int* sampled;          // [1]
     smp::SampleScratch sample_scratch;
+    unsigned long long* trace;  // optional: timestamps of workgroup 0 at every grid barrier
 };
 
 // ---------------------------------------------------------------------------
 // Activation staging
 // ---------------------------------------------------------------------------
 
-// xs[0..n) = src, zero padded to a multiple of 8.
+// xs[0..n) = src, zero padded to a multiple of 8.  n is even.
+template <bool kCoh>
 __device__ __forceinline__ void stage_plain(float* xs, const float* src, int n) {
     const int n_pad = (n + 7) & ~7;
-    for (int i = threadIdx.x; i < n_pad; i += blockDim.x) xs[i] = (i < n) ? src[i] : 0.0f;
+    for (int i = 2 * threadIdx.x; i < n_pad; i += 2 * blockDim.x) {
+        float2 v = make_float2(0.0f, 0.0f);
+        if (i < n) v = Mem<kCoh>::ld2(src + i);
+        xs[i] = v.x;
+        xs[i + 1] = v.y;
+    }
     __syncthreads();
 }
 
 // xs = rmsnorm(src) * gain, ops.cpp:20-32: (x * s) * w with s = 1/sqrtf(mean + 1e-5f).
+template <bool kCoh>
 __device__ __forceinline__ void stage_rmsnorm(float* xs, const float* src, const float* gain, int n) {
 #pragma clang fp contract(off)
     __shared__ float scratch[16];
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const float v = src[i];
-        xs[i] = v;
-        ss += v * v;
+    for (int i = 2 * threadIdx.x; i < n; i += 2 * blockDim.x) {
+        const float2 v = Mem<kCoh>::ld2(src + i);
+        xs[i] = v.x;
+        xs[i + 1] = v.y;
+        ss += v.x * v.x;
+        ss += v.y * v.y;
     }
     ss = block_sum(ss, scratch);
     ss /= static_cast<float>(n);
     ss += 1e-5f;
     const float scale = 1.0f / sqrtf(ss);
     const int n_pad = (n + 7) & ~7;
-    for (int i = threadIdx.x; i < n_pad; i += blockDim.x) xs[i] = (i < n) ? xs[i] * scale * gain[i] : 0.0f;
+    for (int i = 2 * threadIdx.x; i < n_pad; i += 2 * blockDim.x) {
+        if (i < n) {
+            const float2 g = *reinterpret_cast<const float2*>(gain + i);
+            xs[i] = xs[i] * scale * g.x;
+            xs[i + 1] = xs[i + 1] * scale * g.y;
+        } else {
+            xs[i] = 0.0f;
+            xs[i + 1] = 0.0f;
+        }
+    }
     __syncthreads();
 }
 
@@ -143,64 +167,86 @@ struct Tile {
     }
 };
 
+// Position of one wavefront in its list of work: a tile (kRows rows) and, inside
+// it, a group of kUnroll 1-KiB chunks of every row.
+template <int kRows>
+struct Cursor {
+    int tile;
+    int cg;
+    bool have;
+    const char* rows[kRows];
+};
+
 // One wavefront walks tiles wave_g, wave_g + waves_total, ...; a tile is kRows
-// rows given by row_ptr(tile, r) (null = no such row) and is consumed in groups
-// of kUnroll 1-KiB chunks.  While group g is multiplied, group g+1 (possibly of
-// the next tile) is already in flight.  pre() runs once, after the first loads
-// have been issued and before anything reads xs; every wavefront of the
-// workgroup calls it, with or without work.  epi(tile, sums) receives
-// wave-uniform dot products.
+// rows given by row_ptr(tile, r) (null = no such row) and is consumed in steps
+// of kUnroll chunks.  Two steps are always in flight: both are requested before
+// pre() runs, and each register set is refilled with the step after next as soon
+// as it has been multiplied.  pre() runs once, after those first requests and
+// before anything reads xs; every wavefront of the workgroup calls it, with or
+// without work.  epi(tile, sums) receives wave-uniform dot products.
 template <bool kF16, int kRows, int kUnroll, class RowFn, class EpiFn, class PreFn>
 __device__ __forceinline__ void gemv_phase(int ntiles, int d, const float* xs, int wave_g, int waves_total,
                                            RowFn row_ptr, EpiFn epi, PreFn pre) {
     using T = Tile<kF16, kRows, kUnroll>;
+    using C = Cursor<kRows>;
     const int ncg = (d + T::kChunk * kUnroll - 1) / (T::kChunk * kUnroll);
-    T a, b;
-    int tile = wave_g, cg = 0;
-    bool have = tile < ntiles && ncg > 0;
-    const char* rows[kRows];
+
+    auto start = [&](C& c) {
+        c.tile = wave_g;
+        c.cg = 0;
+        c.have = c.tile < ntiles && ncg > 0;
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) rows[r] = have ? row_ptr(tile, r) : nullptr;
-    if (have) a.load(rows, 0, d);
+        for (int r = 0; r < kRows; ++r) c.rows[r] = c.have ? row_ptr(c.tile, r) : nullptr;
+    };
+    // c <- the step after c
+    auto advance = [&](C& c) {
+        if (!c.have) return;
+        if (c.cg + 1 < ncg) {
+            c.cg += 1;
+            return;
+        }
+        c.cg = 0;
+        c.tile += waves_total;
+        c.have = c.tile < ntiles;
+        if (c.have) {
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) c.rows[r] = row_ptr(c.tile, r);
+        }
+    };
+
+    T ta, tb;
+    C ca, cb;
+    start(ca);
+    cb = ca;
+    advance(cb);
+    if (ca.have) ta.load(ca.rows, ca.cg, d);
+    if (cb.have) tb.load(cb.rows, cb.cg, d);
     pre();
     float acc[kRows];
 #pragma unroll
     for (int r = 0; r < kRows; ++r) acc[r] = 0.0f;
 
-#define LPP_GEMV_STEP(CUR, NXT)                                                   \
+#define LPP_GEMV_STEP(TCUR, CCUR)                                                 \
     {                                                                             \
-        int ntile = tile, ncgi = cg + 1;                                          \
-        if (ncgi == ncg) {                                                        \
-            ncgi = 0;                                                             \
-            ntile = tile + waves_total;                                           \
-        }                                                                         \
-        const bool nhave = ntile < ntiles;                                        \
-        const char* nrows[kRows];                                                 \
-        _Pragma("unroll") for (int r = 0; r < kRows; ++r) nrows[r] = rows[r];     \
-        if (nhave) {                                                              \
-            if (ncgi == 0) {                                                      \
-                _Pragma("unroll") for (int r = 0; r < kRows; ++r) nrows[r] = row_ptr(ntile, r); \
-            }                                                                     \
-            NXT.load(nrows, ncgi, d);                                             \
-        }                                                                         \
-        CUR.fma(xs, cg, d, acc);                                                  \
-        if (ncgi == 0) {                                                          \
+        TCUR.fma(xs, CCUR.cg, d, acc);                                            \
+        const int done_tile = CCUR.tile;                                          \
+        const bool tile_ends = (CCUR.cg + 1 == ncg);                              \
+        advance(CCUR);                                                            \
+        advance(CCUR);                                                            \
+        if (CCUR.have) TCUR.load(CCUR.rows, CCUR.cg, d);                          \
+        if (tile_ends) {                                                          \
             float sums[kRows];                                                    \
             _Pragma("unroll") for (int r = 0; r < kRows; ++r) {                   \
                 sums[r] = wave_sum(acc[r]);                                       \
                 acc[r] = 0.0f;                                                    \
             }                                                                     \
-            epi(tile, sums);                                                      \
+            epi(done_tile, sums);                                                 \
         }                                                                         \
-        tile = ntile;                                                             \
-        cg = ncgi;                                                                \
-        have = nhave;                                                             \
-        _Pragma("unroll") for (int r = 0; r < kRows; ++r) rows[r] = nrows[r];     \
     }
-    while (have) {
-        LPP_GEMV_STEP(a, b)
-        if (!have) break;
-        LPP_GEMV_STEP(b, a)
+    while (ca.have) {
+        LPP_GEMV_STEP(ta, ca)
+        if (!cb.have) break;
+        LPP_GEMV_STEP(tb, cb)
     }
 #undef LPP_GEMV_STEP
 }
@@ -216,10 +262,20 @@ __device__ __forceinline__ const float* layer_input(const DecodeArgs& a, int lay
     return layer == 0 ? a.emb + static_cast<size_t>(a.step->token) * a.dim : a.x;
 }
 
+// Pick element `lane` of a small wave-uniform array without dynamic indexing.
+template <int kN>
+__device__ __forceinline__ float pick(const float (&v)[kN], int lane) {
+    float out = v[0];
+#pragma unroll
+    for (int r = 1; r < kN; ++r)
+        if (lane == r) out = v[r];
+    return out;
+}
+
 // ---------------------------------------------------------------------------
 // Phase: rmsnorm -> QKV -> RoPE -> q buffer and K/V cache
 // ---------------------------------------------------------------------------
-template <bool kF16, int kRows, class PreFn>
+template <bool kF16, int kRows, bool kCoh, class PreFn>
 __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg, int nwg, float* xs, PreFn pre) {
 #pragma clang fp contract(off)
     static_assert(kRows % 2 == 0, "RoPE pairs must stay inside a tile");
@@ -239,7 +295,7 @@ __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg
     };
     auto prologue = [&]() {
         pre();
-        stage_rmsnorm(xs, layer_input(a, layer), a.rms_att + static_cast<size_t>(layer) * dim, dim);
+        stage_rmsnorm<kCoh>(xs, layer_input(a, layer), a.rms_att + static_cast<size_t>(layer) * dim, dim);
     };
     auto epilogue = [&](int tile, float (&sums)[kRows]) {
         if (lane_id() != 0) return;
@@ -261,8 +317,8 @@ __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg
                 e1 = r1;
             }
             if (g < dim) {
-                a.q[g] = e0;
-                a.q[g + 1] = e1;
+                Mem<kCoh>::st(a.q + g, e0);
+                Mem<kCoh>::st(a.q + g + 1, e1);
             } else {
                 // model.cpp:171-176 / scatter_kv.cu:15-18.
                 const bool is_k = g < dim + kv_dim;
@@ -272,8 +328,8 @@ __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg
                                    static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(pos) * hs + within;
                 float* plain = is_k ? a.k : a.v;
                 uint16_t* cache = is_k ? a.key_cache : a.value_cache;
-                plain[i] = e0;
-                plain[i + 1] = e1;
+                Mem<kCoh>::st(plain + i, e0);
+                Mem<kCoh>::st(plain + i + 1, e1);
                 cache[dst] = f32_to_f16_bits(e0);
                 cache[dst + 1] = f32_to_f16_bits(e1);
             }
@@ -285,7 +341,7 @@ __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg
 // ---------------------------------------------------------------------------
 // Phase: out = W . xs + residual   (O projection and down projection)
 // ---------------------------------------------------------------------------
-template <bool kF16, int kRows, class PreFn>
+template <bool kF16, int kRows, bool kCoh, class PreFn>
 __device__ __forceinline__ void phase_proj_residual(const char* w_layer, int n, int d, const float* src,
                                                     const float* residual, float* out, int wg, int nwg,
                                                     float* xs, PreFn pre) {
@@ -299,18 +355,15 @@ __device__ __forceinline__ void phase_proj_residual(const char* w_layer, int n, 
     };
     auto prologue = [&]() {
         pre();
-        stage_plain(xs, src, d);
+        stage_plain<kCoh>(xs, src, d);
     };
     auto epilogue = [&](int tile, float (&sums)[kRows]) {
         const int lane = lane_id();
         if (lane >= kRows) return;
         const int g = tile * kRows + lane;
         if (g >= n) return;
-        float v = sums[0];
-#pragma unroll
-        for (int r = 1; r < kRows; ++r)
-            if (lane == r) v = sums[r];
-        out[g] = residual[g] + v;  // model.cpp:232,239: x[i] += xb2[i]
+        const float v = pick<kRows>(sums, lane);
+        Mem<kCoh>::st(out + g, Mem<kCoh>::ld(residual + g) + v);  // model.cpp:232,239: x[i] += xb2[i]
     };
     gemv_phase<kF16, kRows, 4>(ntiles, d, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
 }
@@ -318,7 +371,7 @@ __device__ __forceinline__ void phase_proj_residual(const char* w_layer, int n, 
 // ---------------------------------------------------------------------------
 // Phase: rmsnorm -> gate/up -> SwiGLU -> hb
 // ---------------------------------------------------------------------------
-template <bool kF16, int kPairRows, class PreFn>
+template <bool kF16, int kPairRows, bool kCoh, class PreFn>
 __device__ __forceinline__ void phase_gateup(const DecodeArgs& a, int layer, int wg, int nwg, float* xs, PreFn pre) {
 #pragma clang fp contract(off)
     constexpr int kRows = 2 * kPairRows;
@@ -334,7 +387,7 @@ __device__ __forceinline__ void phase_gateup(const DecodeArgs& a, int layer, int
     };
     auto prologue = [&]() {
         pre();
-        stage_rmsnorm(xs, a.x, a.rms_ffn + static_cast<size_t>(layer) * dim, dim);
+        stage_rmsnorm<kCoh>(xs, a.x, a.rms_ffn + static_cast<size_t>(layer) * dim, dim);
     };
     auto epilogue = [&](int tile, float (&sums)[kRows]) {
         const int lane = lane_id();
@@ -350,7 +403,7 @@ __device__ __forceinline__ void phase_gateup(const DecodeArgs& a, int layer, int
             }
         // ops.cpp:80-85
         const float sigma = 1.0f / (1.0f + expf(-gate));
-        a.hb[g] = (gate * sigma) * up;
+        Mem<kCoh>::st(a.hb + g, (gate * sigma) * up);
     };
     gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
 }
@@ -358,7 +411,7 @@ __device__ __forceinline__ void phase_gateup(const DecodeArgs& a, int layer, int
 // ---------------------------------------------------------------------------
 // Phase: final rmsnorm -> classifier -> logits
 // ---------------------------------------------------------------------------
-template <bool kF16, int kRows, class PreFn>
+template <bool kF16, int kRows, bool kCoh, class PreFn>
 __device__ __forceinline__ void phase_lmhead(const DecodeArgs& a, int wg, int nwg, float* xs, PreFn pre) {
     const int wbytes = kF16 ? 2 : 4;
     const int waves_per_wg = static_cast<int>(blockDim.x) / kWave;
@@ -371,18 +424,14 @@ __device__ __forceinline__ void phase_lmhead(const DecodeArgs& a, int wg, int nw
     };
     auto prologue = [&]() {
         pre();
-        stage_rmsnorm(xs, a.x, a.rms_final, dim);
+        stage_rmsnorm<kCoh>(xs, a.x, a.rms_final, dim);
     };
     auto epilogue = [&](int tile, float (&sums)[kRows]) {
         const int lane = lane_id();
         if (lane >= kRows) return;
         const int g = tile * kRows + lane;
         if (g >= vocab) return;
-        float v = sums[0];
-#pragma unroll
-        for (int r = 1; r < kRows; ++r)
-            if (lane == r) v = sums[r];
-        a.logits[g] = v;
+        Mem<kCoh>::st(a.logits + g, pick<kRows>(sums, lane));
     };
     gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
 }
@@ -419,14 +468,40 @@ __host__ __device__ inline int attention_lds_floats(int gqa, int head_size, int 
            + (nthreads / kWave) * gqa * hs_pad;  // cross-wave reduction
 }
 
+// 8 binary16 values of a cache row.  The row of the position being decoded was
+// stored by another workgroup earlier in the same persistent kernel; there it is
+// taken from the fp32 k / v vector (coherent read) and rounded exactly as the
+// cache store rounds it, so both schedules see identical values.
+template <bool kCoh>
+__device__ __forceinline__ uintx4 cache_row8(const uint16_t* cache_row, const float* fresh, bool is_current,
+                                             int offset) {
+    if constexpr (kCoh) {
+        if (is_current) {
+            union {
+                half8_t h;
+                uintx4 u;
+            } c;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float2 f = Mem<true>::ld2(fresh + offset + 2 * j);
+                c.h[2 * j] = static_cast<half_t>(f.x);
+                c.h[2 * j + 1] = static_cast<half_t>(f.y);
+            }
+            return c.u;
+        }
+    }
+    return load16(cache_row + offset);
+}
+
 // One work item: KV head `kvh`, context split `split` of `nsplits`.  kGroup lanes
 // cover one position (8 binary16 each).  Sub-blocks of kAttBlock positions:
 // scores -> LDS, per-head max/exp/sum by one wavefront per head, then V
 // accumulation with the running-max correction (the sum the CPU forms at
-// model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped).  The partial
-// (max, sum, unnormalised output) goes to att_partial; the last split to arrive
-// for this KV head combines all splits into xb.
-template <int kGroup>
+// model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped).  With one
+// split the result goes straight to xb; otherwise the partial (max, sum,
+// unnormalised output) goes to att_partial and the last split to arrive for
+// this KV head combines all of them.
+template <int kGroup, bool kCoh>
 __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int split, int nsplits, int npos,
                                float* lds) {
     const int hs = a.head_size, gqa = a.gqa;
@@ -448,7 +523,7 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
     const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
     for (int i = tid; i < gqa * hs_pad; i += nthreads) {
         const int qh = i / hs_pad, e = i - qh * hs_pad;
-        qs[i] = (e < hs) ? a.q[static_cast<size_t>(kvh * gqa + qh) * hs + e] : 0.0f;
+        qs[i] = (e < hs) ? Mem<kCoh>::ld(a.q + static_cast<size_t>(kvh * gqa + qh) * hs + e) : 0.0f;
     }
     if (tid < gqa) {
         run_max[tid] = -INFINITY;
@@ -457,9 +532,12 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
     const int chunk = (npos + nsplits - 1) / nsplits;
     const int t_begin = split * chunk;
     const int t_end = min(npos, t_begin + chunk);
+    const int current = npos - 1;
     const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
     const uint16_t* kbase = a.key_cache + head_base;
     const uint16_t* vbase = a.value_cache + head_base;
+    const float* k_fresh = a.k + static_cast<size_t>(kvh) * hs;
+    const float* v_fresh = a.v + static_cast<size_t>(kvh) * hs;
 
     float acc[kMaxGqa][8];
 #pragma unroll
@@ -468,20 +546,43 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
         for (int e = 0; e < 8; ++e) acc[qh][e] = 0.0f;
     __syncthreads();
 
-    for (int b0 = t_begin; b0 < t_end; b0 += kAttBlock) {
-        const int b1 = min(t_end, b0 + kAttBlock);
-        // scores of this sub-block
-        for (int t = b0 + grp; t < b1; t += ngroups) {
-            uintx4 kb = uintx4{0u, 0u, 0u, 0u};
-            if (sub * 8 < hs) kb = load16(kbase + static_cast<size_t>(t) * hs + sub * 8);
+    // A sub-block is `per_group` consecutive rounds of ngroups positions.  Every
+    // lane requests all its K rows and all its V rows of the sub-block before the
+    // first multiply (up to 16 independent 16-byte loads in flight), so a
+    // sub-block costs about one memory round trip instead of one per position.
+    constexpr int kMaxPerGroup = 8;
+    int per_group = kAttBlock / ngroups;
+    if (per_group > kMaxPerGroup) per_group = kMaxPerGroup;
+    if (per_group < 1) per_group = 1;
+    const int sub_block = per_group * ngroups;  // <= kAttBlock
+    const bool lane_live = sub * 8 < hs;
+    for (int b0 = t_begin; b0 < t_end; b0 += sub_block) {
+        const int b1 = min(t_end, b0 + sub_block);
+        uintx4 kreg[kMaxPerGroup], vreg[kMaxPerGroup];
 #pragma unroll
-            for (int qh = 0; qh < kMaxGqa; ++qh) {
-                if (qh < gqa) {
-                    const float* qv = qs + qh * hs_pad + sub * 8;
-                    const floatx4 xa = *reinterpret_cast<const floatx4*>(qv);
-                    const floatx4 xb = *reinterpret_cast<const floatx4*>(qv + 4);
-                    const float s = group_sum<kGroup>(dot8(kb, xa, xb, 0.0f));
-                    if (sub == 0) sc[qh * kAttBlock + (t - b0)] = s * scale;
+        for (int j = 0; j < kMaxPerGroup; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            kreg[j] = uintx4{0u, 0u, 0u, 0u};
+            vreg[j] = uintx4{0u, 0u, 0u, 0u};
+            if (j < per_group && t < b1 && lane_live) {
+                kreg[j] = cache_row8<kCoh>(kbase + static_cast<size_t>(t) * hs, k_fresh, t == current, sub * 8);
+                vreg[j] = cache_row8<kCoh>(vbase + static_cast<size_t>(t) * hs, v_fresh, t == current, sub * 8);
+            }
+        }
+        // scores of this sub-block
+#pragma unroll
+        for (int j = 0; j < kMaxPerGroup; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            if (j < per_group && t < b1) {
+#pragma unroll
+                for (int qh = 0; qh < kMaxGqa; ++qh) {
+                    if (qh < gqa) {
+                        const float* qv = qs + qh * hs_pad + sub * 8;
+                        const floatx4 xa = *reinterpret_cast<const floatx4*>(qv);
+                        const floatx4 xb = *reinterpret_cast<const floatx4*>(qv + 4);
+                        const float s = group_sum<kGroup>(dot8(kreg[j], xa, xb, 0.0f));
+                        if (sub == 0) sc[qh * kAttBlock + (t - b0)] = s * scale;
+                    }
                 }
             }
         }
@@ -510,7 +611,7 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
             }
         }
         __syncthreads();
-        // value accumulation
+        // value accumulation from the rows already in registers
 #pragma unroll
         for (int qh = 0; qh < kMaxGqa; ++qh) {
             if (qh < gqa) {
@@ -519,9 +620,11 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
                 for (int e = 0; e < 8; ++e) acc[qh][e] *= c;
             }
         }
-        if (sub * 8 < hs) {
-            for (int t = b0 + grp; t < b1; t += ngroups) {
-                const half8_t vv = as_half8(load16(vbase + static_cast<size_t>(t) * hs + sub * 8));
+#pragma unroll
+        for (int j = 0; j < kMaxPerGroup; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            if (j < per_group && t < b1 && lane_live) {
+                const half8_t vv = as_half8(vreg[j]);
 #pragma unroll
                 for (int qh = 0; qh < kMaxGqa; ++qh) {
                     if (qh < gqa) {
@@ -561,53 +664,52 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
             const int qh = i / hs, e = i - qh * hs;
             float o = 0.0f;
             for (int w = 0; w < nwaves; ++w) o += red[(w * gqa + qh) * hs_pad + e];
-            a.xb[static_cast<size_t>(kvh * gqa + qh) * hs + e] = o / run_sum[qh];
+            Mem<kCoh>::st(a.xb + static_cast<size_t>(kvh * gqa + qh) * hs + e, o / run_sum[qh]);
         }
         return;
     }
+    // Partials always travel with device-coherent accesses: writer and combiner
+    // are different workgroups of one launch in both schedules.
     for (int i = tid; i < gqa * hs; i += nthreads) {
         const int qh = i / hs, e = i - qh * hs;
         float o = 0.0f;
         for (int w = 0; w < nwaves; ++w) o += red[(w * gqa + qh) * hs_pad + e];
         float* part = a.att_partial + (static_cast<size_t>(kvh * gqa + qh) * a.max_splits + split) * stride;
-        part[e] = o;
+        Mem<true>::st(part + e, o);
         if (e == 0) {
-            part[hs] = run_max[qh];
-            part[hs + 1] = run_sum[qh];
+            Mem<true>::st(part + hs, run_max[qh]);
+            Mem<true>::st(part + hs + 1, run_sum[qh]);
         }
     }
 
-    // The last split to arrive for this KV head combines all of them.  Writers
-    // publish with a release fence before taking a ticket; the combiner acquires
-    // after seeing the last ticket, then reads the partials with ordinary loads.
+    // The last split to arrive for this KV head combines all of them.  The block
+    // barrier waits for this workgroup's stores; the ticket is taken after it.
     __shared__ int is_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     if (tid == 0) {
-        const unsigned ticket = atomicAdd(&a.att_count[kvh], 1u);
+        const unsigned ticket = __hip_atomic_fetch_add(&a.att_count[kvh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (ticket == static_cast<unsigned>(nsplits - 1)) ? 1 : 0;
-        if (is_last) a.att_count[kvh] = 0u;  // ready for the next layer
+        if (is_last) __hip_atomic_store(&a.att_count[kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!is_last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     for (int i = tid; i < gqa * hs; i += nthreads) {
         const int qh = i / hs, e = i - qh * hs;
         const float* base = a.att_partial + static_cast<size_t>(kvh * gqa + qh) * a.max_splits * stride;
         float top = -INFINITY;
-        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, base[s * stride + hs]);
+        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, Mem<true>::ld(base + s * stride + hs));
         float o = 0.0f, l = 0.0f;
         for (int s = 0; s < nsplits; ++s) {
-            const float ms = base[s * stride + hs];
+            const float ms = Mem<true>::ld(base + s * stride + hs);
             const float wgt = (ms == -INFINITY) ? 0.0f : expf(ms - top);
-            o += base[s * stride + e] * wgt;
-            l += base[s * stride + hs + 1] * wgt;
+            o += Mem<true>::ld(base + s * stride + e) * wgt;
+            l += Mem<true>::ld(base + s * stride + hs + 1) * wgt;
         }
-        a.xb[static_cast<size_t>(kvh * gqa + qh) * hs + e] = o / l;
+        Mem<kCoh>::st(a.xb + static_cast<size_t>(kvh * gqa + qh) * hs + e, o / l);
     }
 }
 
-template <class PreFn>
+template <bool kCoh, class PreFn>
 __device__ __forceinline__ void phase_attention(const DecodeArgs& a, int layer, int wg, int nwg, float* lds,
                                                 PreFn pre) {
     pre();
@@ -617,11 +719,11 @@ __device__ __forceinline__ void phase_attention(const DecodeArgs& a, int layer, 
     const int hs = a.head_size;
     for (int item = wg; item < items; item += nwg) {
         const int kvh = item / nsplits, split = item - kvh * nsplits;
-        if (hs <= 8) attention_item<1>(a, layer, kvh, split, nsplits, npos, lds);
-        else if (hs <= 16) attention_item<2>(a, layer, kvh, split, nsplits, npos, lds);
-        else if (hs <= 32) attention_item<4>(a, layer, kvh, split, nsplits, npos, lds);
-        else if (hs <= 64) attention_item<8>(a, layer, kvh, split, nsplits, npos, lds);
-        else attention_item<16>(a, layer, kvh, split, nsplits, npos, lds);
+        if (hs <= 8) attention_item<1, kCoh>(a, layer, kvh, split, nsplits, npos, lds);
+        else if (hs <= 16) attention_item<2, kCoh>(a, layer, kvh, split, nsplits, npos, lds);
+        else if (hs <= 32) attention_item<4, kCoh>(a, layer, kvh, split, nsplits, npos, lds);
+        else if (hs <= 64) attention_item<8, kCoh>(a, layer, kvh, split, nsplits, npos, lds);
+        else attention_item<16, kCoh>(a, layer, kvh, split, nsplits, npos, lds);
         __syncthreads();
     }
 }
@@ -632,6 +734,37 @@ __device__ __forceinline__ void phase_attention(const DecodeArgs& a, int layer, 
 
 __device__ __forceinline__ float step_uniform(const DecodeArgs& a) {
     return a.uniforms ? a.uniforms[a.step->step_index] : a.step->r;
+}
+
+// Chunk c of the vocabulary: penalty, temperature, chunk maximum.
+template <bool kCoh>
+__device__ __forceinline__ void sample_step_scale(const DecodeArgs& a, int chunk, int c) {
+    const StepParams* sp = a.step;
+    smp::scale_max_chunk<kCoh>(a.logits, a.work, a.vocab, chunk, c, sp->temperature, sp->penalty,
+                               sp->history_len > 0 ? a.history : nullptr, sp->history_len, a.sample_scratch);
+}
+// Greedy (model.cpp:272-283) finishes here in chunk 0; otherwise exponentials.
+template <bool kCoh>
+__device__ __forceinline__ void sample_step_exp(const DecodeArgs& a, int chunk, int nchunks, int c) {
+    if (a.step->temperature == 0.0f) {
+        if (c == 0) {
+            const int tok = smp::argmax_over_chunks<kCoh>(nchunks, a.sample_scratch);
+            if (threadIdx.x == 0) Mem<kCoh>::sti(a.sampled, tok);
+        }
+        return;
+    }
+    smp::exp_sum_chunk<kCoh>(a.work, a.vocab, chunk, nchunks, c, a.sample_scratch);
+}
+template <bool kCoh>
+__device__ __forceinline__ void sample_step_norm(const DecodeArgs& a, int chunk, int nchunks, int c) {
+    if (a.step->temperature == 0.0f) return;
+    smp::normalise_chunk<kCoh>(a.work, a.vocab, chunk, nchunks, c, a.sample_scratch);
+    if (c == 0 && threadIdx.x == 0) Mem<kCoh>::sti(a.sampled, a.vocab - 1);  // model.cpp:302
+}
+template <bool kCoh>
+__device__ __forceinline__ void sample_step_search(const DecodeArgs& a, int chunk, int c) {
+    if (a.step->temperature == 0.0f) return;
+    smp::cdf_search_chunk<kCoh>(a.work, a.vocab, chunk, c, step_uniform(a), a.sample_scratch, a.sampled);
 }
 
 // After the sampler: publish the token, feed it back as the next input, advance
@@ -653,7 +786,7 @@ __device__ __forceinline__ void finish_token(const DecodeArgs& a, int token, uns
     sp->token = token;
     sp->pos += 1;
     sp->step_index = index + 1;
-    if (a.out_tokens) __hip_atomic_store(a.out_tokens + index, token, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (a.out_tokens) __hip_atomic_store(a.out_tokens + index, token, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 }  // namespace ph

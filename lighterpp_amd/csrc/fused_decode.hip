@@ -41,12 +41,12 @@ struct NoWait {
 template <bool kF16>
 __global__ __launch_bounds__(kThreads) void k_qkv(DecodeArgs a, int layer) {
     extern __shared__ __align__(16) float lds[];
-    phase_qkv<kF16, 2>(a, layer, blockIdx.x, gridDim.x, lds, NoWait{});
+    phase_qkv<kF16, 2, false>(a, layer, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
 __global__ __launch_bounds__(kThreads) void k_attention(DecodeArgs a, int layer) {
     extern __shared__ __align__(16) float lds[];
-    phase_attention(a, layer, blockIdx.x, gridDim.x, lds, NoWait{});
+    phase_attention<false>(a, layer, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
 template <bool kF16>
@@ -54,14 +54,14 @@ __global__ __launch_bounds__(kThreads) void k_oproj(DecodeArgs a, int layer) {
     extern __shared__ __align__(16) float lds[];
     const int wbytes = kF16 ? 2 : 4;
     const char* w = a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes;
-    phase_proj_residual<kF16, 2>(w, a.dim, a.dim, a.xb, layer_input(a, layer), a.x, blockIdx.x, gridDim.x, lds,
+    phase_proj_residual<kF16, 2, false>(w, a.dim, a.dim, a.xb, layer_input(a, layer), a.x, blockIdx.x, gridDim.x, lds,
                                  NoWait{});
 }
 
 template <bool kF16>
 __global__ __launch_bounds__(kThreads) void k_gateup(DecodeArgs a, int layer) {
     extern __shared__ __align__(16) float lds[];
-    phase_gateup<kF16, 2>(a, layer, blockIdx.x, gridDim.x, lds, NoWait{});
+    phase_gateup<kF16, 2, false>(a, layer, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
 template <bool kF16>
@@ -69,53 +69,27 @@ __global__ __launch_bounds__(kThreads) void k_down(DecodeArgs a, int layer) {
     extern __shared__ __align__(16) float lds[];
     const int wbytes = kF16 ? 2 : 4;
     const char* w = a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes;
-    phase_proj_residual<kF16, 1>(w, a.dim, a.hidden, a.hb, a.x, a.x, blockIdx.x, gridDim.x, lds, NoWait{});
+    phase_proj_residual<kF16, 1, false>(w, a.dim, a.hidden, a.hb, a.x, a.x, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
 template <bool kF16>
 __global__ __launch_bounds__(kThreads) void k_lmhead(DecodeArgs a) {
     extern __shared__ __align__(16) float lds[];
-    phase_lmhead<kF16, 4>(a, blockIdx.x, gridDim.x, lds, NoWait{});
+    phase_lmhead<kF16, 4, false>(a, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
 // Sampler steps; chunk c of the vocabulary is handled by workgroup c.
-__device__ __forceinline__ void sample_step_scale(const DecodeArgs& a, int chunk, int c) {
-    const StepParams* sp = a.step;
-    smp::scale_max_chunk(a.logits, a.work, a.vocab, chunk, c, sp->temperature, sp->penalty,
-                         sp->history_len > 0 ? a.history : nullptr, sp->history_len, a.sample_scratch);
-}
-// Greedy (model.cpp:272-283) finishes here in chunk 0; otherwise exponentials.
-__device__ __forceinline__ void sample_step_exp(const DecodeArgs& a, int chunk, int nchunks, int c) {
-    if (a.step->temperature == 0.0f) {
-        if (c == 0) {
-            const int tok = smp::argmax_over_chunks(nchunks, a.sample_scratch);
-            if (threadIdx.x == 0) a.sampled[0] = tok;
-        }
-        return;
-    }
-    smp::exp_sum_chunk(a.work, a.vocab, chunk, nchunks, c, a.sample_scratch);
-}
-__device__ __forceinline__ void sample_step_norm(const DecodeArgs& a, int chunk, int nchunks, int c) {
-    if (a.step->temperature == 0.0f) return;
-    smp::normalise_chunk(a.work, a.vocab, chunk, nchunks, c, a.sample_scratch);
-    if (c == 0 && threadIdx.x == 0) a.sampled[0] = a.vocab - 1;  // model.cpp:302
-}
-__device__ __forceinline__ void sample_step_search(const DecodeArgs& a, int chunk, int c) {
-    if (a.step->temperature == 0.0f) return;
-    smp::cdf_search_chunk(a.work, a.vocab, chunk, c, step_uniform(a), a.sample_scratch, a.sampled);
-}
-
 __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_scale(DecodeArgs a, int chunk) {
-    sample_step_scale(a, chunk, blockIdx.x);
+    sample_step_scale<false>(a, chunk, blockIdx.x);
 }
 __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_exp(DecodeArgs a, int chunk, int nchunks) {
-    sample_step_exp(a, chunk, nchunks, blockIdx.x);
+    sample_step_exp<false>(a, chunk, nchunks, blockIdx.x);
 }
 __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_norm(DecodeArgs a, int chunk, int nchunks) {
-    sample_step_norm(a, chunk, nchunks, blockIdx.x);
+    sample_step_norm<false>(a, chunk, nchunks, blockIdx.x);
 }
 __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_search(DecodeArgs a, int chunk) {
-    sample_step_search(a, chunk, blockIdx.x);
+    sample_step_search<false>(a, chunk, blockIdx.x);
 }
 __global__ void k_finish(DecodeArgs a) {
     if (threadIdx.x == 0 && blockIdx.x == 0) finish_token(a, a.sampled[0], 0u);
@@ -128,9 +102,12 @@ __global__ void k_finish(DecodeArgs a) {
 // Grid barrier over a monotonically increasing arrival counter.  Barrier number
 // i of the token whose generation base is `base` is complete when the counter
 // has reached (base + i + 1) * nwg; the counter is never reset, comparisons are
-// wrap-safe.  The wait is bounded: after spin_limit polls the workgroup records
-// an error, raises the shared abort flag and every later wait returns at once,
-// so the grid always drains.
+// wrap-safe.  No cache-wide fence is issued: everything that crosses the
+// barrier is written and read with device-coherent accesses (dev::Mem<true>),
+// and the block barrier in arrive() has already waited for those stores.  The
+// wait is bounded: after spin_limit polls the workgroup records an error, raises
+// the shared abort flag and every later wait returns at once, so the grid always
+// drains.
 struct GridSync {
     unsigned* counter;
     unsigned* abort_flag;
@@ -139,12 +116,13 @@ struct GridSync {
     unsigned nwg;
     unsigned spin_limit;
     unsigned index;
+    unsigned long long* trace;  // workgroup 0 only: [2i] = arrival at barrier i, [2i+1] = release from it
 
     __device__ __forceinline__ void arrive() {
-        __syncthreads();  // every wavefront of the workgroup has issued its stores
+        __syncthreads();  // every wavefront's stores of this phase have completed
         if (threadIdx.x == 0) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (trace) trace[2u * index] = wall_clock64();
         }
     }
 
@@ -153,17 +131,19 @@ struct GridSync {
             const unsigned target = (base + index + 1u) * nwg;
             unsigned spins = 0;
             while (static_cast<int>(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-                if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
+                if ((spins & 63u) == 63u &&
+                    __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
+                    break;
                 if (++spins > spin_limit) {
                     __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     step->error = 1;
                     break;
                 }
-                __builtin_amdgcn_s_sleep(2);
+                __builtin_amdgcn_s_sleep(1);
             }
+            if (trace) trace[2u * index + 1u] = wall_clock64();
         }
         __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         ++index;
     }
 };
@@ -178,45 +158,47 @@ __global__ __launch_bounds__(kPersistThreads) void k_decode_token(DecodeArgs a, 
                                                                   unsigned spin_limit) {
     extern __shared__ __align__(16) float lds[];
     const int wg = blockIdx.x, nwg = gridDim.x;
-    GridSync gs{counter, abort_flag, a.step, a.step->epoch, static_cast<unsigned>(nwg), spin_limit, 0u};
+    GridSync gs{counter, abort_flag, a.step, a.step->epoch, static_cast<unsigned>(nwg), spin_limit, 0u,
+                (wg == 0) ? a.trace : nullptr};
+    if (gs.trace && threadIdx.x == 0) gs.trace[2u * barriers_per_token(a.n_layers)] = wall_clock64();
     auto wait = [&]() { gs.wait(); };
     const int wbytes = kF16 ? 2 : 4;
 
     for (int layer = 0; layer < a.n_layers; ++layer) {
-        if (layer == 0) phase_qkv<kF16, 2>(a, layer, wg, nwg, lds, NoWait{});  // previous token ended at a kernel boundary
-        else phase_qkv<kF16, 2>(a, layer, wg, nwg, lds, wait);
+        if (layer == 0) phase_qkv<kF16, 2, true>(a, layer, wg, nwg, lds, NoWait{});  // previous token ended at a kernel boundary
+        else phase_qkv<kF16, 2, true>(a, layer, wg, nwg, lds, wait);
         gs.arrive();
-        phase_attention(a, layer, wg, nwg, lds, wait);
+        phase_attention<true>(a, layer, wg, nwg, lds, wait);
         gs.arrive();
-        phase_proj_residual<kF16, 2>(a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes, a.dim, a.dim, a.xb,
+        phase_proj_residual<kF16, 2, true>(a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes, a.dim, a.dim, a.xb,
                                      layer_input(a, layer), a.x, wg, nwg, lds, wait);
         gs.arrive();
-        phase_gateup<kF16, 2>(a, layer, wg, nwg, lds, wait);
+        phase_gateup<kF16, 2, true>(a, layer, wg, nwg, lds, wait);
         gs.arrive();
-        phase_proj_residual<kF16, 1>(a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden,
+        phase_proj_residual<kF16, 1, true>(a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden,
                                      a.hb, a.x, a.x, wg, nwg, lds, wait);
         gs.arrive();
     }
-    phase_lmhead<kF16, 4>(a, wg, nwg, lds, wait);
+    phase_lmhead<kF16, 4, true>(a, wg, nwg, lds, wait);
     gs.arrive();
 
     const int chunk = smp::chunk_size_for(a.vocab);
     const int nchunks = (a.vocab + chunk - 1) / chunk;
     gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_scale(a, chunk, c);
+    for (int c = wg; c < nchunks; c += nwg) sample_step_scale<true>(a, chunk, c);
     gs.arrive();
     gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_exp(a, chunk, nchunks, c);
+    for (int c = wg; c < nchunks; c += nwg) sample_step_exp<true>(a, chunk, nchunks, c);
     gs.arrive();
     gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_norm(a, chunk, nchunks, c);
+    for (int c = wg; c < nchunks; c += nwg) sample_step_norm<true>(a, chunk, nchunks, c);
     gs.arrive();
     gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_search(a, chunk, c);
+    for (int c = wg; c < nchunks; c += nwg) sample_step_search<true>(a, chunk, c);
     gs.arrive();
     if (wg == 0) {
         gs.wait();
-        if (threadIdx.x == 0) finish_token(a, a.sampled[0], barriers_per_token(a.n_layers));
+        if (threadIdx.x == 0) finish_token(a, Mem<true>::ldi(a.sampled), barriers_per_token(a.n_layers));
     }
 }
 
@@ -271,6 +253,7 @@ DecodeArgs make_args(const lpp_model* m, bool with_arrays) {
     float* sc = m->sample_scratch;
     a.sample_scratch = smp::SampleScratch{sc, reinterpret_cast<int*>(sc + smp::kMaxChunks),
                                           sc + 2 * smp::kMaxChunks, sc + 3 * smp::kMaxChunks};
+    a.trace = nullptr;
     return a;
 }
 
@@ -744,4 +727,50 @@ extern "C" lpp_status lpp_profile_kernels(lpp_model* m, int pos, int reps, lpp_k
     LPP_HIP(hipStreamSynchronize(stream()));
     return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? profile_impl<true>(m, pos, reps, out, capacity, count)
                                                       : profile_impl<false>(m, pos, reps, out, capacity, count);
+}
+
+// Timeline of one token on the persistent path: for every grid barrier, when
+// workgroup 0 arrived at it and when it was released, in 10 ns ticks relative to
+// the kernel's first instruction.  out[2i] / out[2i+1]; *count = 2 * barriers.
+extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count) {
+    using namespace lpp;
+    LPP_REQUIRE(m && out && count, "lpp_trace_token: null argument");
+    LPP_REQUIRE(pos >= 0 && pos < m->cfg.seq_len, "lpp_trace_token: pos %d outside [0, %d)", pos, m->cfg.seq_len);
+    if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
+    for (int t = 0; t < LPP_T_COUNT; ++t)
+        if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
+    const int nb = static_cast<int>(barriers_per_token(m->cfg.n_layers));
+    LPP_REQUIRE(capacity >= 2 * nb, "lpp_trace_token: capacity %d < %d", capacity, 2 * nb);
+    const int saved_path = m->path;
+    m->path = LPP_PATH_PERSISTENT;
+    unsigned long long* d_trace = nullptr;
+    void* p = nullptr;
+    LPP_TRY(lpp_malloc(&p, static_cast<size_t>(2 * nb + 1) * sizeof(unsigned long long)));
+    d_trace = static_cast<unsigned long long*>(p);
+    StepParams sp{};
+    sp.pos = pos;
+    sp.temperature = 0.8f;
+    sp.penalty = 1.0f;
+    sp.r = 0.5f;
+    sp.freeze = 1;
+    lpp_status st = begin_run(m, sp, stream());
+    hipStream_t s = stream();
+    for (int rep = 0; rep < 3 && st == LPP_OK; ++rep) {  // the last replay is the one reported
+        DecodeArgs a = make_args(m, false);
+        a.trace = d_trace;
+        st = m->cfg.weight_precision == LPP_WEIGHT_FP16 ? persistent_launch<true>(m, a, s)
+                                                        : persistent_launch<false>(m, a, s);
+    }
+    std::vector<unsigned long long> host(static_cast<size_t>(2 * nb + 1));
+    if (st == LPP_OK && hipStreamSynchronize(s) != hipSuccess) st = fail(LPP_ERR_HIP, "trace run failed");
+    if (st == LPP_OK && hipMemcpy(host.data(), d_trace, host.size() * sizeof(unsigned long long),
+                                  hipMemcpyDeviceToHost) != hipSuccess)
+        st = fail(LPP_ERR_HIP, "trace copy failed");
+    lpp_free(d_trace);
+    m->path = saved_path;
+    if (st != LPP_OK) return st;
+    const unsigned long long t0 = host[static_cast<size_t>(2 * nb)];
+    for (int i = 0; i < 2 * nb; ++i) out[i] = host[static_cast<size_t>(i)] - t0;
+    *count = 2 * nb;
+    return LPP_OK;
 }

@@ -243,6 +243,47 @@ __device__ __forceinline__ void wave_rows_dot(const char* const (&rows)[kRows], 
     for (int r = 0; r < kRows; ++r) result[r] = wave_sum(acc[r]);
 }
 
+// Accessors for values that cross workgroups INSIDE one kernel (the persistent
+// decode kernel).  The eight XCDs of the device have separate L2 caches, and
+// whole-cache acquire/release fences cost tens of microseconds per grid barrier
+// here; instead, every such value is written through and read around the
+// non-coherent cache levels with device-scope accesses (sc1), which is all a
+// consumer needs once the barrier has ordered the two sides.  kCoherent = false
+// is the ordinary access for kernels whose inputs were complete before launch.
+template <bool kCoherent>
+struct Mem {
+    static __device__ __forceinline__ float ld(const float* p) {
+        if constexpr (kCoherent) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else return *p;
+    }
+    static __device__ __forceinline__ int ldi(const int* p) {
+        if constexpr (kCoherent) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else return *p;
+    }
+    static __device__ __forceinline__ void st(float* p, float v) {
+        if constexpr (kCoherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else *p = v;
+    }
+    static __device__ __forceinline__ void sti(int* p, int v) {
+        if constexpr (kCoherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else *p = v;
+    }
+    // Two adjacent floats (8-byte aligned) in one access.
+    static __device__ __forceinline__ float2 ld2(const float* p) {
+        if constexpr (kCoherent) {
+            union {
+                unsigned long long u;
+                float2 f;
+            } c;
+            c.u = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_AGENT);
+            return c.f;
+        } else {
+            return *reinterpret_cast<const float2*>(p);
+        }
+    }
+};
+
 // Block-wide sum for blocks of up to 16 wavefronts; scratch is 16 floats of LDS.
 // Every thread gets the total.  Contains two block barriers.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

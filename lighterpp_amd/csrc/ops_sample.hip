@@ -32,28 +32,28 @@ __global__ __launch_bounds__(kSampleThreads) void penalty_kernel(float* logits, 
 
 __global__ __launch_bounds__(kSampleThreads) void scale_max_kernel(float* logits, int vocab, int chunk,
                                                                    float temperature) {
-    scale_max_chunk(logits, logits, vocab, chunk, blockIdx.x, temperature, 1.0f, nullptr, 0, scratch());
+    scale_max_chunk<false>(logits, logits, vocab, chunk, blockIdx.x, temperature, 1.0f, nullptr, 0, scratch());
 }
 
 __global__ __launch_bounds__(kSampleThreads) void argmax_final_kernel(int nchunks, int* result) {
-    const int a = argmax_over_chunks(nchunks, scratch());
+    const int a = argmax_over_chunks<false>(nchunks, scratch());
     if (threadIdx.x == 0) result[0] = a;
 }
 
 __global__ __launch_bounds__(kSampleThreads) void exp_sum_kernel(float* logits, int vocab, int chunk,
                                                                  int nchunks) {
-    exp_sum_chunk(logits, vocab, chunk, nchunks, blockIdx.x, scratch());
+    exp_sum_chunk<false>(logits, vocab, chunk, nchunks, blockIdx.x, scratch());
 }
 
 __global__ __launch_bounds__(kSampleThreads) void normalise_kernel(float* logits, int vocab, int chunk,
                                                                    int nchunks, int* result) {
-    normalise_chunk(logits, vocab, chunk, nchunks, blockIdx.x, scratch());
+    normalise_chunk<false>(logits, vocab, chunk, nchunks, blockIdx.x, scratch());
     if (blockIdx.x == 0 && threadIdx.x == 0) result[0] = vocab - 1;  // model.cpp:302 fallback
 }
 
 __global__ __launch_bounds__(kSampleThreads) void cdf_search_kernel(const float* probs, int vocab, int chunk,
                                                                     float r, int* result) {
-    cdf_search_chunk(probs, vocab, chunk, blockIdx.x, r, scratch(), result);
+    cdf_search_chunk<false>(probs, vocab, chunk, blockIdx.x, r, scratch(), result);
 }
 
 }  // namespace

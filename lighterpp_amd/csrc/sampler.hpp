@@ -6,9 +6,11 @@
 //   2. temperature 0: lowest index of the maximum;
 //   3. otherwise x / temperature, softmax, and the smallest index i with
 //      r < p_0 + ... + p_i, or vocab-1 when there is none.
-// The vocabulary is cut into chunks of `chunk` entries, one workgroup of
-// kSampleThreads threads per chunk; the per-chunk results that the next step
-// needs are kept in a SampleScratch the caller provides.
+// The vocabulary is cut into chunks of `chunk` entries, one workgroup per chunk;
+// the per-chunk results the next step needs are kept in a SampleScratch the
+// caller provides.  kCoh selects device-coherent accesses for everything another
+// workgroup wrote earlier in the SAME kernel (see dev::Mem); between separate
+// launches ordinary accesses do.
 #pragma once
 
 #include "lpp_device.hpp"
@@ -19,7 +21,6 @@ namespace smp {
 using namespace dev;
 
 constexpr int kSampleThreads = 256;
-constexpr int kSampleWaves = kSampleThreads / kWave;
 constexpr int kMaxChunks = 1024;
 
 struct SampleScratch {
@@ -29,7 +30,8 @@ struct SampleScratch {
     float* chunk_prob;  // [kMaxChunks]
 };
 
-// Entries per chunk so that at most kMaxChunks chunks cover the vocabulary.
+// Entries per chunk so that at most kMaxChunks chunks cover the vocabulary; a
+// multiple of 1024 so that any workgroup size up to 1024 divides it.
 __host__ __device__ inline int chunk_size_for(int vocab) {
     int per_thread = 4;
     while (static_cast<long>(per_thread) * kSampleThreads * kMaxChunks < vocab) per_thread *= 2;
@@ -46,6 +48,16 @@ __device__ __forceinline__ float penalise(float v, float penalty, int count) {
     return v;
 }
 
+// Occurrences of history[i] in the window if i is its first occurrence, else 0.
+__device__ __forceinline__ int owned_count(const int* __restrict__ history, int history_len, int i) {
+    const int tok = history[i];
+    for (int j = 0; j < i; ++j)
+        if (history[j] == tok) return 0;
+    int count = 1;
+    for (int j = i + 1; j < history_len; ++j) count += (history[j] == tok) ? 1 : 0;
+    return count;
+}
+
 // Step 0 (one workgroup): penalty over the whole window, in place.  The thread
 // holding a token's first occurrence replays all of that token's occurrences,
 // so duplicates never race.
@@ -54,23 +66,16 @@ __device__ __forceinline__ void penalty_all(float* logits, int vocab, float pena
     for (int i = threadIdx.x; i < history_len; i += blockDim.x) {
         const int tok = history[i];
         if (tok < 0 || tok >= vocab) continue;
-        bool first = true;
-        for (int j = 0; j < i; ++j)
-            if (history[j] == tok) {
-                first = false;
-                break;
-            }
-        if (!first) continue;
-        int count = 1;
-        for (int j = i + 1; j < history_len; ++j) count += (history[j] == tok) ? 1 : 0;
-        logits[tok] = penalise(logits[tok], penalty, count);
+        const int count = owned_count(history, history_len, i);
+        if (count > 0) logits[tok] = penalise(logits[tok], penalty, count);
     }
 }
 
 // Step 1 (chunk c): src -> dst with the optional penalty (tokens that fall into
 // this chunk only) and division by the temperature; records the chunk maximum
-// and its lowest index.  src may equal dst.  When history is null no penalty is
-// applied.
+// and its lowest index.  src may equal dst.  A null history applies no penalty.
+// dst[chunk c] is only ever touched again by the workgroup that owns chunk c.
+template <bool kCoh>
 __device__ __forceinline__ void scale_max_chunk(const float* src, float* dst, int vocab, int chunk,
                                                 int c, float temperature, float penalty,
                                                 const int* __restrict__ history, int history_len,
@@ -80,29 +85,21 @@ __device__ __forceinline__ void scale_max_chunk(const float* src, float* dst, in
     const int begin = c * chunk;
     const int end = min(begin + chunk, vocab);
     const int nthreads = static_cast<int>(blockDim.x);
-    if (history != nullptr && penalty > 1.0f && history_len > 0) {
-        for (int i = begin + threadIdx.x; i < end; i += nthreads) dst[i] = src[i];
+    const bool penalise_here = history != nullptr && penalty > 1.0f && history_len > 0;
+    if (penalise_here) {
+        for (int i = begin + threadIdx.x; i < end; i += nthreads) dst[i] = Mem<kCoh>::ld(src + i);
         __syncthreads();
         for (int i = threadIdx.x; i < history_len; i += nthreads) {
             const int tok = history[i];
             if (tok < begin || tok >= end) continue;
-            bool first = true;
-            for (int j = 0; j < i; ++j)
-                if (history[j] == tok) {
-                    first = false;
-                    break;
-                }
-            if (!first) continue;
-            int count = 1;
-            for (int j = i + 1; j < history_len; ++j) count += (history[j] == tok) ? 1 : 0;
-            dst[tok] = penalise(dst[tok], penalty, count);
+            const int count = owned_count(history, history_len, i);
+            if (count > 0) dst[tok] = penalise(dst[tok], penalty, count);
         }
         __syncthreads();
-        src = dst;
     }
     ArgMax best{-INFINITY, 0x7fffffff};
     for (int i = begin + threadIdx.x; i < end; i += nthreads) {
-        float v = src[i];
+        float v = penalise_here ? dst[i] : Mem<kCoh>::ld(src + i);
         if (temperature != 0.0f) v = v / temperature;
         dst[i] = v;
         best = argmax_better(best, ArgMax{v, i});
@@ -119,20 +116,21 @@ __device__ __forceinline__ void scale_max_chunk(const float* src, float* dst, in
     if (threadIdx.x == 0) {
         ArgMax m{sv[0], si[0]};
         for (int w = 1; w < nwaves; ++w) m = argmax_better(m, ArgMax{sv[w], si[w]});
-        sc.chunk_max[c] = m.v;
-        sc.chunk_arg[c] = m.i;
+        Mem<kCoh>::st(sc.chunk_max + c, m.v);
+        Mem<kCoh>::sti(sc.chunk_arg + c, m.i);
     }
 }
 
 // Temperature 0 (one workgroup): model.cpp:272-283, first maximum wins.
 // Returns the answer in every thread.
+template <bool kCoh>
 __device__ __forceinline__ int argmax_over_chunks(int nchunks, SampleScratch sc) {
     __shared__ float sv[16];
     __shared__ int si[16];
     __shared__ int answer;
     ArgMax best{-INFINITY, 0x7fffffff};
     for (int c = threadIdx.x; c < nchunks; c += blockDim.x)
-        best = argmax_better(best, ArgMax{sc.chunk_max[c], sc.chunk_arg[c]});
+        best = argmax_better(best, ArgMax{Mem<kCoh>::ld(sc.chunk_max + c), Mem<kCoh>::ldi(sc.chunk_arg + c)});
     best = wave_argmax(best);
     const int wave = static_cast<int>(threadIdx.x) / kWave;
     const int nwaves = (static_cast<int>(blockDim.x) + kWave - 1) / kWave;
@@ -154,22 +152,25 @@ __device__ __forceinline__ int argmax_over_chunks(int nchunks, SampleScratch sc)
 
 // Every workgroup derives the same global value from a chunk table in the same
 // order, so all of them agree to the bit.
+template <bool kCoh>
 __device__ __forceinline__ float table_max(const float* table, int n, float* scratch) {
     float v = -INFINITY;
-    for (int c = threadIdx.x; c < n; c += blockDim.x) v = fmaxf(v, table[c]);
+    for (int c = threadIdx.x; c < n; c += blockDim.x) v = fmaxf(v, Mem<kCoh>::ld(table + c));
     return block_max(v, scratch);
 }
+template <bool kCoh>
 __device__ __forceinline__ float table_sum(const float* table, int n, float* scratch) {
     float v = 0.0f;
-    for (int c = threadIdx.x; c < n; c += blockDim.x) v += table[c];
+    for (int c = threadIdx.x; c < n; c += blockDim.x) v += Mem<kCoh>::ld(table + c);
     return block_sum(v, scratch);
 }
 
 // Step 2 (chunk c): e = expf(x - max) in place; per-chunk sum.
+template <bool kCoh>
 __device__ __forceinline__ void exp_sum_chunk(float* vals, int vocab, int chunk, int nchunks, int c,
                                               SampleScratch sc) {
     __shared__ float scratch[16];
-    const float top = table_max(sc.chunk_max, nchunks, scratch);
+    const float top = table_max<kCoh>(sc.chunk_max, nchunks, scratch);
     const int begin = c * chunk;
     const int end = min(begin + chunk, vocab);
     float total = 0.0f;
@@ -179,15 +180,16 @@ __device__ __forceinline__ void exp_sum_chunk(float* vals, int vocab, int chunk,
         total += e;
     }
     total = block_sum(total, scratch);
-    if (threadIdx.x == 0) sc.chunk_sum[c] = total;
+    if (threadIdx.x == 0) Mem<kCoh>::st(sc.chunk_sum + c, total);
 }
 
 // Step 3 (chunk c): p = e / sum in place (the CPU leaves probabilities in the
 // buffer too); per-chunk probability mass.
+template <bool kCoh>
 __device__ __forceinline__ void normalise_chunk(float* vals, int vocab, int chunk, int nchunks, int c,
                                                 SampleScratch sc) {
     __shared__ float scratch[16];
-    const float total = table_sum(sc.chunk_sum, nchunks, scratch);
+    const float total = table_sum<kCoh>(sc.chunk_sum, nchunks, scratch);
     const int begin = c * chunk;
     const int end = min(begin + chunk, vocab);
     float mass = 0.0f;
@@ -197,7 +199,7 @@ __device__ __forceinline__ void normalise_chunk(float* vals, int vocab, int chun
         mass += p;
     }
     mass = block_sum(mass, scratch);
-    if (threadIdx.x == 0) sc.chunk_prob[c] = mass;
+    if (threadIdx.x == 0) Mem<kCoh>::st(sc.chunk_prob + c, mass);
 }
 
 // Step 4 (chunk c): cdf_i = (mass of earlier chunks) + (running sum inside the
@@ -205,12 +207,13 @@ __device__ __forceinline__ void normalise_chunk(float* vals, int vocab, int chun
 // (model.cpp:296-301).  *result must hold vocab-1 (the :302 fallback) before any
 // chunk runs this step.  Each thread owns chunk/blockDim consecutive entries and
 // adds them in index order.
-__device__ __forceinline__ void cdf_search_chunk(const float* __restrict__ probs, int vocab, int chunk,
-                                                 int c, float r, SampleScratch sc, int* result) {
+template <bool kCoh>
+__device__ __forceinline__ void cdf_search_chunk(const float* probs, int vocab, int chunk, int c, float r,
+                                                 SampleScratch sc, int* result) {
     __shared__ float scratch[16];
     __shared__ float wave_tot[16];
     float before = 0.0f;
-    for (int k = threadIdx.x; k < c; k += blockDim.x) before += sc.chunk_prob[k];
+    for (int k = threadIdx.x; k < c; k += blockDim.x) before += Mem<kCoh>::ld(sc.chunk_prob + k);
     before = block_sum(before, scratch);
 
     const int per_thread = chunk / static_cast<int>(blockDim.x);
@@ -233,7 +236,21 @@ __device__ __forceinline__ void cdf_search_chunk(const float* __restrict__ probs
         run += probs[i];
         if (found == 0x7fffffff && r < offset + run) found = i;
     }
-    if (found != 0x7fffffff) atomicMin(result, found);
+    // One atomic per workgroup: about half of all threads hold a candidate (every
+    // entry past the crossing qualifies), and that many device-scope atomics on
+    // one word would serialise for hundreds of microseconds.
+    __shared__ int wave_found[16];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) found = min(found, __shfl_xor(found, off));
+    __syncthreads();
+    if (lane_id() == 0) wave_found[wave] = found;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int nwaves = (static_cast<int>(blockDim.x) + kWave - 1) / kWave;
+        int best = wave_found[0];
+        for (int w = 1; w < nwaves; ++w) best = min(best, wave_found[w]);
+        if (best != 0x7fffffff) atomicMin(result, best);
+    }
 }
 
 }  // namespace smp
