@@ -124,6 +124,13 @@ __device__ __forceinline__ void stage_rmsnorm(float* xs, const float* src, const
 // Pipelined row-tile GEMV
 // ---------------------------------------------------------------------------
 
+// Register image of one step of a tile: kUnroll chunks of kRows rows.  Loads are
+// unconditional (no branch around any of them): a lane whose columns lie beyond
+// d reads column 0 instead and its activations are zeroed in fma(); row pointers
+// must always be readable (callers clamp rows past the end to a valid row and
+// discard the result).  Branch-free requests let the compiler count outstanding
+// loads exactly, so the multiply of one step only waits for its own data while
+// the next step's requests stay in flight.
 template <bool kF16, int kRows, int kUnroll>
 struct Tile {
     static constexpr int kPer = WTraits<kF16>::kPerLoad;
@@ -135,33 +142,70 @@ struct Tile {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int col = (cg * kUnroll + u) * kChunk + lane * kPer;
-            const bool live = col < d;
+            const int safe_col = (col < d) ? col : 0;
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) {
-                if (live && rows[r] != nullptr)
-                    w[u][r] = load16_stream(rows[r] + static_cast<size_t>(col) * WTraits<kF16>::kBytes);
-                else
-                    w[u][r] = uintx4{0u, 0u, 0u, 0u};
+            for (int r = 0; r < kRows; ++r)
+                w[u][r] = load16_stream(rows[r] + static_cast<size_t>(safe_col) * WTraits<kF16>::kBytes);
+        }
+    }
+
+    // Multiply this step and hand every register back to the memory system the
+    // moment it has been used: the 16 bytes just consumed are replaced by the
+    // same position of step (next_rows, next_cg).  One request leaves for each one
+    // retired, so the number in flight stays constant through the whole phase.
+    __device__ __forceinline__ void fma_refill(const float* xs, int cg, int d, float (&acc)[kRows],
+                                               const char* const (&next_rows)[kRows], int next_cg) {
+        const int lane = lane_id();
+        const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int col = (cg * kUnroll + u) * kChunk + lane * kPer;
+            const bool live = col < d;
+            const int safe_col = live ? col : 0;
+            const int ncol = (next_cg * kUnroll + u) * kChunk + lane * kPer;
+            const size_t noff = static_cast<size_t>(ncol < d ? ncol : 0) * WTraits<kF16>::kBytes;
+            if constexpr (kF16) {
+                floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                floatx4 xb = *reinterpret_cast<const floatx4*>(xs + safe_col + 4);
+                xa = live ? xa : zero;
+                xb = live ? xb : zero;
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    acc[r] = dot8(w[u][r], xa, xb, acc[r]);
+                    w[u][r] = load16_stream(next_rows[r] + noff);
+                }
+            } else {
+                floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                xa = live ? xa : zero;
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    acc[r] = dot4(w[u][r], xa, acc[r]);
+                    w[u][r] = load16_stream(next_rows[r] + noff);
+                }
             }
         }
     }
 
     __device__ __forceinline__ void fma(const float* xs, int cg, int d, float (&acc)[kRows]) const {
         const int lane = lane_id();
+        const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int col = (cg * kUnroll + u) * kChunk + lane * kPer;
-            if (col < d) {
-                if constexpr (kF16) {
-                    const floatx4 xa = *reinterpret_cast<const floatx4*>(xs + col);
-                    const floatx4 xb = *reinterpret_cast<const floatx4*>(xs + col + 4);
+            const bool live = col < d;
+            const int safe_col = live ? col : 0;
+            if constexpr (kF16) {
+                floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                floatx4 xb = *reinterpret_cast<const floatx4*>(xs + safe_col + 4);
+                xa = live ? xa : zero;
+                xb = live ? xb : zero;
 #pragma unroll
-                    for (int r = 0; r < kRows; ++r) acc[r] = dot8(w[u][r], xa, xb, acc[r]);
-                } else {
-                    const floatx4 xa = *reinterpret_cast<const floatx4*>(xs + col);
+                for (int r = 0; r < kRows; ++r) acc[r] = dot8(w[u][r], xa, xb, acc[r]);
+            } else {
+                floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                xa = live ? xa : zero;
 #pragma unroll
-                    for (int r = 0; r < kRows; ++r) acc[r] = dot4(w[u][r], xa, acc[r]);
-                }
+                for (int r = 0; r < kRows; ++r) acc[r] = dot4(w[u][r], xa, acc[r]);
             }
         }
     }
@@ -178,77 +222,132 @@ struct Cursor {
 };
 
 // One wavefront walks tiles wave_g, wave_g + waves_total, ...; a tile is kRows
-// rows given by row_ptr(tile, r) (null = no such row) and is consumed in steps
+// rows given by row_ptr(tile, r) (always a readable row) and is consumed in steps
 // of kUnroll chunks.  Two steps are always in flight: both are requested before
 // pre() runs, and each register set is refilled with the step after next as soon
-// as it has been multiplied.  pre() runs once, after those first requests and
-// before anything reads xs; every wavefront of the workgroup calls it, with or
-// without work.  epi(tile, sums) receives wave-uniform dot products.
-template <bool kF16, int kRows, int kUnroll, class RowFn, class EpiFn, class PreFn>
+// as it has been multiplied.  The steady-state loop contains no conditional
+// load (a conditionally refilled register set would make the compiler copy it
+// and wait for every outstanding load) and no global store (on this target
+// stores share the loads' wait counter, and a pending store makes every wait a
+// full drain): the dot products of up to 64 (tile, row) pairs are parked one
+// per lane in a single register and written out when the wavefront's work is
+// done, by emit(tile, r, value, neighbour), where neighbour is the value of row
+// r^1 of the same tile.  pre() runs once, after the first requests and before
+// anything reads xs; every wavefront of the workgroup calls it, with or without
+// work.
+template <bool kF16, int kRows, int kUnroll, class RowFn, class EmitFn, class PreFn>
 __device__ __forceinline__ void gemv_phase(int ntiles, int d, const float* xs, int wave_g, int waves_total,
-                                           RowFn row_ptr, EpiFn epi, PreFn pre) {
+                                           RowFn row_ptr, EmitFn emit, PreFn pre) {
     using T = Tile<kF16, kRows, kUnroll>;
     using C = Cursor<kRows>;
+    static_assert(kWave % kRows == 0, "results are parked kRows per tile");
+    constexpr int kParkRegs = 2;
+    constexpr int kTilesPerRound = kParkRegs * kWave / kRows;  // results one round can park
+    const int lane = lane_id();
     const int ncg = (d + T::kChunk * kUnroll - 1) / (T::kChunk * kUnroll);
+    const int my_tiles = (wave_g < ntiles) ? (ntiles - wave_g + waves_total - 1) / waves_total : 0;
 
-    auto start = [&](C& c) {
-        c.tile = wave_g;
-        c.cg = 0;
-        c.have = c.tile < ntiles && ncg > 0;
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) c.rows[r] = c.have ? row_ptr(c.tile, r) : nullptr;
-    };
-    // c <- the step after c
+    // c <- the step after c (row pointers change only at tile boundaries)
     auto advance = [&](C& c) {
-        if (!c.have) return;
         if (c.cg + 1 < ncg) {
             c.cg += 1;
             return;
         }
         c.cg = 0;
         c.tile += waves_total;
-        c.have = c.tile < ntiles;
-        if (c.have) {
+        const int t = c.tile < ntiles ? c.tile : wave_g;  // past the end: any valid tile, never loaded
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) c.rows[r] = row_ptr(c.tile, r);
-        }
+        for (int r = 0; r < kRows; ++r) c.rows[r] = row_ptr(t, r);
     };
 
-    T ta, tb;
-    C ca, cb;
-    start(ca);
-    cb = ca;
-    advance(cb);
-    if (ca.have) ta.load(ca.rows, ca.cg, d);
-    if (cb.have) tb.load(cb.rows, cb.cg, d);
-    pre();
-    float acc[kRows];
+    C next;  // next step to request
+    next.tile = wave_g;
+    next.cg = 0;
+    next.have = true;
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < kRows; ++r) next.rows[r] = row_ptr(wave_g < ntiles ? wave_g : 0, r);
 
-#define LPP_GEMV_STEP(TCUR, CCUR)                                                 \
-    {                                                                             \
-        TCUR.fma(xs, CCUR.cg, d, acc);                                            \
-        const int done_tile = CCUR.tile;                                          \
-        const bool tile_ends = (CCUR.cg + 1 == ncg);                              \
-        advance(CCUR);                                                            \
-        advance(CCUR);                                                            \
-        if (CCUR.have) TCUR.load(CCUR.rows, CCUR.cg, d);                          \
-        if (tile_ends) {                                                          \
-            float sums[kRows];                                                    \
-            _Pragma("unroll") for (int r = 0; r < kRows; ++r) {                   \
-                sums[r] = wave_sum(acc[r]);                                       \
-                acc[r] = 0.0f;                                                    \
-            }                                                                     \
-            epi(done_tile, sums);                                                 \
-        }                                                                         \
-    }
-    while (ca.have) {
-        LPP_GEMV_STEP(ta, ca)
-        if (!cb.have) break;
-        LPP_GEMV_STEP(tb, cb)
-    }
-#undef LPP_GEMV_STEP
+    // A round is at most kTilesPerRound tiles: its dot products are parked in
+    // registers and written out after its last multiply, outside the streaming
+    // loop.  One round covers a whole phase for every shape met in practice.
+    bool first_round = true;
+    int tiles_done = 0;
+    do {
+        const int round_tiles = min(my_tiles - tiles_done, kTilesPerRound);
+        const int n_steps = round_tiles * ncg;
+        int use_cg = 0;  // chunk group of the next step to multiply
+        int parked = 0;  // tiles of this round already reduced
+        float park[kParkRegs];  // lane (slot % 64) of register (slot / 64) holds slot = k * kRows + r
+#pragma unroll
+        for (int p = 0; p < kParkRegs; ++p) park[p] = 0.0f;
+
+        T ta, tb;
+        if (n_steps > 0) {
+            ta.load(next.rows, next.cg, d);
+            advance(next);
+        }
+        if (n_steps > 1) {
+            tb.load(next.rows, next.cg, d);
+            advance(next);
+        }
+        if (first_round) pre();
+        first_round = false;
+        float acc[kRows];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) acc[r] = 0.0f;
+
+        auto park_if_tile_done = [&]() {
+            if (use_cg + 1 == ncg) {
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const float sum = wave_sum(acc[r]);
+                    const int slot = parked * kRows + r;
+#pragma unroll
+                    for (int p = 0; p < kParkRegs; ++p) park[p] = (lane + p * kWave == slot) ? sum : park[p];
+                    acc[r] = 0.0f;
+                }
+                use_cg = 0;
+                parked += 1;
+            } else {
+                use_cg += 1;
+            }
+        };
+        auto consume = [&](const T& t) {
+            t.fma(xs, use_cg, d, acc);
+            park_if_tile_done();
+        };
+
+        int i = 0;
+        for (; i + 3 < n_steps; i += 2) {
+            ta.fma_refill(xs, use_cg, d, acc, next.rows, next.cg);
+            advance(next);
+            park_if_tile_done();
+            tb.fma_refill(xs, use_cg, d, acc, next.rows, next.cg);
+            advance(next);
+            park_if_tile_done();
+        }
+        const int left = n_steps - i;  // 0..3 steps: ta holds step i, tb step i+1
+        if (left >= 1) consume(ta);
+        if (left == 3) {
+            ta.load(next.rows, next.cg, d);
+            advance(next);
+        }
+        if (left >= 2) consume(tb);
+        if (left == 3) consume(ta);
+
+        // write the round's results: one lane per (tile, row)
+        const int first_tile = wave_g + tiles_done * waves_total;
+#pragma unroll
+        for (int p = 0; p < kParkRegs; ++p) {
+            const float neighbour = dpp_move<kDppXor1>(park[p]);
+            const int slot = lane + p * kWave;
+            if (slot < parked * kRows) {
+                const int k = slot / kRows;
+                emit(first_tile + k * waves_total, slot - k * kRows, park[p], neighbour);
+            }
+        }
+        tiles_done += round_tiles;
+    } while (tiles_done < my_tiles);
 }
 
 __device__ __forceinline__ const char* row_at(const char* base, size_t layer_rows, int layer, int row, int d,
@@ -260,16 +359,6 @@ __device__ __forceinline__ const char* row_at(const char* base, size_t layer_row
 // later layers read x.
 __device__ __forceinline__ const float* layer_input(const DecodeArgs& a, int layer) {
     return layer == 0 ? a.emb + static_cast<size_t>(a.step->token) * a.dim : a.x;
-}
-
-// Pick element `lane` of a small wave-uniform array without dynamic indexing.
-template <int kN>
-__device__ __forceinline__ float pick(const float (&v)[kN], int lane) {
-    float out = v[0];
-#pragma unroll
-    for (int r = 1; r < kN; ++r)
-        if (lane == r) out = v[r];
-    return out;
 }
 
 // ---------------------------------------------------------------------------
@@ -290,49 +379,40 @@ __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg
         const int g = tile * kRows + r;
         if (g < dim) return row_at(a.wq, dim, layer, g, dim, wbytes);
         if (g < dim + kv_dim) return row_at(a.wk, kv_dim, layer, g - dim, dim, wbytes);
-        if (g < total_rows) return row_at(a.wv, kv_dim, layer, g - dim - kv_dim, dim, wbytes);
-        return nullptr;
+        const int gv = (g < total_rows ? g : total_rows - 1) - dim - kv_dim;  // past the end: a valid row, result unused
+        return row_at(a.wv, kv_dim, layer, gv, dim, wbytes);
     };
     auto prologue = [&]() {
         pre();
         stage_rmsnorm<kCoh>(xs, layer_input(a, layer), a.rms_att + static_cast<size_t>(layer) * dim, dim);
     };
-    auto epilogue = [&](int tile, float (&sums)[kRows]) {
-        if (lane_id() != 0) return;
-        const int pos = a.step->pos;
-        const int hs = a.head_size;
-        const float2* cs_row = a.rope + static_cast<size_t>(pos) * (hs / 2);
-#pragma unroll
-        for (int r = 0; r < kRows; r += 2) {
-            const int g = tile * kRows + r;
-            if (g >= total_rows) break;
-            float e0 = sums[r], e1 = sums[r + 1];
-            if (g < dim + kv_dim) {
-                // ops.cpp:36-52 on the pair (i, i+1); i is the index inside q or k.
-                const int i = (g < dim) ? g : g - dim;
-                const float2 cs = cs_row[(i % hs) >> 1];
-                const float r0 = e0 * cs.x - e1 * cs.y;
-                const float r1 = e0 * cs.y + e1 * cs.x;
-                e0 = r0;
-                e1 = r1;
-            }
-            if (g < dim) {
-                Mem<kCoh>::st(a.q + g, e0);
-                Mem<kCoh>::st(a.q + g + 1, e1);
-            } else {
-                // model.cpp:171-176 / scatter_kv.cu:15-18.
-                const bool is_k = g < dim + kv_dim;
-                const int i = is_k ? g - dim : g - dim - kv_dim;
-                const int head = i / hs, within = i - head * hs;
-                const size_t dst = static_cast<size_t>(layer) * kv_dim * a.seq_len +
-                                   static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(pos) * hs + within;
-                float* plain = is_k ? a.k : a.v;
-                uint16_t* cache = is_k ? a.key_cache : a.value_cache;
-                Mem<kCoh>::st(plain + i, e0);
-                Mem<kCoh>::st(plain + i + 1, e1);
-                cache[dst] = f32_to_f16_bits(e0);
-                cache[dst + 1] = f32_to_f16_bits(e1);
-            }
+    const int pos = a.step->pos;
+    const int hs = a.head_size;
+    const float2* cs_row = a.rope + static_cast<size_t>(pos) * (hs / 2);
+    // One lane per output row; rows (2j, 2j+1) of a tile are a RoPE pair, the odd
+    // one being this lane's neighbour.
+    auto epilogue = [&](int tile, int r, float mine, float neighbour) {
+        const int g = tile * kRows + r;
+        if (g >= total_rows) return;
+        float out = mine;
+        if (g < dim + kv_dim) {
+            // ops.cpp:36-52 on the pair (i, i+1); i is the even index inside q or k.
+            const int gi = (g < dim) ? g : g - dim;
+            const float2 cs = cs_row[((gi & ~1) % hs) >> 1];
+            out = (gi & 1) ? neighbour * cs.y + mine * cs.x   // q[i+1] = q0*sin + q1*cos
+                           : mine * cs.x - neighbour * cs.y;  // q[i]   = q0*cos - q1*sin
+        }
+        if (g < dim) {
+            Mem<kCoh>::st(a.q + g, out);
+        } else {
+            // model.cpp:171-176 / scatter_kv.cu:15-18.
+            const bool is_k = g < dim + kv_dim;
+            const int i = is_k ? g - dim : g - dim - kv_dim;
+            const int head = i / hs, within = i - head * hs;
+            const size_t dst = static_cast<size_t>(layer) * kv_dim * a.seq_len +
+                               static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(pos) * hs + within;
+            Mem<kCoh>::st((is_k ? a.k : a.v) + i, out);
+            (is_k ? a.key_cache : a.value_cache)[dst] = f32_to_f16_bits(out);
         }
     };
     gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
@@ -341,7 +421,7 @@ __device__ __forceinline__ void phase_qkv(const DecodeArgs& a, int layer, int wg
 // ---------------------------------------------------------------------------
 // Phase: out = W . xs + residual   (O projection and down projection)
 // ---------------------------------------------------------------------------
-template <bool kF16, int kRows, bool kCoh, class PreFn>
+template <bool kF16, int kRows, bool kCoh, int kUnroll = 4, class PreFn>
 __device__ __forceinline__ void phase_proj_residual(const char* w_layer, int n, int d, const float* src,
                                                     const float* residual, float* out, int wg, int nwg,
                                                     float* xs, PreFn pre) {
@@ -351,21 +431,18 @@ __device__ __forceinline__ void phase_proj_residual(const char* w_layer, int n, 
     const int ntiles = (n + kRows - 1) / kRows;
     auto row_ptr = [&](int tile, int r) -> const char* {
         const int g = tile * kRows + r;
-        return g < n ? w_layer + static_cast<size_t>(g) * d * wbytes : nullptr;
+        return w_layer + static_cast<size_t>(g < n ? g : n - 1) * d * wbytes;  // past the end: a valid row, result unused
     };
     auto prologue = [&]() {
         pre();
         stage_plain<kCoh>(xs, src, d);
     };
-    auto epilogue = [&](int tile, float (&sums)[kRows]) {
-        const int lane = lane_id();
-        if (lane >= kRows) return;
-        const int g = tile * kRows + lane;
+    auto epilogue = [&](int tile, int r, float mine, float) {
+        const int g = tile * kRows + r;
         if (g >= n) return;
-        const float v = pick<kRows>(sums, lane);
-        Mem<kCoh>::st(out + g, Mem<kCoh>::ld(residual + g) + v);  // model.cpp:232,239: x[i] += xb2[i]
+        Mem<kCoh>::st(out + g, Mem<kCoh>::ld(residual + g) + mine);  // model.cpp:232,239: x[i] += xb2[i]
     };
-    gemv_phase<kF16, kRows, 4>(ntiles, d, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
+    gemv_phase<kF16, kRows, kUnroll>(ntiles, d, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
 }
 
 // ---------------------------------------------------------------------------
@@ -380,27 +457,20 @@ __device__ __forceinline__ void phase_gateup(const DecodeArgs& a, int layer, int
     const int wave_g = wg * waves_per_wg + wave_index();
     const int hidden = a.hidden, dim = a.dim;
     const int ntiles = (hidden + kPairRows - 1) / kPairRows;
+    // Row 2j of a tile is gate row j, row 2j+1 the matching up row, so the two
+    // halves of one output sit in neighbouring lanes.
     auto row_ptr = [&](int tile, int r) -> const char* {
-        const int g = tile * kPairRows + (r % kPairRows);
-        if (g >= hidden) return nullptr;
-        return row_at(r < kPairRows ? a.w1 : a.w3, hidden, layer, g, dim, wbytes);
+        const int g = tile * kPairRows + (r >> 1);
+        return row_at((r & 1) ? a.w3 : a.w1, hidden, layer, g < hidden ? g : hidden - 1, dim, wbytes);
     };
     auto prologue = [&]() {
         pre();
         stage_rmsnorm<kCoh>(xs, a.x, a.rms_ffn + static_cast<size_t>(layer) * dim, dim);
     };
-    auto epilogue = [&](int tile, float (&sums)[kRows]) {
-        const int lane = lane_id();
-        if (lane >= kPairRows) return;
-        const int g = tile * kPairRows + lane;
+    auto epilogue = [&](int tile, int r, float gate, float up) {
+        if (r & 1) return;
+        const int g = tile * kPairRows + (r >> 1);
         if (g >= hidden) return;
-        float gate = sums[0], up = sums[kPairRows];
-#pragma unroll
-        for (int r = 1; r < kPairRows; ++r)
-            if (lane == r) {
-                gate = sums[r];
-                up = sums[kPairRows + r];
-            }
         // ops.cpp:80-85
         const float sigma = 1.0f / (1.0f + expf(-gate));
         Mem<kCoh>::st(a.hb + g, (gate * sigma) * up);
@@ -420,18 +490,15 @@ __device__ __forceinline__ void phase_lmhead(const DecodeArgs& a, int wg, int nw
     const int ntiles = (vocab + kRows - 1) / kRows;
     auto row_ptr = [&](int tile, int r) -> const char* {
         const int g = tile * kRows + r;
-        return g < vocab ? a.wcls + static_cast<size_t>(g) * dim * wbytes : nullptr;
+        return a.wcls + static_cast<size_t>(g < vocab ? g : vocab - 1) * dim * wbytes;
     };
     auto prologue = [&]() {
         pre();
         stage_rmsnorm<kCoh>(xs, a.x, a.rms_final, dim);
     };
-    auto epilogue = [&](int tile, float (&sums)[kRows]) {
-        const int lane = lane_id();
-        if (lane >= kRows) return;
-        const int g = tile * kRows + lane;
-        if (g >= vocab) return;
-        Mem<kCoh>::st(a.logits + g, pick<kRows>(sums, lane));
+    auto epilogue = [&](int tile, int r, float mine, float) {
+        const int g = tile * kRows + r;
+        if (g < vocab) Mem<kCoh>::st(a.logits + g, mine);
     };
     gemv_phase<kF16, kRows, 4>(ntiles, dim, xs, wave_g, nwg * waves_per_wg, row_ptr, epilogue, prologue);
 }
@@ -502,7 +569,7 @@ __device__ __forceinline__ uintx4 cache_row8(const uint16_t* cache_row, const fl
 // unnormalised output) goes to att_partial and the last split to arrive for
 // this KV head combines all of them.
 template <int kGroup, bool kCoh>
-__device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int split, int nsplits, int npos,
+__device__ __forceinline__ void attention_item(const DecodeArgs& a, int layer, int kvh, int split, int nsplits, int npos,
                                float* lds) {
     const int hs = a.head_size, gqa = a.gqa;
     const int hs_pad = kGroup * 8;
@@ -547,9 +614,10 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
     __syncthreads();
 
     // A sub-block is `per_group` consecutive rounds of ngroups positions.  Every
-    // lane requests all its K rows and all its V rows of the sub-block before the
-    // first multiply (up to 16 independent 16-byte loads in flight), so a
-    // sub-block costs about one memory round trip instead of one per position.
+    // lane requests all its K rows of the sub-block before the first multiply, and
+    // all its V rows before the softmax (8 independent 16-byte loads in flight
+    // each time), so a sub-block costs about two memory round trips instead of
+    // two per position.
     constexpr int kMaxPerGroup = 8;
     int per_group = kAttBlock / ngroups;
     if (per_group > kMaxPerGroup) per_group = kMaxPerGroup;
@@ -558,33 +626,37 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
     const bool lane_live = sub * 8 < hs;
     for (int b0 = t_begin; b0 < t_end; b0 += sub_block) {
         const int b1 = min(t_end, b0 + sub_block);
-        uintx4 kreg[kMaxPerGroup], vreg[kMaxPerGroup];
+        uintx4 rows8[kMaxPerGroup];
 #pragma unroll
         for (int j = 0; j < kMaxPerGroup; ++j) {
             const int t = b0 + grp + j * ngroups;
-            kreg[j] = uintx4{0u, 0u, 0u, 0u};
-            vreg[j] = uintx4{0u, 0u, 0u, 0u};
-            if (j < per_group && t < b1 && lane_live) {
-                kreg[j] = cache_row8<kCoh>(kbase + static_cast<size_t>(t) * hs, k_fresh, t == current, sub * 8);
-                vreg[j] = cache_row8<kCoh>(vbase + static_cast<size_t>(t) * hs, v_fresh, t == current, sub * 8);
-            }
+            rows8[j] = uintx4{0u, 0u, 0u, 0u};
+            if (j < per_group && t < b1 && lane_live)
+                rows8[j] = cache_row8<kCoh>(kbase + static_cast<size_t>(t) * hs, k_fresh, t == current, sub * 8);
         }
-        // scores of this sub-block
+        // scores of this sub-block (query head outermost: only one head's q slice
+        // is held in registers at a time)
 #pragma unroll
-        for (int j = 0; j < kMaxPerGroup; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            if (j < per_group && t < b1) {
+        for (int qh = 0; qh < kMaxGqa; ++qh) {
+            if (qh < gqa) {
+                const float* qv = qs + qh * hs_pad + sub * 8;
+                const floatx4 xa = *reinterpret_cast<const floatx4*>(qv);
+                const floatx4 xb = *reinterpret_cast<const floatx4*>(qv + 4);
 #pragma unroll
-                for (int qh = 0; qh < kMaxGqa; ++qh) {
-                    if (qh < gqa) {
-                        const float* qv = qs + qh * hs_pad + sub * 8;
-                        const floatx4 xa = *reinterpret_cast<const floatx4*>(qv);
-                        const floatx4 xb = *reinterpret_cast<const floatx4*>(qv + 4);
-                        const float s = group_sum<kGroup>(dot8(kreg[j], xa, xb, 0.0f));
-                        if (sub == 0) sc[qh * kAttBlock + (t - b0)] = s * scale;
-                    }
+                for (int j = 0; j < kMaxPerGroup; ++j) {
+                    const int t = b0 + grp + j * ngroups;
+                    const float s = group_sum<kGroup>(dot8(rows8[j], xa, xb, 0.0f));
+                    if (j < per_group && t < b1 && sub == 0) sc[qh * kAttBlock + (t - b0)] = s * scale;
                 }
             }
+        }
+        // the V rows of the same positions travel while the softmax is formed
+#pragma unroll
+        for (int j = 0; j < kMaxPerGroup; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            rows8[j] = uintx4{0u, 0u, 0u, 0u};
+            if (j < per_group && t < b1 && lane_live)
+                rows8[j] = cache_row8<kCoh>(vbase + static_cast<size_t>(t) * hs, v_fresh, t == current, sub * 8);
         }
         __syncthreads();
         // per head: new running max, probabilities, running sum, correction
@@ -624,7 +696,7 @@ __device__ void attention_item(const DecodeArgs& a, int layer, int kvh, int spli
         for (int j = 0; j < kMaxPerGroup; ++j) {
             const int t = b0 + grp + j * ngroups;
             if (j < per_group && t < b1 && lane_live) {
-                const half8_t vv = as_half8(vreg[j]);
+                const half8_t vv = as_half8(rows8[j]);
 #pragma unroll
                 for (int qh = 0; qh < kMaxGqa; ++qh) {
                     if (qh < gqa) {

@@ -15,6 +15,7 @@
 // per token.
 #include <chrono>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(kThreads) void k_down(DecodeArgs a, int layer) {
     extern __shared__ __align__(16) float lds[];
     const int wbytes = kF16 ? 2 : 4;
     const char* w = a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes;
-    phase_proj_residual<kF16, 1, false>(w, a.dim, a.hidden, a.hb, a.x, a.x, blockIdx.x, gridDim.x, lds, NoWait{});
+    phase_proj_residual<kF16, 1, false, 8>(w, a.dim, a.hidden, a.hb, a.x, a.x, blockIdx.x, gridDim.x, lds, NoWait{});
 }
 
 template <bool kF16>
@@ -173,13 +174,13 @@ __global__ __launch_bounds__(kPersistThreads) void k_decode_token(DecodeArgs a, 
         phase_proj_residual<kF16, 2, true>(a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes, a.dim, a.dim, a.xb,
                                      layer_input(a, layer), a.x, wg, nwg, lds, wait);
         gs.arrive();
-        phase_gateup<kF16, 2, true>(a, layer, wg, nwg, lds, wait);
+        phase_gateup<kF16, 1, true>(a, layer, wg, nwg, lds, wait);
         gs.arrive();
-        phase_proj_residual<kF16, 1, true>(a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden,
+        phase_proj_residual<kF16, 1, true, 8>(a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden,
                                      a.hb, a.x, a.x, wg, nwg, lds, wait);
         gs.arrive();
     }
-    phase_lmhead<kF16, 4, true>(a, wg, nwg, lds, wait);
+    phase_lmhead<kF16, 2, true>(a, wg, nwg, lds, wait);
     gs.arrive();
 
     const int chunk = smp::chunk_size_for(a.vocab);
@@ -259,7 +260,12 @@ DecodeArgs make_args(const lpp_model* m, bool with_arrays) {
 
 int blocks_for_tiles(int ntiles) {
     int blocks = (ntiles + kWavesPerWg - 1) / kWavesPerWg;
-    const int cap = compute_units() * 8;
+    static const int per_cu = [] {
+        const char* e = std::getenv("LPP_BLOCKS_PER_CU");  // tuning aid
+        const int v = e ? std::atoi(e) : 0;
+        return v > 0 ? v : 8;
+    }();
+    const int cap = compute_units() * per_cu;
     if (blocks > cap) blocks = cap;
     return blocks < 1 ? 1 : blocks;
 }
