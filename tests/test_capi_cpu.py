@@ -41,6 +41,37 @@ def test_compat_header_covers_the_twelve_wrappers():
     assert "MAX_SHARED_FLOATS" in text and "checkCuda" in text
 
 
+def test_compat_header_compiles_and_links_as_cxx(tmp_path):
+    """A translation unit written against the reference's kernels.cuh surface must
+    compile with plain g++ against the compat header and link with the library."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("g++ not available")
+    src = tmp_path / "caller.cpp"
+    src.write_text(
+        "enum WeightPrecision : int { WEIGHT_FP32 = 0, WEIGHT_FP16 = 1, WEIGHT_INT4 = 2 };\n"
+        '#include "lpp_kernels_compat.h"\n'
+        "int main() {\n"
+        "  float* f = nullptr; __half* h = nullptr; int* i = nullptr;\n"
+        "  if (MAX_SHARED_FLOATS < 14336) return 1;\n"
+        "  if (false) {\n"
+        "    cuda_convert_f32_to_f16(h, f, 0); cuda_gemv(f, f, h, h, 0, 0, WEIGHT_FP16); cuda_rmsnorm(f, f, f, 0);\n"
+        "    cuda_rope(f, f, 0, 0, 0, 0, 1.f); cuda_swiglu(f, f, f, 0); cuda_softmax_multihead(f, f, 0, 0, 0);\n"
+        "    cuda_scale_multihead(f, 1.f, 0, 0, 0); cuda_aggregation_multihead(f, h, f, 0, 0, 0, 0, 0);\n"
+        "    cuda_residual_add(f, f, f, 0); cuda_scatter_kv(h, h, f, f, 0, 0, 0, 0, 0);\n"
+        "    cuda_multihead_gemv(f, f, h, 0, 0, 0, 0, 0, 0); cuda_sample(f, 0, 0.f, 0.f, 0.f, i, 0, i, nullptr);\n"
+        "  }\n"
+        "  cuda_gemv(nullptr, nullptr, nullptr, nullptr, 0, 0, WEIGHT_FP16);  // n == 0: accepted, no launch\n"
+        "  return 0;\n"
+        "}\n")
+    exe = tmp_path / "caller"
+    libdir = ROOT / "lighterpp_amd"
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", f"-I{ROOT / 'include'}", str(src),
+                    f"-L{libdir}", "-llpp_hip", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True)
+    assert subprocess.run([str(exe)]).returncode == 0
+
+
 def test_version_and_error_string():
     lib = capi.load()
     assert b"gfx950" in lib.lpp_version()
