@@ -862,4 +862,10 @@ __device__ __forceinline__ void finish_token(const DecodeArgs& a, int token, uns
 }
 
 }  // namespace ph
+
+// Persistent one-kernel-per-token schedule, implemented in dataflow_decode.hip.
+size_t dataflow_tagged_bytes(const lpp_model* m);
+lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s);
+unsigned dataflow_phases_per_token(int n_layers);
+
 }  // namespace lpp

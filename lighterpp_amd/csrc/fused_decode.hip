@@ -359,6 +359,8 @@ size_t persistent_lds_bytes(const lpp_model* m) {
 
 template <bool kF16>
 lpp_status persistent_launch(lpp_model* m, const DecodeArgs& a, hipStream_t s) {
+    static const bool use_barriers = std::getenv("LPP_DECODE_BARRIERS") != nullptr;
+    if (!use_barriers) return dataflow_launch(m, a, s);
     if (m->persist_grid == 0) {
         int per_cu = 0;
         LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode_token<kF16>, kPersistThreads,
@@ -474,6 +476,10 @@ lpp_status fused_prepare(lpp_model* m) {
     LPP_TRY(lpp_memset(m->sync_words, 0, 128 * sizeof(unsigned)));
     LPP_TRY(lpp_malloc(&p, 4 * smp::kMaxChunks * sizeof(float)));
     m->sample_scratch = static_cast<float*>(p);
+    LPP_TRY(lpp_malloc(&p, dataflow_tagged_bytes(m)));
+    m->tagged = p;
+    LPP_TRY(lpp_memset(m->tagged, 0, dataflow_tagged_bytes(m)));
+    m->df_base = 0;
     return LPP_OK;
 }
 
@@ -486,6 +492,7 @@ lpp_status fused_release(lpp_model* m) {
     lpp_free(m->work_logits);
     lpp_free(m->sync_words);
     lpp_free(m->sample_scratch);
+    lpp_free(m->tagged);
     lpp_free(m->gen_uniforms);
     return LPP_OK;
 }
@@ -745,7 +752,8 @@ extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long*
     if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
     for (int t = 0; t < LPP_T_COUNT; ++t)
         if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
-    const int nb = static_cast<int>(barriers_per_token(m->cfg.n_layers));
+    const int nb = static_cast<int>(std::getenv("LPP_DECODE_BARRIERS") ? barriers_per_token(m->cfg.n_layers)
+                                                                       : dataflow_phases_per_token(m->cfg.n_layers));
     LPP_REQUIRE(capacity >= 2 * nb, "lpp_trace_token: capacity %d < %d", capacity, 2 * nb);
     const int saved_path = m->path;
     m->path = LPP_PATH_PERSISTENT;

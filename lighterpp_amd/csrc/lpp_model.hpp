@@ -53,6 +53,8 @@ struct lpp_model {
     float* sample_scratch = nullptr;         // 4 x kMaxChunks words
     float* gen_uniforms = nullptr;           // device copy of the per-step draws
     int gen_cap = 0;
+    void* tagged = nullptr;                  // value+sequence-number vectors of the persistent kernel
+    unsigned df_base = 0;                    // sequence-number base of the next persistent launch
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
     unsigned spin_limit = 1u << 20;          // polls a grid-barrier wait may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
