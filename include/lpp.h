@@ -243,11 +243,15 @@ typedef struct lpp_kernel_time {
 lpp_status lpp_profile_kernels(lpp_model *m, int pos, int reps, lpp_kernel_time *out, int capacity,
                                int *count);
 
-/* Timeline of one token on LPP_PATH_PERSISTENT at position `pos`: for grid barrier
- * i, out[2i] is when workgroup 0 arrived and out[2i+1] when it was released, in
- * 10 ns ticks from the kernel's start.  Barrier order per layer: qkv, attention,
- * o-projection, gate/up, down; then classifier and four sampler steps. */
-lpp_status lpp_trace_token(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count);
+/* Timeline of one token on LPP_PATH_PERSISTENT at position `pos`, as seen by
+ * workgroup 0: out[marks * i + k] is mark k of phase i in 10 ns ticks from the
+ * kernel's start (0 = mark not taken).  Phase order per layer: qkv, attention,
+ * o-projection, gate/up, down; then classifier and sampler.  Marks: 0 phase
+ * entered, 1 own inputs received, 2 inputs staged, 3 row results ready,
+ * 4 outputs published, 5 first weight step multiplied, 6 last row finished.
+ * *count = marks * phases, *marks_per_phase = marks. */
+lpp_status lpp_trace_token(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count,
+                           int *marks_per_phase);
 
 /* ===================================================================== */
 /* C. Runtime plumbing                                                    */

@@ -90,7 +90,7 @@ SIGNATURES = {
     "lpp_forward": (_i, [_vp, _i, _i, _f, _f, _f, _vp, _i, _f, _ip]),
     "lpp_generate": (_i, [_vp, _i, _i, _i, _f, _f, _f, _vp, _ip, _i, _vp, _vp, C.POINTER(LppGenStats)]),
     "lpp_profile_kernels": (_i, [_vp, _i, _i, C.POINTER(LppKernelTime), _i, _ip]),
-    "lpp_trace_token": (_i, [_vp, _i, C.POINTER(C.c_ulonglong), _i, _ip]),
+    "lpp_trace_token": (_i, [_vp, _i, C.POINTER(C.c_ulonglong), _i, _ip, _ip]),
     # C. runtime
     "lpp_last_error": (C.c_char_p, []),
     "lpp_version": (C.c_char_p, []),

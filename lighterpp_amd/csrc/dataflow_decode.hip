@@ -1,26 +1,42 @@
 // dataflow_decode.hip -- LPP_PATH_PERSISTENT: one kernel per token, no grid
-// barrier.  The phases of forward() (reference src/model.cpp:342-371; see
-// decode_phases.hpp for the split) are chained by the data itself: every value
-// one phase hands to the next is published as ONE 8-byte device-scope store
-// holding the fp32 value and a 32-bit sequence number, and a consumer simply
-// polls the values it needs until their sequence number is the one it expects.
+// barrier, weights streamed independently of the dependency chain.
 //
-// Why: on this part a counter barrier across 256 workgroups costs ~3.7 us and
-// the staging read behind it another memory round trip, five times per layer;
-// with tagged values the hand-over is one round trip (the poll that sees the
-// tag has the data in hand), and nothing waits for workgroups it does not
-// depend on.  Weights never depend on activations: each phase requests its
-// first weight tiles before it starts polling.
+// The phases of forward() (reference src/model.cpp:342-371; decode_phases.hpp
+// describes the split) need a full activation vector from all workgroups at
+// every boundary.  Here the hand-over is the data itself: every value one phase
+// gives to the next is published as ONE 8-byte device-scope store holding the
+// fp32 value and a 32-bit sequence number, and a consumer polls the values it
+// needs until they carry the number it expects.  A hand-over costs one memory
+// round trip and nobody waits for a workgroup it does not depend on.
+//
+// A batch-1 decode is a chain of ~80 such hand-overs, each a couple of
+// microseconds of pure latency during which a conventional GEMV kernel has
+// nothing in flight.  The weights, however, do not depend on anything, and the
+// order in which a wavefront will need them is fixed.  Each workgroup is
+// therefore split into two kinds of wavefronts:
+//
+//   streaming wavefronts  walk their fixed list of weight rows across ALL phases
+//       and layers of the token with kDepth 2-KiB steps always in flight in
+//       registers.  They never touch global memory otherwise: activations come
+//       from LDS, results go to LDS, and they only ever wait on an LDS flag.
+//       While the dependency chain is stalled they already hold the next
+//       phases' weights.
+//   exchange wavefronts   poll the tagged inputs of a phase (their loads never
+//       queue behind weight traffic), normalise and stage them in LDS, raise the
+//       flag, later pick up the row results, apply the phase's epilogue (RoPE,
+//       SwiGLU, residual) and publish.  They also run attention and the sampler.
 //
 // Sequence numbers grow monotonically for the life of a model (the host hands
 // every launch its base and advances it by the number of phases), so a stale
-// value, even one left by a launch that gave up, is never taken for a fresh one.  Buffer reuse is safe without further synchronisation:
-// every buffer is consumed one phase after it is produced and rewritten no
-// sooner than two phases later, and each phase's inputs transitively require
-// every workgroup to have finished reading the phase before the previous one.
-// Polls are bounded: a workgroup that gives up raises a shared abort flag that
-// ends every other poll, so the grid always drains.
+// value, even one left by a launch that gave up, is never taken for a fresh
+// one.  Buffer reuse needs no further synchronisation: every buffer is consumed
+// one phase after it is produced and rewritten no sooner than two phases later,
+// and the inputs of each phase transitively require every workgroup to have
+// finished reading the phase before the previous one.  Global polls are bounded:
+// a wavefront that gives up raises a shared abort flag that ends every other
+// poll, and no LDS wait depends on a global one, so the grid always drains.
 #include <cstring>
+#include <vector>
 
 #include "decode_phases.hpp"
 
@@ -30,9 +46,15 @@ namespace df {
 using namespace ph;
 using namespace dev;
 
-constexpr int kThreads = 512;
-constexpr int kWaves = kThreads / kWave;
-constexpr int kPollBatch = 16;  // tagged values one thread requests before checking any
+constexpr int kGemvWaves = 8;                      // streaming wavefronts per workgroup
+constexpr int kIoWaves = 8;                        // exchange wavefronts per workgroup
+constexpr int kThreads = (kGemvWaves + kIoWaves) * kWave;
+constexpr int kIoThreads = kIoWaves * kWave;
+constexpr int kDepth = 8;                          // weight steps a streaming wavefront keeps in flight
+constexpr int kStepLoads = 2;                      // 16-byte loads per lane and step: 2 KiB of one row
+constexpr int kPollBatch = 16;                     // tagged values one thread requests before checking any
+constexpr int kItemPositions = 256;                // context positions per attention work item
+constexpr int kMaxHeadPad = 128;
 
 typedef unsigned long long u64;
 
@@ -56,16 +78,74 @@ struct Tagged {
     u64* v;      // [kv_dim]
     u64* xb;     // [dim]     attention output
     u64* hb;     // [hidden]  SwiGLU output
-    u64* part;   // [n_heads][max_splits][head_size + 2] attention split partials
+    u64* part;   // [n_heads][splits_cap][head_size + 2] attention split partials
     u64* stats;  // [nwg][4]  per-workgroup sampler statistics (max, sum, argmax)
+    int splits_cap;
     unsigned base;    // sequence-number base of this launch, advanced by the host once per token
-    unsigned* abort;  // raised by a workgroup whose poll ran out of patience
+    unsigned* abort;  // raised by a wavefront whose poll ran out of patience
     unsigned spin_limit;
 };
+
+// Rows of each matrix one workgroup owns (a contiguous block), and LDS sizes.
+struct Blocks {
+    int qkv;    // rows of the stacked [Wq; Wk; Wv], even
+    int o;      // rows of Wo
+    int gu;     // hidden units (one gate row and one up row each)
+    int down;   // rows of W2
+    int cls;    // rows of the classifier
+    int xs_floats;
+    int results_floats;
+    int gather_floats;
+};
+
+// Workgroup-local coordination words.  Everything here is accessed with plain
+// (volatile) LDS operations: LDS executes one wavefront's operations in order,
+// so a flag written after data is seen after the data.
+struct Control {
+    unsigned staged;                 // += 1 by every exchange wavefront once it has staged a GEMV phase
+    unsigned io_bar;                 // arrival counter of the exchange wavefronts' barrier
+    unsigned progress[kGemvWaves];   // GEMV phases wavefront j has completed
+    float red[2][kIoWaves];
+    float redv[2][kIoWaves];
+    int redi[2][kIoWaves];
+    float wave_tot[kIoWaves];
+    int wave_found[kIoWaves];
+    int target, token;
+};
+
+// (relaxed workgroup-scope atomics rather than volatile: they keep the LDS address
+// space, so they compile to plain ds_read / ds_write, and are never hoisted)
+template <class T>
+__device__ __forceinline__ T lds_ld(const T* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ unsigned lds_peek(const unsigned* p) { return lds_ld(p); }
+__device__ __forceinline__ void lds_poke(unsigned* p, unsigned v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory"); }
+
+// Waits on LDS words are satisfied by construction (neither kind of wavefront
+// ever waits for global memory before raising them); the bound only makes sure a
+// mistake in that reasoning ends as a reported error instead of a hung device.
+constexpr unsigned kLdsSpinLimit = 1u << 22;
+template <class Ready>
+__device__ __forceinline__ void lds_wait(StepParams* step, Ready ready) {
+    unsigned spins = 0;
+    while (!ready()) {
+        if (++spins > kLdsSpinLimit) {
+            step->error = 2;
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
 
 struct Ctx {
     const DecodeArgs& a;
     const Tagged& t;
+    const Blocks& b;
+    Control& ctl;
     unsigned base;  // sequence-number base of this token
     unsigned long long* trace;
     unsigned phase_index;
@@ -74,31 +154,250 @@ struct Ctx {
     // sampler, so nothing reads them from memory after the first phase began.
     int token, pos, history_len;
     float temperature, penalty, r;
+    int wg, nwg;
 
     __device__ __forceinline__ unsigned seq(int layer, int phase) const {
         return base + 1u + 5u * static_cast<unsigned>(layer) + static_cast<unsigned>(phase);
     }
     __device__ __forceinline__ unsigned seq_stats() const { return base + 1u + 5u * static_cast<unsigned>(a.n_layers); }
-    __device__ __forceinline__ void mark(int which) {
-        if (trace && threadIdx.x == 0) trace[2u * phase_index + which] = wall_clock64();
-    }
 };
 
 __host__ __device__ inline unsigned phases_per_token(int n_layers) { return 5u * n_layers + 2u; }
+// Timeline marks per phase (workgroup 0): 0 phase entered, 1 own inputs received,
+// 2 inputs staged, 3 streaming wavefronts done, 4 outputs published (exchange
+// thread 0); 5 staged flag seen, 6 last row done (streaming wavefront 0).
+constexpr unsigned kTraceMarks = 8;
 enum { kQkv = 0, kAtt = 1, kOproj = 2, kGateUp = 3, kDown = 4 };
+// GEMV phases as the streaming wavefronts count them: 4 per layer, then the classifier.
+enum { kGQkv = 0, kGO = 1, kGGateUp = 2, kGDown = 3, kGCls = 4 };
+
+// ---------------------------------------------------------------------------
+// Streaming wavefronts
+// ---------------------------------------------------------------------------
+
+// The order in which a streaming wavefront needs its weights is fixed by the
+// model's shape, so the host lists it once: for every (workgroup, wavefront) the
+// rows it owns, in order, across all GEMV phases of a token.  The wavefront
+// walks the list with scalar loads, which share nothing with the counter its
+// weight loads complete on.
+struct RowEntry {
+    unsigned long long ptr;  // first byte of the row
+    unsigned meta;           // kRowLocal | phase << 16 | flags
+    unsigned pad;
+};
+constexpr unsigned kRowWide = 1u << 28;   // columns = hidden_dim (down projection), else dim
+constexpr unsigned kRowLast = 1u << 29;   // this wavefront's last row of the phase
+constexpr unsigned kRowValid = 1u << 31;  // cleared in the terminating entries
+constexpr unsigned kRowPhaseShift = 16, kRowPhaseMask = 0xfffu, kRowLocalMask = 0xffffu;
+
+template <bool kF16>
+__device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, const uint4* __restrict__ rows, int j,
+                                          const float* xs, float* results, unsigned long long* trace) {
+    constexpr int kPer = WTraits<kF16>::kPerLoad;
+    constexpr int kBytes = WTraits<kF16>::kBytes;
+    constexpr int kChunkCols = kWave * kPer;
+    constexpr int kStepCols = kStepLoads * kChunkCols;
+    const int lane = lane_id();
+    const int dim = a.dim, hidden = a.hidden;
+    const int nseg_dim = (dim + kStepCols - 1) / kStepCols;
+    const int nseg_hidden = (hidden + kStepCols - 1) / kStepCols;
+    const unsigned n_phases = 4u * static_cast<unsigned>(a.n_layers) + 1u;
+
+    // issue side: current row, the one after it (already fetched), segment
+    uint4 cur = rows[0];
+    uint4 nxt = rows[1];
+    int e = 1;
+    int seg = 0;
+    int nseg = (cur.z & kRowWide) ? nseg_hidden : nseg_dim;
+
+    uintx4 w[kDepth][kStepLoads];
+    unsigned meta[kDepth];  // row entry meta of the step held in w[k]
+    unsigned part[kDepth];  // its segment, bit 8: last segment of the row
+
+    auto request = [&](int k) {
+        typedef const char __attribute__((address_space(1)))* GlobalBytes;  // not a generic pointer: plain global loads
+        typedef const uintx4 __attribute__((address_space(1)))* GlobalVec;
+        const GlobalBytes ptr = reinterpret_cast<GlobalBytes>(static_cast<unsigned long long>(cur.x) |
+                                                              (static_cast<unsigned long long>(cur.y) << 32));
+        const int d = (cur.z & kRowWide) ? hidden : dim;
+#pragma unroll
+        for (int u = 0; u < kStepLoads; ++u) {
+            const int col = (seg * kStepLoads + u) * kChunkCols + lane * kPer;
+            const int safe_col = (col < d) ? col : 0;
+            w[k][u] = __builtin_nontemporal_load(reinterpret_cast<GlobalVec>(ptr + static_cast<size_t>(safe_col) * kBytes));
+        }
+        meta[k] = cur.z;
+        part[k] = static_cast<unsigned>(seg) | ((seg + 1 == nseg) ? 0x100u : 0u);
+        if (cur.z & kRowValid) {  // the terminating entry repeats itself
+            if (++seg == nseg) {
+                seg = 0;
+                cur = nxt;
+                e += 1;
+                nxt = rows[e];
+                nseg = (cur.z & kRowWide) ? nseg_hidden : nseg_dim;
+            }
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < kDepth; ++k) request(k);
+    {
+        const unsigned first = (meta[0] & kRowValid) ? ((meta[0] >> kRowPhaseShift) & kRowPhaseMask) : n_phases;
+        if (lane == 0) lds_poke(&ctl.progress[j], first);
+    }
+
+    // timeline slot of GEMV phase p (attention sits between qkv and the O projection)
+    auto trace_phase = [&](unsigned p) {
+        const unsigned kind = p & 3u;
+        return p + 1u == n_phases ? 5u * (p >> 2) : 5u * (p >> 2) + (kind == 0u ? 0u : kind + 1u);
+    };
+    unsigned cur_p = 0xffffffffu;
+    float acc = 0.0f;
+    const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    bool more = true;
+    while (more) {
+#pragma unroll
+        for (int k = 0; k < kDepth; ++k) {
+            const unsigned mt = meta[k];
+            if (more && (mt & kRowValid)) {
+                const int sg = static_cast<int>(part[k] & 0xffu);
+                const int d = (mt & kRowWide) ? hidden : dim;
+                const unsigned p = (mt >> kRowPhaseShift) & kRowPhaseMask;
+                if (p != cur_p) {  // first step of a phase: its activations must be staged
+                    cur_p = p;
+                    const unsigned need = static_cast<unsigned>(kIoWaves) * (p + 1u);
+                    lds_wait(a.step, [&]() { return static_cast<int>(lds_peek(&ctl.staged) - need) >= 0; });
+                    compiler_fence();
+                    if (trace && lane == 0) trace[kTraceMarks * trace_phase(p) + 5u] = wall_clock64();
+                }
+#pragma unroll
+                for (int u = 0; u < kStepLoads; ++u) {
+                    const int col = (sg * kStepLoads + u) * kChunkCols + lane * kPer;
+                    const bool live = col < d;
+                    const int safe_col = live ? col : 0;
+                    if constexpr (kF16) {
+                        floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                        floatx4 xb = *reinterpret_cast<const floatx4*>(xs + safe_col + 4);
+                        xa = live ? xa : zero;
+                        xb = live ? xb : zero;
+                        acc = dot8(w[k][u], xa, xb, acc);
+                    } else {
+                        floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                        xa = live ? xa : zero;
+                        acc = dot4(w[k][u], xa, acc);
+                    }
+                }
+                if (part[k] & 0x100u) {  // last segment of the row
+                    const float sum = wave_sum(acc);
+                    if (lane == 0) results[mt & kRowLocalMask] = sum;
+                    acc = 0.0f;
+                    if (mt & kRowLast) {  // everything before the next step's phase is complete
+                        const unsigned nm = meta[(k + 1) % kDepth];
+                        const unsigned next_p = (nm & kRowValid) ? ((nm >> kRowPhaseShift) & kRowPhaseMask) : n_phases;
+                        compiler_fence();
+                        if (lane == 0) lds_poke(&ctl.progress[j], next_p);
+                        if (trace && lane == 0) trace[kTraceMarks * trace_phase(p) + 6u] = wall_clock64();
+                    }
+                }
+            } else {
+                more = false;
+            }
+            request(k);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Exchange wavefronts: synchronisation among themselves
+// ---------------------------------------------------------------------------
+
+struct Io {
+    int it;        // thread index among the exchange threads
+    int iw;        // exchange wavefront index
+    unsigned gen;  // barrier generation
+    int parity;    // reduction slot parity
+    StepParams* step;
+};
+
+__device__ __forceinline__ void io_sync(Control& ctl, Io& io) {
+    compiler_fence();
+    io.gen += static_cast<unsigned>(kIoWaves);
+    if (lane_id() == 0) __hip_atomic_fetch_add(&ctl.io_bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const unsigned gen = io.gen;
+    lds_wait(io.step, [&]() { return static_cast<int>(lds_peek(&ctl.io_bar) - gen) >= 0; });
+    compiler_fence();
+}
+
+// Sum over all exchange threads; every thread gets the total (wavefront order).
+__device__ __forceinline__ float io_sum(Control& ctl, Io& io, float v) {
+    const float s = wave_sum(v);
+    float* slot = ctl.red[io.parity];
+    if (lane_id() == 0) slot[io.iw] = s;
+    io_sync(ctl, io);
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kIoWaves; ++w) total += lds_ld(slot + w);
+    io.parity ^= 1;
+    return total;
+}
+__device__ __forceinline__ float io_max(Control& ctl, Io& io, float v) {
+    const float s = wave_max(v);
+    float* slot = ctl.red[io.parity];
+    if (lane_id() == 0) slot[io.iw] = s;
+    io_sync(ctl, io);
+    float total = lds_ld(slot);
+#pragma unroll
+    for (int w = 1; w < kIoWaves; ++w) total = fmaxf(total, lds_ld(slot + w));
+    io.parity ^= 1;
+    return total;
+}
+
+__device__ __forceinline__ void signal_staged(Control& ctl) {
+    compiler_fence();
+    if (lane_id() == 0) __hip_atomic_fetch_add(&ctl.staged, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// Wait until every streaming wavefront has completed GEMV phase p.
+__device__ __forceinline__ void wait_gemv(Control& ctl, const Io& io, int p) {
+    const unsigned need = static_cast<unsigned>(p + 1);
+    lds_wait(io.step, [&]() {
+        unsigned lowest = lds_peek(&ctl.progress[0]);
+#pragma unroll
+        for (int w = 1; w < kGemvWaves; ++w) lowest = min(lowest, lds_peek(&ctl.progress[w]));
+        return lowest >= need;
+    });
+    compiler_fence();
+}
+
+__device__ __forceinline__ void mark(Ctx& c, const Io& io, int which) {
+    if (c.trace && io.it == 0) c.trace[kTraceMarks * c.phase_index + which] = wall_clock64();
+}
+
+// ---------------------------------------------------------------------------
+// Polling
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ bool poll_give_up(const Ctx& c, unsigned& spins) {
+    if ((spins & 63u) == 63u && __hip_atomic_load(c.t.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return true;
+    if (++spins > c.t.spin_limit) {
+        __hip_atomic_store(c.t.abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        c.a.step->error = 1;
+        return true;
+    }
+    __builtin_amdgcn_s_sleep(1);
+    return false;
+}
 
 // Fetch n tagged values carrying sequence number `want` and hand each to
-// sink(i, value).  A thread requests up to kPollBatch values, then re-requests
-// only those that were not there yet.
+// sink(i, value); the exchange threads share the range.  A thread requests up
+// to kPollBatch values, then re-requests only those that were not there yet.
 template <class Sink>
-__device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want, const Ctx& c, Sink sink) {
-    const int nthreads = static_cast<int>(blockDim.x);
-    for (int first = static_cast<int>(threadIdx.x); first < n; first += nthreads * kPollBatch) {
+__device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want, const Ctx& c, const Io& io, Sink sink) {
+    for (int first = io.it; first < n; first += kIoThreads * kPollBatch) {
         u64 got[kPollBatch];
         unsigned pending = 0u;
 #pragma unroll
         for (int j = 0; j < kPollBatch; ++j) {
-            const int i = first + j * nthreads;
+            const int i = first + j * kIoThreads;
             if (i < n) {
                 got[j] = peek(src + i);
                 pending |= 1u << j;
@@ -111,99 +410,119 @@ __device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want
                 if ((pending >> j) & 1u)
                     if (tag_of(got[j]) == want) pending &= ~(1u << j);
             if (pending == 0u) break;
-            if ((spins & 63u) == 63u && __hip_atomic_load(c.t.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
-            if (++spins > c.t.spin_limit) {
-                __hip_atomic_store(c.t.abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                c.a.step->error = 1;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
+            if (poll_give_up(c, spins)) break;
 #pragma unroll
             for (int j = 0; j < kPollBatch; ++j)
-                if ((pending >> j) & 1u) got[j] = peek(src + first + j * nthreads);
+                if ((pending >> j) & 1u) got[j] = peek(src + first + j * kIoThreads);
         }
 #pragma unroll
         for (int j = 0; j < kPollBatch; ++j) {
-            const int i = first + j * nthreads;
+            const int i = first + j * kIoThreads;
             if (i < n) sink(i, value_of(got[j]));
         }
     }
 }
 
-// xs = the tagged vector itself, zero padded to a multiple of 8.  The leading
-// block barrier keeps xs intact until every wavefront has left the phase that
-// was reading it.
-__device__ __forceinline__ void stage_tagged(float* xs, const u64* src, int n, unsigned want, const Ctx& c) {
+// N tagged values per thread at addresses addr(j), all requested at once.
+template <int N, class AddrFn>
+__device__ __forceinline__ void poll_n(AddrFn addr, float (&out)[N], unsigned want, const Ctx& c) {
+    static_assert(N <= 32, "pending mask is 32 bits");
+    u64 got[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) got[j] = peek(addr(j));
+    unsigned pending = (N == 32) ? 0xffffffffu : ((1u << N) - 1u);
+    unsigned spins = 0;
+    while (true) {
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            if ((pending >> j) & 1u)
+                if (tag_of(got[j]) == want) pending &= ~(1u << j);
+        if (pending == 0u) break;
+        if (poll_give_up(c, spins)) break;
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            if ((pending >> j) & 1u) got[j] = peek(addr(j));
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = value_of(got[j]);
+}
+
+// ---------------------------------------------------------------------------
+// Staging (exchange wavefronts)
+// ---------------------------------------------------------------------------
+
+struct Lds {
+    float* xraw;     // [dim_pad]   residual stream as last received
+    float* xs;       // [xs_floats] staged GEMV input; sampler tables after the classifier
+    float* results;  // [results_floats] row results of the current GEMV phase
+    float* sc;       // [kItemPositions] attention scores
+    float* red;      // [kIoWaves][kMaxHeadPad] attention cross-wavefront reduction
+    float* gather;   // [gather_floats] attention split partials
+};
+
+// xs = the tagged vector itself, zero padded to a multiple of 8.
+__device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, int n, unsigned want) {
     const int n_pad = (n + 7) & ~7;
-    __syncthreads();
-    for (int i = n + threadIdx.x; i < n_pad; i += blockDim.x) xs[i] = 0.0f;
-    poll_values(src, n, want, c, [&](int i, float v) { xs[i] = v; });
-    __syncthreads();
+    for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
+    poll_values(src, n, want, c, io, [&](int i, float v) { xs[i] = v; });
+    mark(c, io, 1);
+    signal_staged(c.ctl);
 }
 
 // xraw = the input vector (tagged x, or the embedding row for layer 0);
 // xs = rmsnorm(xraw) * gain, ops.cpp:20-32.
-__device__ __forceinline__ void stage_norm(float* xraw, float* xs, const u64* tagged_x, const float* plain_x, int n,
-                                           unsigned want, const float* gain, const Ctx& c) {
+__device__ __forceinline__ void stage_norm(Ctx& c, Io& io, const Lds& l, const u64* tagged_x, const float* plain_x, int n,
+                                           unsigned want, const float* gain) {
 #pragma clang fp contract(off)
-    __shared__ float scratch[16];
+    float* xraw = l.xraw;
+    float* xs = l.xs;
     if (plain_x != nullptr) {
-        for (int i = threadIdx.x; i < n; i += blockDim.x) xraw[i] = plain_x[i];
+        for (int i = io.it; i < n; i += kIoThreads) xraw[i] = plain_x[i];
     } else {
-        poll_values(tagged_x, n, want, c, [&](int i, float v) { xraw[i] = v; });
+        poll_values(tagged_x, n, want, c, io, [&](int i, float v) { xraw[i] = v; });
     }
+    mark(c, io, 1);
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {  // same index set this thread wrote
+    for (int i = io.it; i < n; i += kIoThreads) {  // the index set this thread wrote
         const float v = xraw[i];
         ss += v * v;
     }
-    ss = block_sum(ss, scratch);
+    ss = io_sum(c.ctl, io, ss);
     ss /= static_cast<float>(n);
     ss += 1e-5f;
     const float scale = 1.0f / sqrtf(ss);
     const int n_pad = (n + 7) & ~7;
-    for (int i = threadIdx.x; i < n_pad; i += blockDim.x) xs[i] = (i < n) ? xraw[i] * scale * gain[i] : 0.0f;
-    __syncthreads();
+    for (int i = io.it; i < n_pad; i += kIoThreads) xs[i] = (i < n) ? xraw[i] * scale * gain[i] : 0.0f;
+    signal_staged(c.ctl);
 }
 
-struct Lds {
-    float* xraw;    // [dim_pad]   residual stream as last received
-    float* xs;      // [max(dim, hidden)_pad]  staged GEMV input; attention scratch overlays it
-    float* local;   // [rows per workgroup of the classifier, padded]
-};
-
 // ---------------------------------------------------------------------------
-// GEMV phases
+// GEMV phases as the exchange wavefronts see them
 // ---------------------------------------------------------------------------
 
-template <bool kF16>
-__device__ __forceinline__ void df_qkv(Ctx& c, const Lds& l, int layer, int wg, int nwg) {
+__device__ __forceinline__ int block_rows(int total, int block, int wg) {
+    const int n = total - wg * block;
+    return n < 0 ? 0 : (n > block ? block : n);
+}
+
+__device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) {
 #pragma clang fp contract(off)
-    constexpr int kRows = 2;
     const DecodeArgs& a = c.a;
-    const int wbytes = kF16 ? 2 : 4;
-    const int dim = a.dim, kv_dim = a.kv_dim, total_rows = a.dim + 2 * a.kv_dim;
-    const int ntiles = (total_rows + kRows - 1) / kRows;
-    auto row_ptr = [&](int tile, int r) -> const char* {
-        const int g = tile * kRows + r;
-        if (g < dim) return row_at(a.wq, dim, layer, g, dim, wbytes);
-        if (g < dim + kv_dim) return row_at(a.wk, kv_dim, layer, g - dim, dim, wbytes);
-        const int gv = (g < total_rows ? g : total_rows - 1) - dim - kv_dim;
-        return row_at(a.wv, kv_dim, layer, gv, dim, wbytes);
-    };
-    auto pre = [&]() {
-        const float* emb_row = (layer == 0) ? a.emb + static_cast<size_t>(c.token) * dim : nullptr;
-        stage_norm(l.xraw, l.xs, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
-                   a.rms_att + static_cast<size_t>(layer) * dim, c);
-        c.mark(0);
-    };
-    const int pos = c.pos;
-    const int hs = a.head_size;
-    const float2* cs_row = a.rope + static_cast<size_t>(pos) * (hs / 2);
+    const int dim = a.dim, kv_dim = a.kv_dim, hs = a.head_size;
+    const float* emb_row = (layer == 0) ? a.emb + static_cast<size_t>(c.token) * dim : nullptr;
+    mark(c, io, 0);
+    stage_norm(c, io, l, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
+               a.rms_att + static_cast<size_t>(layer) * dim);
+    mark(c, io, 2);
+    wait_gemv(c.ctl, io, 4 * layer + kGQkv);
+    mark(c, io, 3);
+    const int row0 = c.wg * c.b.qkv;
+    const int nrows = block_rows(dim + 2 * kv_dim, c.b.qkv, c.wg);
+    const float2* cs_row = a.rope + static_cast<size_t>(c.pos) * (hs / 2);
     const unsigned tag = c.seq(layer, kQkv);
-    auto emit = [&](int tile, int r, float mine, float neighbour) {
-        const int g = tile * kRows + r;
-        if (g >= total_rows) return;
+    for (int r = io.it; r < nrows; r += kIoThreads) {
+        const int g = row0 + r;
+        const float mine = l.results[r], neighbour = l.results[r ^ 1];
         float out = mine;
         if (g < dim + kv_dim) {  // ops.cpp:36-52 on the pair (i, i+1)
             const int gi = (g < dim) ? g : g - dim;
@@ -218,457 +537,348 @@ __device__ __forceinline__ void df_qkv(Ctx& c, const Lds& l, int layer, int wg, 
             const int i = is_k ? g - dim : g - dim - kv_dim;
             const int head = i / hs, within = i - head * hs;
             const size_t dst = static_cast<size_t>(layer) * kv_dim * a.seq_len +
-                               static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(pos) * hs + within;
+                               static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(c.pos) * hs + within;
             publish((is_k ? c.t.k : c.t.v) + i, out, tag);
             (is_k ? a.k : a.v)[i] = out;
             (is_k ? a.key_cache : a.value_cache)[dst] = f32_to_f16_bits(out);
         }
-    };
-    gemv_phase<kF16, kRows, 4>(ntiles, dim, l.xs, wg * kWaves + wave_index(), nwg * kWaves, row_ptr, emit, pre);
-    c.mark(1);
+    }
+    mark(c, io, 4);
     ++c.phase_index;
 }
 
-// out = W . src + xraw (model.cpp:160,218 and :225-226); the result is the new x.
-template <bool kF16, int kRows, int kUnroll>
-__device__ __forceinline__ void df_proj(Ctx& c, const Lds& l, const char* w_layer, int n, int d, const u64* src,
-                                        unsigned src_tag, unsigned out_tag, int wg, int nwg) {
-    const int wbytes = kF16 ? 2 : 4;
-    const int ntiles = (n + kRows - 1) / kRows;
-    auto row_ptr = [&](int tile, int r) -> const char* {
-        const int g = tile * kRows + r;
-        return w_layer + static_cast<size_t>(g < n ? g : n - 1) * d * wbytes;
-    };
-    auto pre = [&]() {
-        stage_tagged(l.xs, src, d, src_tag, c);
-        c.mark(0);
-    };
-    auto emit = [&](int tile, int r, float mine, float) {
-        const int g = tile * kRows + r;
-        if (g < n) publish(c.t.x + g, l.xraw[g] + mine, out_tag);
-    };
-    gemv_phase<kF16, kRows, kUnroll>(ntiles, d, l.xs, wg * kWaves + wave_index(), nwg * kWaves, row_ptr, emit, pre);
-    c.mark(1);
+// x = xraw + W . src (model.cpp:160,218 and :225-226)
+__device__ __forceinline__ void io_proj(Ctx& c, Io& io, const Lds& l, int gphase, int block, int d, const u64* src,
+                                        unsigned src_tag, unsigned out_tag) {
+    mark(c, io, 0);
+    stage_tagged(c, io, l.xs, src, d, src_tag);
+    mark(c, io, 2);
+    wait_gemv(c.ctl, io, gphase);
+    mark(c, io, 3);
+    const int row0 = c.wg * block;
+    const int nrows = block_rows(c.a.dim, block, c.wg);
+    for (int r = io.it; r < nrows; r += kIoThreads) publish(c.t.x + row0 + r, l.xraw[row0 + r] + l.results[r], out_tag);
+    mark(c, io, 4);
     ++c.phase_index;
 }
 
-template <bool kF16>
-__device__ __forceinline__ void df_gateup(Ctx& c, const Lds& l, int layer, int wg, int nwg) {
+__device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int layer) {
 #pragma clang fp contract(off)
-    constexpr int kRows = 2;  // row 0 = gate row j, row 1 = up row j
     const DecodeArgs& a = c.a;
-    const int wbytes = kF16 ? 2 : 4;
-    const int hidden = a.hidden, dim = a.dim;
-    auto row_ptr = [&](int tile, int r) -> const char* {
-        return row_at(r ? a.w3 : a.w1, hidden, layer, tile < hidden ? tile : hidden - 1, dim, wbytes);
-    };
-    auto pre = [&]() {
-        stage_norm(l.xraw, l.xs, c.t.x, nullptr, dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * dim, c);
-        c.mark(0);
-    };
+    mark(c, io, 0);
+    stage_norm(c, io, l, c.t.x, nullptr, a.dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * a.dim);
+    mark(c, io, 2);
+    wait_gemv(c.ctl, io, 4 * layer + kGGateUp);
+    mark(c, io, 3);
+    const int unit0 = c.wg * c.b.gu;
+    const int units = block_rows(a.hidden, c.b.gu, c.wg);
     const unsigned tag = c.seq(layer, kGateUp);
-    auto emit = [&](int tile, int r, float gate, float up) {
-        if (r != 0 || tile >= hidden) return;
+    for (int u = io.it; u < units; u += kIoThreads) {
+        const float gate = l.results[2 * u], up = l.results[2 * u + 1];
         const float sigma = 1.0f / (1.0f + expf(-gate));  // ops.cpp:80-85
-        publish(c.t.hb + tile, (gate * sigma) * up, tag);
-    };
-    gemv_phase<kF16, kRows, 4>(hidden, dim, l.xs, wg * kWaves + wave_index(), nwg * kWaves, row_ptr, emit, pre);
-    c.mark(1);
+        publish(c.t.hb + unit0 + u, (gate * sigma) * up, tag);
+    }
+    mark(c, io, 4);
     ++c.phase_index;
 }
 
 // ---------------------------------------------------------------------------
-// Attention
+// Attention (exchange wavefronts)
 // ---------------------------------------------------------------------------
 
-// One work item (KV head, context split); same arithmetic as ph::attention_item.
-// K rows of positions before the current one are requested before q is polled;
-// the current position's k and v arrive tagged and are rounded to binary16
-// exactly as the cache store rounds them.
+// One work item: query head h, context split `split` of `nsplits` (at most
+// kItemPositions positions).  kGroup lanes cover one position, 8 binary16 each.
+// K and V rows of earlier positions do not depend on this token and are
+// requested before q is polled; the current position's k and v arrive tagged and
+// are rounded to binary16 exactly as the cache store rounds them.  Scores go to
+// LDS once; every wavefront then forms the maximum and the sum of exponentials
+// for itself (model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped).
 template <int kGroup>
-__device__ __forceinline__ void df_attention_item(Ctx& c, int layer, int kvh, int split, int nsplits, int npos,
-                                                  float* lds) {
+__device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer, int h, int split, int nsplits,
+                                         int npos, bool first_item) {
     const DecodeArgs& a = c.a;
-    const int hs = a.head_size, gqa = a.gqa;
+    const int hs = a.head_size;
     constexpr int hs_pad = kGroup * 8;
-    const int nthreads = static_cast<int>(blockDim.x);
-    const int nwaves = nthreads / kWave;
-    const int ngroups = nthreads / kGroup;
-    const int tid = static_cast<int>(threadIdx.x);
-    const int sub = tid % kGroup, grp = tid / kGroup;
-    const int wave = tid / kWave;
+    constexpr int ngroups = kIoThreads / kGroup;
+    constexpr int kRounds = (kItemPositions + ngroups - 1) / ngroups;
+    const int kvh = h / a.gqa;
+    const int sub = io.it % kGroup, grp = io.it / kGroup;
     const bool lane_live = sub * 8 < hs;
+    const int off = lane_live ? sub * 8 : 0;
 
-    float* qs = lds;                          // [gqa][hs_pad]
-    float* sc = qs + gqa * hs_pad;            // [gqa][kAttBlock]
-    float* run_max = sc + gqa * kAttBlock;    // [gqa]
-    float* run_sum = run_max + gqa;           // [gqa]
-    float* corr = run_sum + gqa;              // [gqa]
-    float* red = corr + gqa;                  // [nwaves][gqa][hs_pad]
-    float* kv_now = red + nwaves * gqa * hs_pad;  // [2][hs_pad] current position's k and v
-
-    const int chunk = (npos + nsplits - 1) / nsplits;
+    const int chunk = (npos + nsplits - 1) / nsplits;  // <= kItemPositions
     const int t_begin = split * chunk;
     const int t_end = min(npos, t_begin + chunk);
+    const int n = t_end - t_begin;
     const int current = npos - 1;
     const bool has_current = current >= t_begin && current < t_end;
     const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
     const uint16_t* kbase = a.key_cache + head_base;
     const uint16_t* vbase = a.value_cache + head_base;
 
-    constexpr int kMaxPerGroup = 8;
-    int per_group = kAttBlock / ngroups;
-    if (per_group > kMaxPerGroup) per_group = kMaxPerGroup;
-    if (per_group < 1) per_group = 1;
-    const int sub_block = per_group * ngroups;
-
-    // first sub-block's K rows: independent of this token except the current position
-    uintx4 rows8[kMaxPerGroup];
+    uintx4 krow[kRounds], vrow[kRounds];
 #pragma unroll
-    for (int j = 0; j < kMaxPerGroup; ++j) {
+    for (int j = 0; j < kRounds; ++j) {
         const int t = t_begin + grp + j * ngroups;
-        rows8[j] = uintx4{0u, 0u, 0u, 0u};
-        if (j < per_group && t < min(t_end, t_begin + sub_block) && t != current && lane_live)
-            rows8[j] = load16(kbase + static_cast<size_t>(t) * hs + sub * 8);
+        krow[j] = uintx4{0u, 0u, 0u, 0u};
+        vrow[j] = uintx4{0u, 0u, 0u, 0u};
+        if (t < t_end && t != current && lane_live) {
+            krow[j] = load16(kbase + static_cast<size_t>(t) * hs + off);
+            vrow[j] = load16(vbase + static_cast<size_t>(t) * hs + off);
+        }
     }
 
-    // inputs of this token (the block barrier: no wavefront still reads this LDS
-    // area as the activation vector of the previous phase)
+    // this token's q (and, in the last split, k and v of the current position)
     const unsigned tag_in = c.seq(layer, kQkv);
-    __syncthreads();
-    if (hs == hs_pad) {
-        poll_values(c.t.q + static_cast<size_t>(kvh) * gqa * hs, gqa * hs, tag_in, c, [&](int i, float v) { qs[i] = v; });
-    } else {
-        for (int i = tid; i < gqa * hs_pad; i += nthreads) qs[i] = 0.0f;
-        __syncthreads();
-        poll_values(c.t.q + static_cast<size_t>(kvh) * gqa * hs, gqa * hs, tag_in, c,
-                    [&](int i, float v) { qs[(i / hs) * hs_pad + (i % hs)] = v; });
-    }
+    float qv[8], kc[8], vc[8];
     if (has_current) {
-        for (int i = tid; i < 2 * hs_pad; i += nthreads) kv_now[i] = 0.0f;
-        __syncthreads();
-        poll_values(c.t.k + static_cast<size_t>(kvh) * hs, hs, tag_in, c,
-                    [&](int i, float v) { kv_now[i] = f16_bits_to_f32(f32_to_f16_bits(v)); });
-        poll_values(c.t.v + static_cast<size_t>(kvh) * hs, hs, tag_in, c,
-                    [&](int i, float v) { kv_now[hs_pad + i] = f16_bits_to_f32(f32_to_f16_bits(v)); });
-    }
-    if (tid < gqa) {
-        run_max[tid] = -INFINITY;
-        run_sum[tid] = 0.0f;
-    }
-    __syncthreads();
-    c.mark(0);
-
-    // a cache row as 8 fp32 values per lane; the current position comes from LDS
-    auto row_values = [&](uintx4 bits, const float* now, bool is_current, float (&out)[8]) {
-        const half8_t h = as_half8(bits);
+        float in[24];
+        poll_n<24>(
+            [&](int e) -> const u64* {
+                if (e < 8) return c.t.q + static_cast<size_t>(h) * hs + off + e;
+                if (e < 16) return c.t.k + static_cast<size_t>(kvh) * hs + off + (e - 8);
+                return c.t.v + static_cast<size_t>(kvh) * hs + off + (e - 16);
+            },
+            in, tag_in, c);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) out[e] = is_current ? now[sub * 8 + e] : static_cast<float>(h[e]);
-    };
+        for (int e = 0; e < 8; ++e) {
+            qv[e] = lane_live ? in[e] : 0.0f;
+            kc[e] = lane_live ? f16_bits_to_f32(f32_to_f16_bits(in[8 + e])) : 0.0f;
+            vc[e] = lane_live ? f16_bits_to_f32(f32_to_f16_bits(in[16 + e])) : 0.0f;
+        }
+    } else {
+        float in[8];
+        poll_n<8>([&](int e) -> const u64* { return c.t.q + static_cast<size_t>(h) * hs + off + e; }, in, tag_in, c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            qv[e] = lane_live ? in[e] : 0.0f;
+            kc[e] = 0.0f;
+            vc[e] = 0.0f;
+        }
+    }
+    if (first_item) mark(c, io, 1);
+    if (!first_item) io_sync(c.ctl, io);  // the previous item's readers have left sc and red
 
     const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
-    float acc[kMaxGqa][8];
+    float score[kRounds];
 #pragma unroll
-    for (int qh = 0; qh < kMaxGqa; ++qh)
+    for (int j = 0; j < kRounds; ++j) {
+        const int t = t_begin + grp + j * ngroups;
+        const half8_t kh = as_half8(krow[j]);
+        float s = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[qh][e] = 0.0f;
-
-    for (int b0 = t_begin; b0 < t_end; b0 += sub_block) {
-        const int b1 = min(t_end, b0 + sub_block);
-        if (b0 != t_begin) {
-#pragma unroll
-            for (int j = 0; j < kMaxPerGroup; ++j) {
-                const int t = b0 + grp + j * ngroups;
-                rows8[j] = uintx4{0u, 0u, 0u, 0u};
-                if (j < per_group && t < b1 && t != current && lane_live)
-                    rows8[j] = load16(kbase + static_cast<size_t>(t) * hs + sub * 8);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < kMaxPerGroup; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            float kf[8];
-            row_values(rows8[j], kv_now, t == current, kf);
-#pragma unroll
-            for (int qh = 0; qh < kMaxGqa; ++qh) {
-                if (qh < gqa) {
-                    const float* qv = qs + qh * hs_pad + sub * 8;
-                    float s = 0.0f;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) s = fmaf(kf[e], qv[e], s);
-                    s = group_sum<kGroup>(s);
-                    if (j < per_group && t < b1 && sub == 0) sc[qh * kAttBlock + (t - b0)] = s * scale;
-                }
-            }
-        }
-        // V rows travel while the softmax is formed
-#pragma unroll
-        for (int j = 0; j < kMaxPerGroup; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            rows8[j] = uintx4{0u, 0u, 0u, 0u};
-            if (j < per_group && t < b1 && t != current && lane_live)
-                rows8[j] = load16(vbase + static_cast<size_t>(t) * hs + sub * 8);
-        }
-        __syncthreads();
-        for (int qh = wave; qh < gqa; qh += nwaves) {
-            float* row = sc + qh * kAttBlock;
-            const int n = b1 - b0;
-            float m = -INFINITY;
-            for (int i = lane_id(); i < n; i += kWave) m = fmaxf(m, row[i]);
-            m = wave_max(m);
-            const float m_old = run_max[qh];
-            const float m_new = fmaxf(m_old, m);
-            float lsum = 0.0f;
-            for (int i = lane_id(); i < n; i += kWave) {
-                const float p = expf(row[i] - m_new);
-                row[i] = p;
-                lsum += p;
-            }
-            lsum = wave_sum(lsum);
-            if (lane_id() == 0) {
-                const float cf = (m_old == -INFINITY) ? 0.0f : expf(m_old - m_new);
-                corr[qh] = cf;
-                run_sum[qh] = run_sum[qh] * cf + lsum;
-                run_max[qh] = m_new;
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int qh = 0; qh < kMaxGqa; ++qh) {
-            if (qh < gqa) {
-                const float cf = corr[qh];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[qh][e] *= cf;
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < kMaxPerGroup; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            if (j < per_group && t < b1 && lane_live) {
-                float vf[8];
-                row_values(rows8[j], kv_now + hs_pad, t == current, vf);
-#pragma unroll
-                for (int qh = 0; qh < kMaxGqa; ++qh) {
-                    if (qh < gqa) {
-                        const float p = sc[qh * kAttBlock + (t - b0)];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) acc[qh][e] = fmaf(vf[e], p, acc[qh][e]);
-                    }
-                }
-            }
-        }
-        __syncthreads();
+        for (int e = 0; e < 8; ++e) s = fmaf((t == current) ? kc[e] : static_cast<float>(kh[e]), qv[e], s);
+        s = group_sum<kGroup>(s) * scale;
+        score[j] = s;
+        if (t < t_end && sub == 0) l.sc[t - t_begin] = s;
     }
+    io_sync(c.ctl, io);
+    if (first_item) mark(c, io, 2);
+    // every wavefront: maximum and sum of exponentials over the item's scores
+    float m = -INFINITY;
+    for (int i = lane_id(); i < n; i += kWave) m = fmaxf(m, l.sc[i]);
+    m = wave_max(m);
+    float lsum = 0.0f;
+    for (int i = lane_id(); i < n; i += kWave) lsum += expf(l.sc[i] - m);
+    lsum = wave_sum(lsum);
 
-    // per-group partial outputs -> wavefront (lane exchange) -> workgroup (LDS, wave order)
+    float acc[8];
 #pragma unroll
-    for (int qh = 0; qh < kMaxGqa; ++qh) {
-        if (qh < gqa) {
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float v = acc[qh][e];
+    for (int j = 0; j < kRounds; ++j) {
+        const int t = t_begin + grp + j * ngroups;
+        if (t < t_end) {
+            const float p = expf(score[j] - m);
+            const half8_t vh = as_half8(vrow[j]);
 #pragma unroll
-                for (int off = kGroup; off < kWave; off <<= 1) v += __shfl_xor(v, off);
-                acc[qh][e] = v;
-            }
-            if (lane_id() < kGroup) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) red[(wave * gqa + qh) * hs_pad + sub * 8 + e] = acc[qh][e];
-            }
+            for (int e = 0; e < 8; ++e) acc[e] = fmaf((t == current) ? vc[e] : static_cast<float>(vh[e]), p, acc[e]);
         }
     }
-    __syncthreads();
+    // groups of one wavefront by lane exchange, wavefronts through LDS
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float v = acc[e];
+#pragma unroll
+        for (int o = kGroup; o < kWave; o <<= 1) v += __shfl_xor(v, o);
+        acc[e] = v;
+    }
+    if (lane_id() < kGroup) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) l.red[io.iw * kMaxHeadPad + sub * 8 + e] = acc[e];
+    }
+    io_sync(c.ctl, io);
+    if (first_item) mark(c, io, 3);
     const unsigned tag_out = c.seq(layer, kAtt);
-    const int stride = hs + 2;
-    if (nsplits == 1) {
-        for (int i = tid; i < gqa * hs; i += nthreads) {
-            const int qh = i / hs, e = i - qh * hs;
-            float o = 0.0f;
-            for (int w = 0; w < nwaves; ++w) o += red[(w * gqa + qh) * hs_pad + e];
-            publish(c.t.xb + static_cast<size_t>(kvh * gqa + qh) * hs + e, o / run_sum[qh], tag_out);
-        }
-        return;
-    }
-    for (int i = tid; i < gqa * hs; i += nthreads) {
-        const int qh = i / hs, e = i - qh * hs;
+    if (io.it < hs) {
         float o = 0.0f;
-        for (int w = 0; w < nwaves; ++w) o += red[(w * gqa + qh) * hs_pad + e];
-        u64* part = c.t.part + (static_cast<size_t>(kvh * gqa + qh) * a.max_splits + split) * stride;
-        publish(part + e, o, tag_out);
-        if (e == 0) {
-            publish(part + hs, run_max[qh], tag_out);
-            publish(part + hs + 1, run_sum[qh], tag_out);
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) o += l.red[w * kMaxHeadPad + io.it];
+        if (nsplits == 1) {
+            publish(c.t.xb + static_cast<size_t>(h) * hs + io.it, o / lsum, tag_out);
+        } else {
+            u64* part = c.t.part + (static_cast<size_t>(h) * c.t.splits_cap + split) * (hs + 2);
+            publish(part + io.it, o, tag_out);
+            if (io.it == 0) {
+                publish(part + hs, m, tag_out);
+                publish(part + hs + 1, lsum, tag_out);
+            }
         }
     }
+    (void)hs_pad;
 }
 
-// Combine the context splits of one KV head: collect every split's (output,
-// max, sum), rescale to the common maximum and normalise.  Runs after the
-// workgroup has published all of its own partials, so a workgroup waiting here
-// never holds back a partial another combiner needs.
-__device__ __forceinline__ void df_attention_combine(Ctx& c, int layer, int kvh, int nsplits, float* gathered) {
+// Combine the context splits of head h: collect every split's (output, max,
+// sum), rescale to the common maximum and normalise.  Runs after the workgroup
+// has published all of its own partials, so a workgroup waiting here never
+// holds back a partial another combiner needs.
+__device__ __forceinline__ void att_combine(Ctx& c, Io& io, const Lds& l, int layer, int h, int nsplits) {
     const DecodeArgs& a = c.a;
-    const int hs = a.head_size, gqa = a.gqa;
-    const int stride = hs + 2;
-    const int tid = static_cast<int>(threadIdx.x), nthreads = static_cast<int>(blockDim.x);
+    const int hs = a.head_size, stride = hs + 2;
     const unsigned tag_out = c.seq(layer, kAtt);
-    __syncthreads();
-    for (int qh = 0; qh < gqa; ++qh) {  // gathered: [gqa][max_splits][stride]
-        const size_t first = static_cast<size_t>(kvh * gqa + qh) * a.max_splits * stride;
-        float* dst = gathered + static_cast<size_t>(qh) * a.max_splits * stride;
-        poll_values(c.t.part + first, nsplits * stride, tag_out, c, [&](int i, float v) { dst[i] = v; });
-    }
-    __syncthreads();
-    for (int i = tid; i < gqa * hs; i += nthreads) {
-        const int qh = i / hs, e = i - qh * hs;
-        const float* basep = gathered + static_cast<size_t>(qh) * a.max_splits * stride;
+    io_sync(c.ctl, io);  // earlier readers of gather have left
+    const u64* src = c.t.part + static_cast<size_t>(h) * c.t.splits_cap * stride;
+    poll_values(src, nsplits * stride, tag_out, c, io, [&](int i, float v) { l.gather[i] = v; });
+    io_sync(c.ctl, io);
+    if (io.it < hs) {
         float top = -INFINITY;
-        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, basep[s * stride + hs]);
+        for (int s = 0; s < nsplits; ++s) top = fmaxf(top, l.gather[s * stride + hs]);
         float o = 0.0f, lsum = 0.0f;
         for (int s = 0; s < nsplits; ++s) {
-            const float ms = basep[s * stride + hs];
+            const float ms = l.gather[s * stride + hs];
             const float wgt = (ms == -INFINITY) ? 0.0f : expf(ms - top);
-            o += basep[s * stride + e] * wgt;
-            lsum += basep[s * stride + hs + 1] * wgt;
+            o += l.gather[s * stride + io.it] * wgt;
+            lsum += l.gather[s * stride + hs + 1] * wgt;
         }
-        publish(c.t.xb + static_cast<size_t>(kvh * gqa + qh) * hs + e, o / lsum, tag_out);
+        publish(c.t.xb + static_cast<size_t>(h) * hs + io.it, o / lsum, tag_out);
     }
 }
 
-__device__ __forceinline__ void df_attention(Ctx& c, const Lds& l, int layer, int wg, int nwg) {
+__device__ __forceinline__ int item_splits(int npos, int cap) {
+    int s = (npos + kItemPositions - 1) / kItemPositions;
+    return s < 1 ? 1 : (s > cap ? cap : s);
+}
+
+__device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int layer) {
     const DecodeArgs& a = c.a;
     const int npos = c.pos + 1;
-    const int nsplits = active_splits(npos, a.max_splits);
-    const int items = a.n_kv_heads * nsplits;
+    const int nsplits = item_splits(npos, c.t.splits_cap);
+    const int items = a.n_heads * nsplits;
     const int hs = a.head_size;
-    bool marked = false;
-    for (int item = wg; item < items; item += nwg) {
-        const int kvh = item / nsplits, split = item - kvh * nsplits;
-        if (hs <= 8) df_attention_item<1>(c, layer, kvh, split, nsplits, npos, l.xs);
-        else if (hs <= 16) df_attention_item<2>(c, layer, kvh, split, nsplits, npos, l.xs);
-        else if (hs <= 32) df_attention_item<4>(c, layer, kvh, split, nsplits, npos, l.xs);
-        else if (hs <= 64) df_attention_item<8>(c, layer, kvh, split, nsplits, npos, l.xs);
-        else df_attention_item<16>(c, layer, kvh, split, nsplits, npos, l.xs);
-        __syncthreads();
-        marked = true;
+    bool first = true;
+    mark(c, io, 0);
+    for (int item = c.wg; item < items; item += c.nwg) {
+        const int h = item / nsplits, split = item - h * nsplits;
+        if (hs <= 8) att_item<1>(c, io, l, layer, h, split, nsplits, npos, first);
+        else if (hs <= 16) att_item<2>(c, io, l, layer, h, split, nsplits, npos, first);
+        else if (hs <= 32) att_item<4>(c, io, l, layer, h, split, nsplits, npos, first);
+        else if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first);
+        else att_item<16>(c, io, l, layer, h, split, nsplits, npos, first);
+        first = false;
     }
     if (nsplits > 1) {
-        for (int item = wg; item < items; item += nwg) {
-            const int kvh = item / nsplits, split = item - kvh * nsplits;
-            if (split == 0) df_attention_combine(c, layer, kvh, nsplits, l.xs);
+        for (int item = c.wg; item < items; item += c.nwg) {
+            const int h = item / nsplits, split = item - h * nsplits;
+            if (split == 0) att_combine(c, io, l, layer, h, nsplits);
         }
     }
-    if (!marked) c.mark(0);
-    c.mark(1);
+    mark(c, io, 4);
     ++c.phase_index;
 }
 
 // ---------------------------------------------------------------------------
-// Classifier + sampler
+// Classifier + sampler (exchange wavefronts)
 // ---------------------------------------------------------------------------
 
-// Workgroup w owns the contiguous vocabulary rows [w*rows_per_wg, ...): their
-// logits stay in LDS, the sampler's per-row work happens there, and only three
-// numbers per workgroup (maximum, its lowest index, sum of exponentials) are
-// exchanged.  The workgroup whose slice of the CDF contains the draw (or that
-// holds the first maximum, for temperature 0) finishes the token
-// (model.cpp:256-303, main.cpp:200-208).
-template <bool kF16>
-__device__ __forceinline__ void df_classify_sample(Ctx& c, const Lds& l, int wg, int nwg, int rows_per_wg) {
-    constexpr int kRows = 2;
+// Workgroup w owns the contiguous vocabulary rows [w*cls, ...): their logits
+// stay in LDS, the sampler's per-row work happens there, and only three numbers
+// per workgroup (maximum, its lowest index, sum of exponentials) are exchanged.
+// The workgroup whose slice of the CDF contains the draw (or that holds the
+// first maximum, for temperature 0) finishes the token (model.cpp:256-303,
+// main.cpp:200-208).
+__device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l) {
     const DecodeArgs& a = c.a;
-    const int wbytes = kF16 ? 2 : 4;
-    const int vocab = a.vocab, dim = a.dim;
-    const int r0 = min(vocab, wg * rows_per_wg), r1 = min(vocab, r0 + rows_per_wg);
-    const int n = r1 - r0;
-    const int ntiles = (n + kRows - 1) / kRows;
-    const int tid = static_cast<int>(threadIdx.x), nthreads = static_cast<int>(blockDim.x);
-    float* lg = l.local;
-    auto row_ptr = [&](int tile, int r) -> const char* {
-        int g = r0 + tile * kRows + r;
-        if (g >= vocab) g = vocab - 1;
-        return a.wcls + static_cast<size_t>(g) * dim * wbytes;
-    };
-    auto pre = [&]() {
-        stage_norm(l.xraw, l.xs, c.t.x, nullptr, dim, c.seq(a.n_layers - 1, kDown), a.rms_final, c);
-        c.mark(0);
-    };
-    auto emit = [&](int tile, int r, float mine, float) {
-        const int i = tile * kRows + r;
-        if (i < n) {
-            lg[i] = mine;
-            a.logits[r0 + i] = mine;  // raw logits stay readable after the token
-        }
-    };
-    gemv_phase<kF16, kRows, 4>(ntiles, dim, l.xs, wave_index(), kWaves, row_ptr, emit, pre);
-    __syncthreads();
-    c.mark(1);
+    Control& ctl = c.ctl;
+    const int vocab = a.vocab, dim = a.dim, wg = c.wg, nwg = c.nwg;
+    const int it = io.it;
+    mark(c, io, 0);
+    stage_norm(c, io, l, c.t.x, nullptr, dim, c.seq(a.n_layers - 1, kDown), a.rms_final);
+    mark(c, io, 2);
+    wait_gemv(ctl, io, 4 * a.n_layers);
+    mark(c, io, 3);
+    const int r0 = min(vocab, wg * c.b.cls);
+    const int n = block_rows(vocab, c.b.cls, wg);
+    const int r1 = r0 + n;
+    float* lg = l.results;
+    for (int i = it; i < n; i += kIoThreads) a.logits[r0 + i] = lg[i];  // raw logits stay readable after the token
+    mark(c, io, 4);
     ++c.phase_index;
 
-    // ---- sampler on the local rows ----
-    __shared__ float s_val[16];
-    __shared__ int s_idx[16];
-    __shared__ float s_scratch[16];
-    __shared__ int s_target, s_token;
     const float temperature = c.temperature, penalty = c.penalty;
     const int history_len = c.history_len;
     if (penalty > 1.0f && history_len > 0) {  // model.cpp:258-270, once per occurrence
-        for (int i = tid; i < history_len; i += nthreads) {
+        io_sync(ctl, io);
+        for (int i = it; i < history_len; i += kIoThreads) {
             const int tok = a.history[i];
             if (tok < r0 || tok >= r1) continue;
             const int count = smp::owned_count(a.history, history_len, i);
             if (count > 0) lg[tok - r0] = smp::penalise(lg[tok - r0], penalty, count);
         }
-        __syncthreads();
+        io_sync(ctl, io);
     }
     ArgMax best{-INFINITY, 0x7fffffff};
-    for (int i = tid; i < n; i += nthreads) {
+    for (int i = it; i < n; i += kIoThreads) {
         float v = lg[i];
         if (temperature != 0.0f) v = v / temperature;  // model.cpp:286-288
         lg[i] = v;
         best = argmax_better(best, ArgMax{v, r0 + i});
     }
     best = wave_argmax(best);
-    if (lane_id() == 0) {
-        s_val[tid / kWave] = best.v;
-        s_idx[tid / kWave] = best.i;
+    {
+        float* sv = ctl.redv[io.parity];
+        int* si = ctl.redi[io.parity];
+        if (lane_id() == 0) {
+            sv[io.iw] = best.v;
+            si[io.iw] = best.i;
+        }
+        io_sync(ctl, io);
+        best = ArgMax{lds_ld(sv), lds_ld(si)};
+        for (int w = 1; w < kIoWaves; ++w)
+            best = argmax_better(best, ArgMax{lds_ld(sv + w), lds_ld(si + w)});
     }
-    __syncthreads();
-    ArgMax mine{s_val[0], s_idx[0]};
-    for (int w = 1; w < kWaves; ++w) mine = argmax_better(mine, ArgMax{s_val[w], s_idx[w]});
+    const ArgMax mine = best;
     float local_sum = 0.0f;
     if (temperature != 0.0f) {
         float part = 0.0f;
-        for (int i = tid; i < n; i += nthreads) {
+        for (int i = it; i < n; i += kIoThreads) {
             const float e = expf(lg[i] - mine.v);  // ops.cpp:65, against the local maximum
             lg[i] = e;
             part += e;
         }
-        local_sum = block_sum(part, s_scratch);
+        local_sum = io_sum(ctl, io, part);
     }
     const unsigned tag = c.seq_stats();
-    if (tid == 0) {
+    if (it == 0) {
         publish(c.t.stats + wg * 4 + 0, mine.v, tag);
         publish(c.t.stats + wg * 4 + 1, local_sum, tag);
         publish(c.t.stats + wg * 4 + 2, __int_as_float(mine.i), tag);
         publish(c.t.stats + wg * 4 + 3, 0.0f, tag);
     }
     // every workgroup reads all statistics and reaches the same decision
-    float* st_max = l.xs;            // [nwg]
+    float* st_max = l.xs;            // [nwg]  (the streaming wavefronts are done with xs)
     float* st_sum = l.xs + nwg;      // [nwg]
     float* st_arg = l.xs + 2 * nwg;  // [nwg] (int bits)
-    float* st_cum = l.xs + 3 * nwg;  // [nwg] inclusive mass
-    __syncthreads();
-    poll_values(c.t.stats, nwg * 4, tag, c, [&](int i, float v) {
+    float* st_cum = l.xs + 3 * nwg;  // [nwg] mass before the workgroup
+    poll_values(c.t.stats, nwg * 4, tag, c, io, [&](int i, float v) {
         const int w = i >> 2, f = i & 3;
         if (f == 0) st_max[w] = v;
         else if (f == 1) st_sum[w] = v;
         else if (f == 2) st_arg[w] = v;
     });
-    __syncthreads();
-    c.mark(0);
+    io_sync(ctl, io);
+    mark(c, io, 2);
     if (temperature == 0.0f) {  // model.cpp:272-283: first maximum wins
-        if (tid == 0) {
+        if (it == 0) {
             ArgMax g{-INFINITY, 0x7fffffff};
             int target = 0;
             for (int w = 0; w < nwg; ++w) {
@@ -678,23 +888,23 @@ __device__ __forceinline__ void df_classify_sample(Ctx& c, const Lds& l, int wg,
                     target = w;
                 }
             }
-            s_target = target;
-            s_token = (g.i == 0x7fffffff) ? 0 : g.i;
+            ctl.target = target;
+            ctl.token = (g.i == 0x7fffffff) ? 0 : g.i;
         }
-        __syncthreads();
+        io_sync(ctl, io);
     } else {
         float top = -INFINITY;
-        for (int w = tid; w < nwg; w += nthreads) top = fmaxf(top, st_max[w]);
-        top = block_max(top, s_scratch);
+        for (int w = it; w < nwg; w += kIoThreads) top = fmaxf(top, st_max[w]);
+        top = io_max(ctl, io, top);
         float mass = 0.0f;
-        for (int w = tid; w < nwg; w += nthreads) {
-            const float m = (st_max[w] == -INFINITY) ? 0.0f : st_sum[w] * expf(st_max[w] - top);
-            st_cum[w] = m;
-            mass += m;
+        for (int w = it; w < nwg; w += kIoThreads) {
+            const float mw = (st_max[w] == -INFINITY) ? 0.0f : st_sum[w] * expf(st_max[w] - top);
+            st_cum[w] = mw;
+            mass += mw;
         }
-        const float total = block_sum(mass, s_scratch);
+        const float total = io_sum(ctl, io, mass);
         const float r = c.r;
-        if (tid == 0) {
+        if (it == 0) {
             // sequential in workgroup order = index order of the CDF (model.cpp:294-301)
             float cum = 0.0f;
             int target = -1;
@@ -704,24 +914,23 @@ __device__ __forceinline__ void df_classify_sample(Ctx& c, const Lds& l, int wg,
                 st_cum[w] = before;
                 if (target < 0 && r < cum) target = w;
             }
-            s_target = target;
-            s_token = vocab - 1;  // model.cpp:302 when no bucket is reached
+            ctl.target = target;
+            ctl.token = vocab - 1;  // model.cpp:302 when no bucket is reached
         }
-        __syncthreads();
-        if (s_target == wg) {
+        io_sync(ctl, io);
+        if (lds_ld(&ctl.target) == wg) {
             // inside the target workgroup: p_i = e_i * exp(m_w - top) / total, running sum in index order
             const float f = expf(mine.v - top) / total;
             const float before = st_cum[wg];
-            const int per_thread = (n + nthreads - 1) / nthreads;
-            const int begin = tid * per_thread, end = min(n, begin + per_thread);
+            const int per_thread = (n + kIoThreads - 1) / kIoThreads;
+            const int begin = it * per_thread, end = min(n, begin + per_thread);
             float chunk_sum = 0.0f;
             for (int i = begin; i < end; ++i) chunk_sum += lg[i] * f;
             const float incl = wave_inclusive_scan(chunk_sum);
-            __shared__ float wave_tot[16];
-            if (lane_id() == kWave - 1) wave_tot[tid / kWave] = incl;
-            __syncthreads();
+            if (lane_id() == kWave - 1) ctl.wave_tot[io.iw] = incl;
+            io_sync(ctl, io);
             float offset = before;
-            for (int w = 0; w < tid / kWave; ++w) offset += wave_tot[w];
+            for (int w = 0; w < io.iw; ++w) offset += lds_ld(&ctl.wave_tot[w]);
             offset += incl - chunk_sum;
             float run = 0.0f;
             int found = 0x7fffffff;
@@ -730,25 +939,37 @@ __device__ __forceinline__ void df_classify_sample(Ctx& c, const Lds& l, int wg,
                 if (found == 0x7fffffff && r < offset + run) found = r0 + i;
             }
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) found = min(found, __shfl_xor(found, off));
-            __shared__ int wave_found[16];
-            if (lane_id() == 0) wave_found[tid / kWave] = found;
-            __syncthreads();
-            if (tid == 0) {
-                int f0 = wave_found[0];
-                for (int w = 1; w < kWaves; ++w) f0 = min(f0, wave_found[w]);
-                s_token = (f0 == 0x7fffffff) ? r1 - 1 : f0;  // rounding left the bucket short: its last row
+            for (int o = 32; o >= 1; o >>= 1) found = min(found, __shfl_xor(found, o));
+            if (lane_id() == 0) ctl.wave_found[io.iw] = found;
+            io_sync(ctl, io);
+            if (it == 0) {
+                int f0 = lds_ld(&ctl.wave_found[0]);
+                for (int w = 1; w < kIoWaves; ++w) f0 = min(f0, lds_ld(&ctl.wave_found[w]));
+                ctl.token = (f0 == 0x7fffffff) ? r1 - 1 : f0;  // rounding left the bucket short: its last row
             }
-            __syncthreads();
         }
     }
     // Exactly one workgroup finishes the token: the target, or (no bucket reached) the last one.
-    const bool finisher = (s_target == wg) || (s_target < 0 && wg == nwg - 1);
-    if (finisher && tid == 0) {
-        finish_token(a, s_token, 0u);
+    if (it == 0) {
+        const int target = lds_ld(&ctl.target);
+        const bool finisher = (target == wg) || (target < 0 && wg == nwg - 1);
+        if (finisher) finish_token(a, lds_ld(&ctl.token), 0u);
     }
-    c.mark(1);
+    mark(c, io, 4);
     ++c.phase_index;
+}
+
+template <bool kF16>
+__device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
+    const DecodeArgs& a = c.a;
+    for (int layer = 0; layer < a.n_layers; ++layer) {
+        io_qkv(c, io, l, layer);
+        io_attention(c, io, l, layer);
+        io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.t.xb, c.seq(layer, kAtt), c.seq(layer, kOproj));
+        io_gateup(c, io, l, layer);
+        io_proj(c, io, l, 4 * layer + kGDown, c.b.down, a.hidden, c.t.hb, c.seq(layer, kGateUp), c.seq(layer, kDown));
+    }
+    io_classify_sample(c, io, l);
 }
 
 // ---------------------------------------------------------------------------
@@ -756,27 +977,34 @@ __device__ __forceinline__ void df_classify_sample(Ctx& c, const Lds& l, int wg,
 // ---------------------------------------------------------------------------
 
 template <bool kF16>
-__global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagged t, int rows_per_wg,
-                                                              int lds_xs_floats) {
+__global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagged t, Blocks b,
+                                                              const uint4* __restrict__ row_lists, int row_list_stride) {
     extern __shared__ __align__(16) float lds[];
+    __shared__ Control ctl;
     const int wg = blockIdx.x, nwg = gridDim.x;
     const int dim_pad = (a.dim + 7) & ~7;
-    Lds l{lds, lds + dim_pad, lds + dim_pad + lds_xs_floats};
-    const StepParams* sp = a.step;
-    Ctx c{a, t, t.base, (wg == 0) ? a.trace : nullptr, 0u,
-          sp->token, sp->pos, sp->history_len, sp->temperature, sp->penalty, step_uniform(a)};
-    if (c.trace && threadIdx.x == 0) c.trace[2u * phases_per_token(a.n_layers)] = wall_clock64();
-    const int wbytes = kF16 ? 2 : 4;
-    for (int layer = 0; layer < a.n_layers; ++layer) {
-        df_qkv<kF16>(c, l, layer, wg, nwg);
-        df_attention(c, l, layer, wg, nwg);
-        df_proj<kF16, 2, 4>(c, l, a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes, a.dim, a.dim, t.xb,
-                            c.seq(layer, kAtt), c.seq(layer, kOproj), wg, nwg);
-        df_gateup<kF16>(c, l, layer, wg, nwg);
-        df_proj<kF16, 1, 8>(c, l, a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden, t.hb,
-                            c.seq(layer, kGateUp), c.seq(layer, kDown), wg, nwg);
+    Lds l;
+    l.xraw = lds;
+    l.xs = l.xraw + dim_pad;
+    l.results = l.xs + b.xs_floats;
+    l.sc = l.results + b.results_floats;
+    l.red = l.sc + kItemPositions;
+    l.gather = l.red + kIoWaves * kMaxHeadPad;
+    for (unsigned i = threadIdx.x; i < sizeof(Control) / sizeof(unsigned); i += blockDim.x)
+        reinterpret_cast<unsigned*>(&ctl)[i] = 0u;
+    __syncthreads();  // the only workgroup-wide barrier: the two kinds of wavefronts part ways here
+    const int wave = wave_index();
+    if (wave < kGemvWaves) {
+        gemv_role<kF16>(a, ctl, row_lists + static_cast<size_t>(wg * kGemvWaves + wave) * row_list_stride, wave, l.xs,
+                        l.results, (wg == 0 && wave == 0) ? a.trace : nullptr);
+    } else {
+        const StepParams* sp = a.step;
+        Ctx c{a, t, b, ctl, t.base, (wg == 0) ? a.trace : nullptr, 0u,
+              sp->token, sp->pos, sp->history_len, sp->temperature, sp->penalty, step_uniform(a), wg, nwg};
+        Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
+        if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
+        io_role<kF16>(c, io, l);
     }
-    df_classify_sample<kF16>(c, l, wg, nwg, rows_per_wg);
 }
 
 }  // namespace df
@@ -787,10 +1015,14 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
 
 namespace {
 
+int splits_cap_for(const lpp_model* m) {
+    const int s = (m->cfg.seq_len + df::kItemPositions - 1) / df::kItemPositions;
+    return s < 1 ? 1 : s;
+}
+
 struct Plan {
     int grid;
-    int rows_per_wg;
-    int xs_floats;
+    df::Blocks blocks;
     size_t lds_bytes;
 };
 
@@ -798,22 +1030,34 @@ Plan plan_for(const lpp_model* m) {
     const lpp_config& c = m->cfg;
     Plan p;
     p.grid = compute_units();
-    const int per = (c.vocab_size + p.grid - 1) / p.grid;
-    p.rows_per_wg = (per + 1) & ~1;
+    auto per = [&](int total) { return (total + p.grid - 1) / p.grid; };
+    df::Blocks& b = p.blocks;
+    b.qkv = (per(c.dim + 2 * m->kv_dim) + 1) & ~1;  // RoPE pairs stay inside one workgroup
+    b.o = per(c.dim);
+    b.gu = per(c.hidden_dim);
+    b.down = per(c.dim);
+    b.cls = per(c.vocab_size);
     const int dim_pad = (c.dim + 7) & ~7;
     int xs = (c.hidden_dim + 7) & ~7;
     if (dim_pad > xs) xs = dim_pad;
-    int hs_pad = 8;  // lanes per position * 8, as df_attention_item rounds it
-    while (hs_pad < m->head_size) hs_pad *= 2;
-    const int nwaves = df::kThreads / dev::kWave;
-    const int att = m->gqa * hs_pad + m->gqa * ph::kAttBlock + 3 * m->gqa + nwaves * m->gqa * hs_pad  // q, scores, reduce
-                    + 2 * hs_pad                                                                   // current k, v
-                    + m->gqa * m->max_splits * (m->head_size + 2);                                 // split gather
-    if (att > xs) xs = att;
-    if (4 * p.grid > xs) xs = 4 * p.grid;
-    p.xs_floats = xs;
-    p.lds_bytes = static_cast<size_t>(dim_pad + xs + ((p.rows_per_wg + 7) & ~7)) * sizeof(float);
+    if (4 * p.grid > xs) xs = 4 * p.grid;  // sampler tables
+    b.xs_floats = xs;
+    int rows = b.qkv;
+    if (b.o > rows) rows = b.o;
+    if (2 * b.gu > rows) rows = 2 * b.gu;
+    if (b.down > rows) rows = b.down;
+    if (b.cls > rows) rows = b.cls;
+    b.results_floats = (rows + 7) & ~7;
+    b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
+    p.lds_bytes = static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + df::kItemPositions +
+                                      df::kIoWaves * df::kMaxHeadPad + b.gather_floats) * sizeof(float);
     return p;
+}
+
+size_t tagged_count(const lpp_model* m, int grid_cap) {
+    const lpp_config& c = m->cfg;
+    return static_cast<size_t>(c.dim) * 3 + static_cast<size_t>(m->kv_dim) * 2 + c.hidden_dim +
+           static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2) + 4u * grid_cap;
 }
 
 df::Tagged tagged_of(const lpp_model* m) {
@@ -826,28 +1070,107 @@ df::Tagged tagged_of(const lpp_model* m) {
     t.v = p;            p += m->kv_dim;
     t.xb = p;           p += c.dim;
     t.hb = p;           p += c.hidden_dim;
-    t.part = p;         p += static_cast<size_t>(c.n_heads) * m->max_splits * (m->head_size + 2);
+    t.part = p;         p += static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2);
     t.stats = p;
+    t.splits_cap = splits_cap_for(m);
     t.base = m->df_base;
     t.abort = m->sync_words + 65;
     t.spin_limit = m->spin_limit;
     return t;
 }
 
+constexpr int kGridCap = 1024;  // workgroups the statistics table has room for
+
+// Row lists of the streaming wavefronts: [workgroup][wavefront][stride] entries,
+// each list closed by two entries without kRowValid that point at a readable row.
+lpp_status build_row_lists(lpp_model* m, const Plan& p) {
+    const lpp_config& c = m->cfg;
+    const df::Blocks& b = p.blocks;
+    const int L = c.n_layers, dim = c.dim, hidden = c.hidden_dim, kv = m->kv_dim;
+    const size_t wb = c.weight_precision == LPP_WEIGHT_FP16 ? 2 : 4;
+    const size_t rb_dim = static_cast<size_t>(dim) * wb, rb_hidden = static_cast<size_t>(hidden) * wb;
+    auto base = [&](int t) { return reinterpret_cast<unsigned long long>(m->w[t]); };
+    auto block_rows = [](int total, int block, int wg) {
+        const int n = total - wg * block;
+        return n < 0 ? 0 : (n > block ? block : n);
+    };
+    auto own = [](int nrows, int j) { return nrows > j ? (nrows - j + df::kGemvWaves - 1) / df::kGemvWaves : 0; };
+    int longest = 0;
+    for (int wg = 0; wg < p.grid; ++wg)
+        for (int j = 0; j < df::kGemvWaves; ++j) {
+            const int n = L * (own(block_rows(dim + 2 * kv, b.qkv, wg), j) + own(block_rows(dim, b.o, wg), j) +
+                               own(block_rows(2 * hidden, 2 * b.gu, wg), j) + own(block_rows(dim, b.down, wg), j)) +
+                          own(block_rows(c.vocab_size, b.cls, wg), j);
+            if (n > longest) longest = n;
+        }
+    const int stride = longest + 2;
+    LPP_REQUIRE(4 * L + 1 <= static_cast<int>(df::kRowPhaseMask), "persistent decode: too many layers for the row lists");
+    LPP_REQUIRE(b.cls <= static_cast<int>(df::kRowLocalMask) && 2 * b.gu <= static_cast<int>(df::kRowLocalMask),
+                "persistent decode: row block too large for the row lists");
+    std::vector<df::RowEntry> host(static_cast<size_t>(p.grid) * df::kGemvWaves * stride);
+    for (int wg = 0; wg < p.grid; ++wg)
+        for (int j = 0; j < df::kGemvWaves; ++j) {
+            df::RowEntry* out = host.data() + (static_cast<size_t>(wg) * df::kGemvWaves + j) * stride;
+            int n = 0;
+            auto phase_rows = [&](int phase, int nrows, bool wide, auto row_address) {
+                const int mine = own(nrows, j);
+                for (int i = 0; i < mine; ++i) {
+                    const int r = j + i * df::kGemvWaves;
+                    out[n].ptr = row_address(r);
+                    out[n].meta = static_cast<unsigned>(r) | (static_cast<unsigned>(phase) << df::kRowPhaseShift) |
+                                  (wide ? df::kRowWide : 0u) | (i + 1 == mine ? df::kRowLast : 0u) | df::kRowValid;
+                    out[n].pad = 0;
+                    ++n;
+                }
+            };
+            for (int l = 0; l < L; ++l) {
+                phase_rows(4 * l + df::kGQkv, block_rows(dim + 2 * kv, b.qkv, wg), false, [&](int r) {
+                    const int g = wg * b.qkv + r;
+                    if (g < dim) return base(LPP_T_WQ) + (static_cast<size_t>(l) * dim + g) * rb_dim;
+                    if (g < dim + kv) return base(LPP_T_WK) + (static_cast<size_t>(l) * kv + (g - dim)) * rb_dim;
+                    return base(LPP_T_WV) + (static_cast<size_t>(l) * kv + (g - dim - kv)) * rb_dim;
+                });
+                phase_rows(4 * l + df::kGO, block_rows(dim, b.o, wg), false,
+                           [&](int r) { return base(LPP_T_WO) + (static_cast<size_t>(l) * dim + wg * b.o + r) * rb_dim; });
+                // local row 2u = gate row of hidden unit u, 2u + 1 = its up row
+                phase_rows(4 * l + df::kGGateUp, block_rows(2 * hidden, 2 * b.gu, wg), false, [&](int r) {
+                    return base((r & 1) ? LPP_T_W3 : LPP_T_W1) + (static_cast<size_t>(l) * hidden + wg * b.gu + (r >> 1)) * rb_dim;
+                });
+                phase_rows(4 * l + df::kGDown, block_rows(dim, b.down, wg), true, [&](int r) {
+                    return base(LPP_T_W2) + (static_cast<size_t>(l) * dim + wg * b.down + r) * rb_hidden;
+                });
+            }
+            phase_rows(4 * L, block_rows(c.vocab_size, b.cls, wg), false,
+                       [&](int r) { return base(LPP_T_WCLS) + (static_cast<size_t>(wg) * b.cls + r) * rb_dim; });
+            for (int k = 0; k < 2; ++k) {
+                out[n].ptr = base(LPP_T_WCLS);
+                out[n].meta = 0;
+                out[n].pad = 0;
+                ++n;
+            }
+        }
+    lpp_free(m->df_rows);
+    m->df_rows = nullptr;
+    void* d = nullptr;
+    LPP_TRY(lpp_malloc(&d, host.size() * sizeof(df::RowEntry)));
+    m->df_rows = d;
+    m->df_row_stride = stride;
+    LPP_TRY(lpp_memcpy_h2d(d, host.data(), host.size() * sizeof(df::RowEntry)));
+    for (int t = 0; t < LPP_T_COUNT; ++t) m->df_rows_key[t] = m->w[t];
+    return LPP_OK;
+}
+
 }  // namespace
 
-size_t dataflow_tagged_bytes(const lpp_model* m) {
-    const lpp_config& c = m->cfg;
-    const size_t n = static_cast<size_t>(c.dim) * 3 + static_cast<size_t>(m->kv_dim) * 2 + c.hidden_dim +
-                     static_cast<size_t>(c.n_heads) * m->max_splits * (m->head_size + 2) + 4u * 1024u;
-    return n * sizeof(df::u64);
-}
+size_t dataflow_tagged_bytes(const lpp_model* m) { return tagged_count(m, kGridCap) * sizeof(df::u64); }
 
 template <bool kF16>
 static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
     const Plan p = plan_for(m);
     if (m->persist_grid == 0) {
-        LPP_REQUIRE(p.grid <= 1024, "persistent decode: %d compute units exceed the statistics table", p.grid);
+        LPP_REQUIRE(p.grid <= kGridCap, "persistent decode: %d compute units exceed the statistics table", p.grid);
+        LPP_REQUIRE(m->head_size <= df::kMaxHeadPad, "persistent decode: head_size %d exceeds %d", m->head_size,
+                    df::kMaxHeadPad);
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&df::k_decode_dataflow<kF16>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(p.lds_bytes)) != hipSuccess)
             return fail(LPP_ERR_UNSUPPORTED, "persistent decode needs %zu bytes of LDS per workgroup", p.lds_bytes);
@@ -859,8 +1182,14 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
                         p.lds_bytes);
         m->persist_grid = p.grid;
     }
+    bool stale = m->df_rows == nullptr;
+    for (int t = 0; t < LPP_T_COUNT && !stale; ++t) stale = m->df_rows_key[t] != m->w[t];
+    if (stale) {
+        LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the old lists
+        LPP_TRY(build_row_lists(m, p));
+    }
     hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a,
-                       tagged_of(m), p.rows_per_wg, p.xs_floats);
+                       tagged_of(m), p.blocks, static_cast<const uint4*>(m->df_rows), m->df_row_stride);
     LPP_CHECK_LAUNCH("k_decode_dataflow");
     m->df_base += df::phases_per_token(m->cfg.n_layers);
     return LPP_OK;
@@ -871,5 +1200,6 @@ lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s)
 }
 
 unsigned dataflow_phases_per_token(int n_layers) { return df::phases_per_token(n_layers); }
+unsigned dataflow_trace_marks() { return df::kTraceMarks; }
 
 }  // namespace lpp

@@ -867,5 +867,6 @@ __device__ __forceinline__ void finish_token(const DecodeArgs& a, int token, uns
 size_t dataflow_tagged_bytes(const lpp_model* m);
 lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s);
 unsigned dataflow_phases_per_token(int n_layers);
+unsigned dataflow_trace_marks();
 
 }  // namespace lpp

@@ -28,7 +28,6 @@ using namespace ph;
 
 constexpr int kThreads = 256;            // graph path
 constexpr int kWavesPerWg = kThreads / dev::kWave;
-constexpr int kPersistThreads = 512;     // persistent path: 8 wavefronts per workgroup
 constexpr int kNoToken = -1;             // sentinel in the pinned token array
 
 struct NoWait {
@@ -94,113 +93,6 @@ __global__ __launch_bounds__(smp::kSampleThreads) void k_sample_search(DecodeArg
 }
 __global__ void k_finish(DecodeArgs a) {
     if (threadIdx.x == 0 && blockIdx.x == 0) finish_token(a, a.sampled[0], 0u);
-}
-
-// ---------------------------------------------------------------------------
-// One kernel per token
-// ---------------------------------------------------------------------------
-
-// Grid barrier over a monotonically increasing arrival counter.  Barrier number
-// i of the token whose generation base is `base` is complete when the counter
-// has reached (base + i + 1) * nwg; the counter is never reset, comparisons are
-// wrap-safe.  No cache-wide fence is issued: everything that crosses the
-// barrier is written and read with device-coherent accesses (dev::Mem<true>),
-// and the block barrier in arrive() has already waited for those stores.  The
-// wait is bounded: after spin_limit polls the workgroup records an error, raises
-// the shared abort flag and every later wait returns at once, so the grid always
-// drains.
-struct GridSync {
-    unsigned* counter;
-    unsigned* abort_flag;
-    StepParams* step;
-    unsigned base;
-    unsigned nwg;
-    unsigned spin_limit;
-    unsigned index;
-    unsigned long long* trace;  // workgroup 0 only: [2i] = arrival at barrier i, [2i+1] = release from it
-
-    __device__ __forceinline__ void arrive() {
-        __syncthreads();  // every wavefront's stores of this phase have completed
-        if (threadIdx.x == 0) {
-            __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (trace) trace[2u * index] = wall_clock64();
-        }
-    }
-
-    __device__ __forceinline__ void wait() {
-        if (threadIdx.x == 0) {
-            const unsigned target = (base + index + 1u) * nwg;
-            unsigned spins = 0;
-            while (static_cast<int>(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-                if ((spins & 63u) == 63u &&
-                    __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
-                    break;
-                if (++spins > spin_limit) {
-                    __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    step->error = 1;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-            if (trace) trace[2u * index + 1u] = wall_clock64();
-        }
-        __syncthreads();
-        ++index;
-    }
-};
-
-// Barriers per token: 5 per layer + classifier + 4 sampler steps.
-__host__ __device__ inline unsigned barriers_per_token(int n_layers) {
-    return static_cast<unsigned>(n_layers) * 5u + 5u;
-}
-
-template <bool kF16>
-__global__ __launch_bounds__(kPersistThreads) void k_decode_token(DecodeArgs a, unsigned* counter, unsigned* abort_flag,
-                                                                  unsigned spin_limit) {
-    extern __shared__ __align__(16) float lds[];
-    const int wg = blockIdx.x, nwg = gridDim.x;
-    GridSync gs{counter, abort_flag, a.step, a.step->epoch, static_cast<unsigned>(nwg), spin_limit, 0u,
-                (wg == 0) ? a.trace : nullptr};
-    if (gs.trace && threadIdx.x == 0) gs.trace[2u * barriers_per_token(a.n_layers)] = wall_clock64();
-    auto wait = [&]() { gs.wait(); };
-    const int wbytes = kF16 ? 2 : 4;
-
-    for (int layer = 0; layer < a.n_layers; ++layer) {
-        if (layer == 0) phase_qkv<kF16, 2, true>(a, layer, wg, nwg, lds, NoWait{});  // previous token ended at a kernel boundary
-        else phase_qkv<kF16, 2, true>(a, layer, wg, nwg, lds, wait);
-        gs.arrive();
-        phase_attention<true>(a, layer, wg, nwg, lds, wait);
-        gs.arrive();
-        phase_proj_residual<kF16, 2, true>(a.wo + static_cast<size_t>(layer) * a.dim * a.dim * wbytes, a.dim, a.dim, a.xb,
-                                     layer_input(a, layer), a.x, wg, nwg, lds, wait);
-        gs.arrive();
-        phase_gateup<kF16, 1, true>(a, layer, wg, nwg, lds, wait);
-        gs.arrive();
-        phase_proj_residual<kF16, 1, true, 8>(a.w2 + static_cast<size_t>(layer) * a.dim * a.hidden * wbytes, a.dim, a.hidden,
-                                     a.hb, a.x, a.x, wg, nwg, lds, wait);
-        gs.arrive();
-    }
-    phase_lmhead<kF16, 2, true>(a, wg, nwg, lds, wait);
-    gs.arrive();
-
-    const int chunk = smp::chunk_size_for(a.vocab);
-    const int nchunks = (a.vocab + chunk - 1) / chunk;
-    gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_scale<true>(a, chunk, c);
-    gs.arrive();
-    gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_exp<true>(a, chunk, nchunks, c);
-    gs.arrive();
-    gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_norm<true>(a, chunk, nchunks, c);
-    gs.arrive();
-    gs.wait();
-    for (int c = wg; c < nchunks; c += nwg) sample_step_search<true>(a, chunk, c);
-    gs.arrive();
-    if (wg == 0) {
-        gs.wait();
-        if (threadIdx.x == 0) finish_token(a, Mem<true>::ldi(a.sampled), barriers_per_token(a.n_layers));
-    }
 }
 
 // ---------------------------------------------------------------------------
@@ -346,42 +238,10 @@ void drop_graphs(lpp_model* m) {
     }
 }
 
-// Persistent path: grid = one workgroup per compute unit, all co-resident.
-size_t persistent_lds_bytes(const lpp_model* m) {
-    const lpp_config& c = m->cfg;
-    size_t floats = static_cast<size_t>((c.dim + 7) & ~7);
-    const size_t hidden = static_cast<size_t>((c.hidden_dim + 7) & ~7);
-    if (hidden > floats) floats = hidden;
-    const size_t att = static_cast<size_t>(attention_lds_floats(m->gqa, m->head_size, kPersistThreads));
-    if (att > floats) floats = att;
-    return floats * 4;
-}
-
-template <bool kF16>
-lpp_status persistent_launch(lpp_model* m, const DecodeArgs& a, hipStream_t s) {
-    static const bool use_barriers = std::getenv("LPP_DECODE_BARRIERS") != nullptr;
-    if (!use_barriers) return dataflow_launch(m, a, s);
-    if (m->persist_grid == 0) {
-        int per_cu = 0;
-        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_decode_token<kF16>, kPersistThreads,
-                                                              persistent_lds_bytes(m)));
-        if (per_cu < 1)
-            return fail(LPP_ERR_UNSUPPORTED, "persistent decode kernel does not fit a compute unit (LDS %zu bytes)",
-                        persistent_lds_bytes(m));
-        m->persist_grid = compute_units();
-    }
-    hipLaunchKernelGGL((k_decode_token<kF16>), dim3(m->persist_grid), dim3(kPersistThreads), persistent_lds_bytes(m), s,
-                       a, m->sync_words + 64, m->sync_words + 65, m->spin_limit);
-    LPP_CHECK_LAUNCH("k_decode_token");
-    return LPP_OK;
-}
-
 // One token on the model's current path.
 lpp_status launch_token(lpp_model* m, bool with_arrays, hipStream_t s) {
     if (m->path == LPP_PATH_PERSISTENT) {
-        const DecodeArgs a = make_args(m, with_arrays);
-        return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? persistent_launch<true>(m, a, s)
-                                                          : persistent_launch<false>(m, a, s);
+        return dataflow_launch(m, make_args(m, with_arrays), s);
     }
     hipGraphExec_t exec = nullptr;
     LPP_TRY(token_graph(m, with_arrays, &exec));
@@ -493,6 +353,7 @@ lpp_status fused_release(lpp_model* m) {
     lpp_free(m->sync_words);
     lpp_free(m->sample_scratch);
     lpp_free(m->tagged);
+    lpp_free(m->df_rows);
     lpp_free(m->gen_uniforms);
     return LPP_OK;
 }
@@ -669,7 +530,7 @@ lpp_status profile_impl(lpp_model* m, int pos, int reps, lpp_kernel_time* out, i
         hipStream_t s = stream();
         LPP_HIP(hipEventRecord(m->ev_a, s));
         for (int r = 0; r < reps; ++r) {
-            LPP_TRY(persistent_launch<kF16>(m, a, s));
+            LPP_TRY(dataflow_launch(m, a, s));
         }
         LPP_HIP(hipEventRecord(m->ev_b, s));
         LPP_HIP(hipEventSynchronize(m->ev_b));
@@ -742,40 +603,40 @@ extern "C" lpp_status lpp_profile_kernels(lpp_model* m, int pos, int reps, lpp_k
                                                       : profile_impl<false>(m, pos, reps, out, capacity, count);
 }
 
-// Timeline of one token on the persistent path: for every grid barrier, when
-// workgroup 0 arrived at it and when it was released, in 10 ns ticks relative to
-// the kernel's first instruction.  out[2i] / out[2i+1]; *count = 2 * barriers.
-extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count) {
+// Timeline of one token on the persistent path, workgroup 0: for phase i, mark k
+// is out[marks * i + k], in 10 ns ticks from the kernel's first instruction
+// (0 where a mark does not apply).  The last of three replays is reported.
+extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count,
+                                      int* marks_per_phase) {
     using namespace lpp;
-    LPP_REQUIRE(m && out && count, "lpp_trace_token: null argument");
+    LPP_REQUIRE(m && out && count && marks_per_phase, "lpp_trace_token: null argument");
     LPP_REQUIRE(pos >= 0 && pos < m->cfg.seq_len, "lpp_trace_token: pos %d outside [0, %d)", pos, m->cfg.seq_len);
     if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
     for (int t = 0; t < LPP_T_COUNT; ++t)
         if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
-    const int nb = static_cast<int>(std::getenv("LPP_DECODE_BARRIERS") ? barriers_per_token(m->cfg.n_layers)
-                                                                       : dataflow_phases_per_token(m->cfg.n_layers));
-    LPP_REQUIRE(capacity >= 2 * nb, "lpp_trace_token: capacity %d < %d", capacity, 2 * nb);
+    const int marks = static_cast<int>(dataflow_trace_marks());
+    const int n = marks * static_cast<int>(dataflow_phases_per_token(m->cfg.n_layers));
+    LPP_REQUIRE(capacity >= n, "lpp_trace_token: capacity %d < %d", capacity, n);
     const int saved_path = m->path;
     m->path = LPP_PATH_PERSISTENT;
-    unsigned long long* d_trace = nullptr;
     void* p = nullptr;
-    LPP_TRY(lpp_malloc(&p, static_cast<size_t>(2 * nb + 1) * sizeof(unsigned long long)));
-    d_trace = static_cast<unsigned long long*>(p);
+    LPP_TRY(lpp_malloc(&p, static_cast<size_t>(n + 1) * sizeof(unsigned long long)));
+    unsigned long long* d_trace = static_cast<unsigned long long*>(p);
     StepParams sp{};
     sp.pos = pos;
     sp.temperature = 0.8f;
     sp.penalty = 1.0f;
     sp.r = 0.5f;
     sp.freeze = 1;
-    lpp_status st = begin_run(m, sp, stream());
     hipStream_t s = stream();
-    for (int rep = 0; rep < 3 && st == LPP_OK; ++rep) {  // the last replay is the one reported
+    lpp_status st = begin_run(m, sp, s);
+    if (st == LPP_OK) st = lpp_memset(d_trace, 0, static_cast<size_t>(n + 1) * sizeof(unsigned long long));
+    for (int rep = 0; rep < 3 && st == LPP_OK; ++rep) {
         DecodeArgs a = make_args(m, false);
         a.trace = d_trace;
-        st = m->cfg.weight_precision == LPP_WEIGHT_FP16 ? persistent_launch<true>(m, a, s)
-                                                        : persistent_launch<false>(m, a, s);
+        st = dataflow_launch(m, a, s);
     }
-    std::vector<unsigned long long> host(static_cast<size_t>(2 * nb + 1));
+    std::vector<unsigned long long> host(static_cast<size_t>(n + 1));
     if (st == LPP_OK && hipStreamSynchronize(s) != hipSuccess) st = fail(LPP_ERR_HIP, "trace run failed");
     if (st == LPP_OK && hipMemcpy(host.data(), d_trace, host.size() * sizeof(unsigned long long),
                                   hipMemcpyDeviceToHost) != hipSuccess)
@@ -783,8 +644,9 @@ extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long*
     lpp_free(d_trace);
     m->path = saved_path;
     if (st != LPP_OK) return st;
-    const unsigned long long t0 = host[static_cast<size_t>(2 * nb)];
-    for (int i = 0; i < 2 * nb; ++i) out[i] = host[static_cast<size_t>(i)] - t0;
-    *count = 2 * nb;
+    const unsigned long long t0 = host[static_cast<size_t>(n)];
+    for (int i = 0; i < n; ++i) out[i] = host[static_cast<size_t>(i)] >= t0 ? host[static_cast<size_t>(i)] - t0 : 0ull;
+    *count = n;
+    *marks_per_phase = marks;
     return LPP_OK;
 }

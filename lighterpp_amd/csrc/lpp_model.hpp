@@ -54,6 +54,9 @@ struct lpp_model {
     float* gen_uniforms = nullptr;           // device copy of the per-step draws
     int gen_cap = 0;
     void* tagged = nullptr;                  // value+sequence-number vectors of the persistent kernel
+    void* df_rows = nullptr;                 // row lists of the persistent kernel's streaming wavefronts
+    int df_row_stride = 0;
+    const void* df_rows_key[12] = {};        // weight addresses the lists were built from
     unsigned df_base = 0;                    // sequence-number base of the next persistent launch
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
     unsigned spin_limit = 1u << 20;          // polls a grid-barrier wait may take before giving up
