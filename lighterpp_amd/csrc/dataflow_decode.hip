@@ -50,10 +50,12 @@ constexpr int kGemvWaves = 8;                      // streaming wavefronts per w
 constexpr int kIoWaves = 8;                        // exchange wavefronts per workgroup
 constexpr int kThreads = (kGemvWaves + kIoWaves) * kWave;
 constexpr int kIoThreads = kIoWaves * kWave;
-constexpr int kDepth = 8;                          // weight steps a streaming wavefront keeps in flight
-constexpr int kStepLoads = 2;                      // 16-byte loads per lane and step: 2 KiB of one row
-constexpr int kPollBatch = 16;                     // tagged values one thread requests before checking any
-constexpr int kItemPositions = 256;                // context positions per attention work item
+constexpr int kDepth = 4;                          // weight steps a streaming wavefront keeps in flight
+constexpr int kStepLoads = 4;                      // 16-byte loads per lane and step: 4 KiB of one row
+constexpr int kPollBatch = 8;                      // tagged values one thread requests before checking any
+constexpr int kItemPositions = 1024;               // context positions per attention work item
+constexpr int kAttSubBlock = 256;                  // positions scored between two barriers of an item
+constexpr int kAttScoreFloats = 512;               // one score area (a sub-block never exceeds kIoThreads positions)
 constexpr int kMaxHeadPad = 128;
 
 typedef unsigned long long u64;
@@ -81,6 +83,9 @@ struct Tagged {
     u64* part;   // [n_heads][splits_cap][head_size + 2] attention split partials
     u64* stats;  // [nwg][4]  per-workgroup sampler statistics (max, sum, argmax)
     int splits_cap;
+    // the step record, except the token id (which the previous launch left in device memory)
+    int pos, history_len;
+    float temperature, penalty, r;
     unsigned base;    // sequence-number base of this launch, advanced by the host once per token
     unsigned* abort;  // raised by a wavefront whose poll ran out of patience
     unsigned spin_limit;
@@ -104,13 +109,15 @@ struct Blocks {
 struct Control {
     unsigned staged;                 // += 1 by every exchange wavefront once it has staged a GEMV phase
     unsigned io_bar;                 // arrival counter of the exchange wavefronts' barrier
-    unsigned progress[kGemvWaves];   // GEMV phases wavefront j has completed
+    alignas(16) unsigned progress[kGemvWaves];   // GEMV phases wavefront j has completed
     float red[2][kIoWaves];
     float redv[2][kIoWaves];
     int redi[2][kIoWaves];
     float wave_tot[kIoWaves];
     int wave_found[kIoWaves];
     int target, token;
+    unsigned error;                  // an LDS wait gave up (reported by the exchange wavefronts at the end)
+    unsigned long long gemv_mark[2]; // timeline: streaming wavefront 0 saw the staged flag / finished its last row
 };
 
 // (relaxed workgroup-scope atomics rather than volatile: they keep the LDS address
@@ -130,14 +137,14 @@ __device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory")
 // mistake in that reasoning ends as a reported error instead of a hung device.
 constexpr unsigned kLdsSpinLimit = 1u << 22;
 template <class Ready>
-__device__ __forceinline__ void lds_wait(StepParams* step, Ready ready) {
+__device__ __forceinline__ void lds_wait(unsigned* error_word, Ready ready) {
     unsigned spins = 0;
     while (!ready()) {
         if (++spins > kLdsSpinLimit) {
-            step->error = 2;
+            lds_poke(error_word, 2u);  // LDS, not global: a store in flight would spoil the streaming wavefronts' load counting
             break;
         }
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(2);
     }
 }
 
@@ -177,132 +184,154 @@ enum { kGQkv = 0, kGO = 1, kGGateUp = 2, kGDown = 3, kGCls = 4 };
 
 // The order in which a streaming wavefront needs its weights is fixed by the
 // model's shape, so the host lists it once: for every (workgroup, wavefront) the
-// rows it owns, in order, across all GEMV phases of a token.  The wavefront
-// walks the list with scalar loads, which share nothing with the counter its
-// weight loads complete on.
-struct RowEntry {
-    unsigned long long ptr;  // first byte of the row
-    unsigned meta;           // kRowLocal | phase << 16 | flags
-    unsigned pad;
+// 2-KiB steps it will request, in order, across all GEMV phases of a token.
+// The wavefront reads its list 64 entries at a time (one entry per lane, one
+// coalesced load that travels in the same in-order stream as the weights and
+// is requested a whole batch ahead) and picks the entry of a step with a lane
+// read.  Scalar loads would not do: they share a completion counter with LDS,
+// so every wait for activations would also wait for the list.
+struct StepEntry {
+    unsigned long long ptr;  // first byte of the step: row + segment * 2 KiB
+    unsigned meta;           // local row | phase << 16 | flags
+    unsigned seg;            // segment of the row
 };
-constexpr unsigned kRowWide = 1u << 28;   // columns = hidden_dim (down projection), else dim
-constexpr unsigned kRowLast = 1u << 29;   // this wavefront's last row of the phase
-constexpr unsigned kRowValid = 1u << 31;  // cleared in the terminating entries
-constexpr unsigned kRowPhaseShift = 16, kRowPhaseMask = 0xfffu, kRowLocalMask = 0xffffu;
+constexpr unsigned kStepPartial = 1u << 26;  // the row ends inside this step: some lanes have no column
+constexpr unsigned kStepWide = 1u << 27;     // columns = hidden_dim (down projection), else dim
+constexpr unsigned kStepLastSeg = 1u << 28;  // last segment of its row
+constexpr unsigned kStepLastRow = 1u << 29;  // ... of this wavefront's last row of the phase
+constexpr unsigned kStepValid = 1u << 31;    // cleared in the terminating entries
+constexpr unsigned kStepPhaseShift = 16, kStepPhaseMask = 0x3ffu, kStepLocalMask = 0xffffu;
+constexpr int kStepBatch = 64;
 
 template <bool kF16>
-__device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, const uint4* __restrict__ rows, int j,
-                                          const float* xs, float* results, unsigned long long* trace) {
+__device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, const uint4* __restrict__ steps, int j,
+                                          const float* xs, float* results, bool trace_on) {
     constexpr int kPer = WTraits<kF16>::kPerLoad;
     constexpr int kBytes = WTraits<kF16>::kBytes;
     constexpr int kChunkCols = kWave * kPer;
     constexpr int kStepCols = kStepLoads * kChunkCols;
+    static_assert(kStepBatch % kDepth == 0, "batches change between rounds of the ring");
+    typedef const char __attribute__((address_space(1)))* GlobalBytes;  // not generic pointers: plain global loads
+    typedef const uintx4 __attribute__((address_space(1)))* GlobalVec;
     const int lane = lane_id();
     const int dim = a.dim, hidden = a.hidden;
-    const int nseg_dim = (dim + kStepCols - 1) / kStepCols;
-    const int nseg_hidden = (hidden + kStepCols - 1) / kStepCols;
     const unsigned n_phases = 4u * static_cast<unsigned>(a.n_layers) + 1u;
+    const GlobalVec list = reinterpret_cast<GlobalVec>(reinterpret_cast<unsigned long long>(steps));
 
-    // issue side: current row, the one after it (already fetched), segment
-    uint4 cur = rows[0];
-    uint4 nxt = rows[1];
-    int e = 1;
-    int seg = 0;
-    int nseg = (cur.z & kRowWide) ? nseg_hidden : nseg_dim;
-
+    uintx4 batch_a = list[lane];               // entries of the steps being requested now, one per lane
+    uintx4 batch_b = list[kStepBatch + lane];  // the batch after it, requested a whole batch ahead
     uintx4 w[kDepth][kStepLoads];
-    unsigned meta[kDepth];  // row entry meta of the step held in w[k]
-    unsigned part[kDepth];  // its segment, bit 8: last segment of the row
+    unsigned meta[kDepth];  // StepEntry::meta of the step held in w[k]
+    unsigned segs[kDepth];  // its segment
 
-    auto request = [&](int k) {
-        typedef const char __attribute__((address_space(1)))* GlobalBytes;  // not a generic pointer: plain global loads
-        typedef const uintx4 __attribute__((address_space(1)))* GlobalVec;
-        const GlobalBytes ptr = reinterpret_cast<GlobalBytes>(static_cast<unsigned long long>(cur.x) |
-                                                              (static_cast<unsigned long long>(cur.y) << 32));
-        const int d = (cur.z & kRowWide) ? hidden : dim;
+    // request step number (round * kDepth + k) of the list into w[k]
+    auto request = [&](int k, const uintx4& batch, int slot) {
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[0]), slot));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[1]), slot));
+        const unsigned mt = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot));
+        const unsigned sg = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[3]), slot));
+        const GlobalBytes ptr =
+            reinterpret_cast<GlobalBytes>(static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
+        const int d = (mt & kStepWide) ? hidden : dim;
 #pragma unroll
         for (int u = 0; u < kStepLoads; ++u) {
-            const int col = (seg * kStepLoads + u) * kChunkCols + lane * kPer;
-            const int safe_col = (col < d) ? col : 0;
-            w[k][u] = __builtin_nontemporal_load(reinterpret_cast<GlobalVec>(ptr + static_cast<size_t>(safe_col) * kBytes));
+            const int local = u * kChunkCols + lane * kPer;  // column inside the step
+            const int col = static_cast<int>(sg) * kStepCols + local;
+            const int safe = (col < d) ? local : 0;
+            w[k][u] = __builtin_nontemporal_load(reinterpret_cast<GlobalVec>(ptr + static_cast<size_t>(safe) * kBytes));
         }
-        meta[k] = cur.z;
-        part[k] = static_cast<unsigned>(seg) | ((seg + 1 == nseg) ? 0x100u : 0u);
-        if (cur.z & kRowValid) {  // the terminating entry repeats itself
-            if (++seg == nseg) {
-                seg = 0;
-                cur = nxt;
-                e += 1;
-                nxt = rows[e];
-                nseg = (cur.z & kRowWide) ? nseg_hidden : nseg_dim;
-            }
-        }
+        meta[k] = mt;
+        segs[k] = sg;
     };
 #pragma unroll
-    for (int k = 0; k < kDepth; ++k) request(k);
+    for (int k = 0; k < kDepth; ++k) request(k, batch_a, k);
     {
-        const unsigned first = (meta[0] & kRowValid) ? ((meta[0] >> kRowPhaseShift) & kRowPhaseMask) : n_phases;
+        const unsigned first = (meta[0] & kStepValid) ? ((meta[0] >> kStepPhaseShift) & kStepPhaseMask) : n_phases;
         if (lane == 0) lds_poke(&ctl.progress[j], first);
     }
 
-    // timeline slot of GEMV phase p (attention sits between qkv and the O projection)
-    auto trace_phase = [&](unsigned p) {
-        const unsigned kind = p & 3u;
-        return p + 1u == n_phases ? 5u * (p >> 2) : 5u * (p >> 2) + (kind == 0u ? 0u : kind + 1u);
-    };
     unsigned cur_p = 0xffffffffu;
     float acc = 0.0f;
     const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     bool more = true;
-    while (more) {
+    // One pass through the ring: multiply the kDepth steps in flight and request
+    // the steps whose entries sit in lanes slot0 .. slot0 + kDepth - 1 of `batch`.
+    auto run_round = [&](const uintx4& batch, int slot0) {
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) {
             const unsigned mt = meta[k];
-            if (more && (mt & kRowValid)) {
-                const int sg = static_cast<int>(part[k] & 0xffu);
-                const int d = (mt & kRowWide) ? hidden : dim;
-                const unsigned p = (mt >> kRowPhaseShift) & kRowPhaseMask;
+            if (more && (mt & kStepValid)) {
+                const int sg = static_cast<int>(segs[k]);
+                const int d = (mt & kStepWide) ? hidden : dim;
+                const unsigned p = (mt >> kStepPhaseShift) & kStepPhaseMask;
                 if (p != cur_p) {  // first step of a phase: its activations must be staged
                     cur_p = p;
                     const unsigned need = static_cast<unsigned>(kIoWaves) * (p + 1u);
-                    lds_wait(a.step, [&]() { return static_cast<int>(lds_peek(&ctl.staged) - need) >= 0; });
+                    lds_wait(&ctl.error, [&]() { return static_cast<int>(lds_peek(&ctl.staged) - need) >= 0; });
                     compiler_fence();
-                    if (trace && lane == 0) trace[kTraceMarks * trace_phase(p) + 5u] = wall_clock64();
+                    if (trace_on && lane == 0) ctl.gemv_mark[0] = wall_clock64();
                 }
+                const float* xrow = xs + sg * kStepCols + lane * kPer;
+                if (!(mt & kStepPartial)) {  // the usual case: every lane has columns in every chunk
 #pragma unroll
-                for (int u = 0; u < kStepLoads; ++u) {
-                    const int col = (sg * kStepLoads + u) * kChunkCols + lane * kPer;
-                    const bool live = col < d;
-                    const int safe_col = live ? col : 0;
-                    if constexpr (kF16) {
-                        floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
-                        floatx4 xb = *reinterpret_cast<const floatx4*>(xs + safe_col + 4);
-                        xa = live ? xa : zero;
-                        xb = live ? xb : zero;
-                        acc = dot8(w[k][u], xa, xb, acc);
-                    } else {
-                        floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
-                        xa = live ? xa : zero;
-                        acc = dot4(w[k][u], xa, acc);
+                    for (int u = 0; u < kStepLoads; ++u) {
+                        if constexpr (kF16) {
+                            const floatx4 xa = *reinterpret_cast<const floatx4*>(xrow + u * kChunkCols);
+                            const floatx4 xb = *reinterpret_cast<const floatx4*>(xrow + u * kChunkCols + 4);
+                            acc = dot8(w[k][u], xa, xb, acc);
+                        } else {
+                            acc = dot4(w[k][u], *reinterpret_cast<const floatx4*>(xrow + u * kChunkCols), acc);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < kStepLoads; ++u) {
+                        const int col = (sg * kStepLoads + u) * kChunkCols + lane * kPer;
+                        const bool live = col < d;
+                        const int safe_col = live ? col : 0;
+                        if constexpr (kF16) {
+                            floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                            floatx4 xb = *reinterpret_cast<const floatx4*>(xs + safe_col + 4);
+                            xa = live ? xa : zero;
+                            xb = live ? xb : zero;
+                            acc = dot8(w[k][u], xa, xb, acc);
+                        } else {
+                            floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
+                            xa = live ? xa : zero;
+                            acc = dot4(w[k][u], xa, acc);
+                        }
                     }
                 }
-                if (part[k] & 0x100u) {  // last segment of the row
+                if (mt & kStepLastSeg) {
                     const float sum = wave_sum(acc);
-                    if (lane == 0) results[mt & kRowLocalMask] = sum;
+                    if (lane == 0) results[mt & kStepLocalMask] = sum;
                     acc = 0.0f;
-                    if (mt & kRowLast) {  // everything before the next step's phase is complete
+                    if (mt & kStepLastRow) {  // everything before the next step's phase is complete
                         const unsigned nm = meta[(k + 1) % kDepth];
-                        const unsigned next_p = (nm & kRowValid) ? ((nm >> kRowPhaseShift) & kRowPhaseMask) : n_phases;
+                        const unsigned next_p = (nm & kStepValid) ? ((nm >> kStepPhaseShift) & kStepPhaseMask) : n_phases;
                         compiler_fence();
                         if (lane == 0) lds_poke(&ctl.progress[j], next_p);
-                        if (trace && lane == 0) trace[kTraceMarks * trace_phase(p) + 6u] = wall_clock64();
+                        if (trace_on && lane == 0) ctl.gemv_mark[1] = wall_clock64();
                     }
                 }
             } else {
                 more = false;
             }
-            request(k);
+            request(k, batch, slot0 + k);
         }
+    };
+    // The two entry batches take turns; each is re-requested, straight into its own
+    // registers, the moment its last entry has been used: a whole batch ahead.
+    constexpr int kRoundsPerBatch = kStepBatch / kDepth;
+    int next_batch = 2;
+    int first_round = 1;  // the priming requests were round 0 of the first batch
+    while (more) {
+        for (int r = first_round; r < kRoundsPerBatch && more; ++r) run_round(batch_a, r * kDepth);
+        first_round = 0;
+        batch_a = list[next_batch * kStepBatch + lane];
+        for (int r = 0; r < kRoundsPerBatch && more; ++r) run_round(batch_b, r * kDepth);
+        batch_b = list[(next_batch + 1) * kStepBatch + lane];
+        next_batch += 2;
     }
 }
 
@@ -323,7 +352,7 @@ __device__ __forceinline__ void io_sync(Control& ctl, Io& io) {
     io.gen += static_cast<unsigned>(kIoWaves);
     if (lane_id() == 0) __hip_atomic_fetch_add(&ctl.io_bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     const unsigned gen = io.gen;
-    lds_wait(io.step, [&]() { return static_cast<int>(lds_peek(&ctl.io_bar) - gen) >= 0; });
+    lds_wait(&ctl.error, [&]() { return static_cast<int>(lds_peek(&ctl.io_bar) - gen) >= 0; });
     compiler_fence();
 }
 
@@ -359,17 +388,25 @@ __device__ __forceinline__ void signal_staged(Control& ctl) {
 // Wait until every streaming wavefront has completed GEMV phase p.
 __device__ __forceinline__ void wait_gemv(Control& ctl, const Io& io, int p) {
     const unsigned need = static_cast<unsigned>(p + 1);
-    lds_wait(io.step, [&]() {
-        unsigned lowest = lds_peek(&ctl.progress[0]);
-#pragma unroll
-        for (int w = 1; w < kGemvWaves; ++w) lowest = min(lowest, lds_peek(&ctl.progress[w]));
+    static_assert(kGemvWaves == 8, "progress is read as two 16-byte vectors");
+    lds_wait(&ctl.error, [&]() {
+        compiler_fence();  // a fresh read every time round
+        const uint4 lo = *reinterpret_cast<const uint4*>(&ctl.progress[0]);
+        const uint4 hi = *reinterpret_cast<const uint4*>(&ctl.progress[4]);
+        const unsigned lowest = min(min(min(lo.x, lo.y), min(lo.z, lo.w)), min(min(hi.x, hi.y), min(hi.z, hi.w)));
         return lowest >= need;
     });
     compiler_fence();
 }
 
 __device__ __forceinline__ void mark(Ctx& c, const Io& io, int which) {
-    if (c.trace && io.it == 0) c.trace[kTraceMarks * c.phase_index + which] = wall_clock64();
+    if (c.trace && io.it == 0) {
+        c.trace[kTraceMarks * c.phase_index + which] = wall_clock64();
+        if (which == 4) {  // the streaming wavefront's marks of this phase are final by now
+            c.trace[kTraceMarks * c.phase_index + 5] = c.ctl.gemv_mark[0];
+            c.trace[kTraceMarks * c.phase_index + 6] = c.ctl.gemv_mark[1];
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -390,13 +427,17 @@ __device__ __forceinline__ bool poll_give_up(const Ctx& c, unsigned& spins) {
 // Fetch n tagged values carrying sequence number `want` and hand each to
 // sink(i, value); the exchange threads share the range.  A thread requests up
 // to kPollBatch values, then re-requests only those that were not there yet.
-template <class Sink>
+template <int kBatch = kPollBatch, class Sink>
 __device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want, const Ctx& c, const Io& io, Sink sink) {
-    for (int first = io.it; first < n; first += kIoThreads * kPollBatch) {
-        u64 got[kPollBatch];
+    // (opaque to the optimiser: otherwise the addresses of every poll in the layer loop are
+    // computed once, ahead of the loop, and occupy registers for the whole token)
+    int lane_first = io.it;
+    asm volatile("" : "+v"(lane_first));
+    for (int first = lane_first; first < n; first += kIoThreads * kBatch) {
+        u64 got[kBatch];
         unsigned pending = 0u;
 #pragma unroll
-        for (int j = 0; j < kPollBatch; ++j) {
+        for (int j = 0; j < kBatch; ++j) {
             const int i = first + j * kIoThreads;
             if (i < n) {
                 got[j] = peek(src + i);
@@ -406,17 +447,17 @@ __device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want
         unsigned spins = 0;
         while (true) {
 #pragma unroll
-            for (int j = 0; j < kPollBatch; ++j)
+            for (int j = 0; j < kBatch; ++j)
                 if ((pending >> j) & 1u)
                     if (tag_of(got[j]) == want) pending &= ~(1u << j);
             if (pending == 0u) break;
             if (poll_give_up(c, spins)) break;
 #pragma unroll
-            for (int j = 0; j < kPollBatch; ++j)
+            for (int j = 0; j < kBatch; ++j)
                 if ((pending >> j) & 1u) got[j] = peek(src + first + j * kIoThreads);
         }
 #pragma unroll
-        for (int j = 0; j < kPollBatch; ++j) {
+        for (int j = 0; j < kBatch; ++j) {
             const int i = first + j * kIoThreads;
             if (i < n) sink(i, value_of(got[j]));
         }
@@ -455,7 +496,8 @@ struct Lds {
     float* xraw;     // [dim_pad]   residual stream as last received
     float* xs;       // [xs_floats] staged GEMV input; sampler tables after the classifier
     float* results;  // [results_floats] row results of the current GEMV phase
-    float* sc;       // [kItemPositions] attention scores
+    float* sc;       // [2][kAttScoreFloats] attention scores of a sub-block, two areas taking turns
+    float* qkv;      // [3][kMaxHeadPad] this token's q, k, v of the head being attended
     float* red;      // [kIoWaves][kMaxHeadPad] attention cross-wavefront reduction
     float* gather;   // [gather_floats] attention split partials
 };
@@ -464,7 +506,7 @@ struct Lds {
 __device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, int n, unsigned want) {
     const int n_pad = (n + 7) & ~7;
     for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
-    poll_values(src, n, want, c, io, [&](int i, float v) { xs[i] = v; });
+    poll_values<2 * kPollBatch>(src, n, want, c, io, [&](int i, float v) { xs[i] = v; });  // 8192 values in one go
     mark(c, io, 1);
     signal_staged(c.ctl);
 }
@@ -587,29 +629,32 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
 // ---------------------------------------------------------------------------
 
 // One work item: query head h, context split `split` of `nsplits` (at most
-// kItemPositions positions).  kGroup lanes cover one position, 8 binary16 each.
-// K and V rows of earlier positions do not depend on this token and are
-// requested before q is polled; the current position's k and v arrive tagged and
-// are rounded to binary16 exactly as the cache store rounds them.  Scores go to
-// LDS once; every wavefront then forms the maximum and the sum of exponentials
-// for itself (model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped).
+// kItemPositions positions), walked in sub-blocks of a few rounds of one
+// position per lane group (kGroup lanes cover one position, 8 binary16 each).
+// K and V rows of earlier positions do not depend on this token: the first
+// sub-block's rows are requested before q is polled, each later sub-block's as
+// soon as the registers are free.  The current position's k and v arrive
+// tagged and are rounded to binary16 exactly as the cache store rounds them.
+// Scores of a sub-block go to LDS once; every wavefront then forms the
+// sub-block's maximum and sum of exponentials for itself and carries the
+// running maximum (model.cpp:186-198 with the softmax of ops.cpp:56-75,
+// regrouped).
 template <int kGroup>
 __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer, int h, int split, int nsplits,
                                          int npos, bool first_item) {
     const DecodeArgs& a = c.a;
     const int hs = a.head_size;
-    constexpr int hs_pad = kGroup * 8;
     constexpr int ngroups = kIoThreads / kGroup;
-    constexpr int kRounds = (kItemPositions + ngroups - 1) / ngroups;
+    constexpr int kRounds = (ngroups >= kAttSubBlock) ? 1 : (kAttSubBlock / ngroups > 4 ? 4 : kAttSubBlock / ngroups);
+    constexpr int kSub = ngroups * kRounds;  // positions per sub-block, <= max(kAttSubBlock, kIoThreads)
     const int kvh = h / a.gqa;
     const int sub = io.it % kGroup, grp = io.it / kGroup;
     const bool lane_live = sub * 8 < hs;
     const int off = lane_live ? sub * 8 : 0;
 
-    const int chunk = (npos + nsplits - 1) / nsplits;  // <= kItemPositions
+    const int chunk = (npos + nsplits - 1) / nsplits;
     const int t_begin = split * chunk;
     const int t_end = min(npos, t_begin + chunk);
-    const int n = t_end - t_begin;
     const int current = npos - 1;
     const bool has_current = current >= t_begin && current < t_end;
     const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
@@ -617,83 +662,89 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
     const uint16_t* vbase = a.value_cache + head_base;
 
     uintx4 krow[kRounds], vrow[kRounds];
+    auto request_rows = [&](uintx4 (&rows)[kRounds], const uint16_t* base, int b0) {
 #pragma unroll
-    for (int j = 0; j < kRounds; ++j) {
-        const int t = t_begin + grp + j * ngroups;
-        krow[j] = uintx4{0u, 0u, 0u, 0u};
-        vrow[j] = uintx4{0u, 0u, 0u, 0u};
-        if (t < t_end && t != current && lane_live) {
-            krow[j] = load16(kbase + static_cast<size_t>(t) * hs + off);
-            vrow[j] = load16(vbase + static_cast<size_t>(t) * hs + off);
+        for (int j = 0; j < kRounds; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            rows[j] = uintx4{0u, 0u, 0u, 0u};
+            if (t < t_end && t != current && lane_live) rows[j] = load16(base + static_cast<size_t>(t) * hs + off);
         }
-    }
+    };
+    request_rows(krow, kbase, t_begin);
+    request_rows(vrow, vbase, t_begin);
 
-    // this token's q (and, in the last split, k and v of the current position)
+    // this token's q (and, in the last split, k and v of the current position):
+    // one value per thread, shared through LDS
     const unsigned tag_in = c.seq(layer, kQkv);
-    float qv[8], kc[8], vc[8];
-    if (has_current) {
-        float in[24];
-        poll_n<24>(
-            [&](int e) -> const u64* {
-                if (e < 8) return c.t.q + static_cast<size_t>(h) * hs + off + e;
-                if (e < 16) return c.t.k + static_cast<size_t>(kvh) * hs + off + (e - 8);
-                return c.t.v + static_cast<size_t>(kvh) * hs + off + (e - 16);
-            },
-            in, tag_in, c);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            qv[e] = lane_live ? in[e] : 0.0f;
-            kc[e] = lane_live ? f16_bits_to_f32(f32_to_f16_bits(in[8 + e])) : 0.0f;
-            vc[e] = lane_live ? f16_bits_to_f32(f32_to_f16_bits(in[16 + e])) : 0.0f;
+    if (!first_item) io_sync(c.ctl, io);  // the previous item's readers have left the LDS areas
+    {
+        const int wanted = has_current ? 3 * hs : hs;
+        if (io.it < wanted) {
+            const int which = io.it / hs, e = io.it - which * hs;
+            const u64* src = which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
+                                        : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
+            float in[1];
+            poll_n<1>([&](int) -> const u64* { return src; }, in, tag_in, c);
+            // k and v as the cache will hold them
+            l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[0] : f16_bits_to_f32(f32_to_f16_bits(in[0]));
         }
-    } else {
-        float in[8];
-        poll_n<8>([&](int e) -> const u64* { return c.t.q + static_cast<size_t>(h) * hs + off + e; }, in, tag_in, c);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            qv[e] = lane_live ? in[e] : 0.0f;
-            kc[e] = 0.0f;
-            vc[e] = 0.0f;
-        }
-    }
-    if (first_item) mark(c, io, 1);
-    if (!first_item) io_sync(c.ctl, io);  // the previous item's readers have left sc and red
-
-    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
-    float score[kRounds];
-#pragma unroll
-    for (int j = 0; j < kRounds; ++j) {
-        const int t = t_begin + grp + j * ngroups;
-        const half8_t kh = as_half8(krow[j]);
-        float s = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s = fmaf((t == current) ? kc[e] : static_cast<float>(kh[e]), qv[e], s);
-        s = group_sum<kGroup>(s) * scale;
-        score[j] = s;
-        if (t < t_end && sub == 0) l.sc[t - t_begin] = s;
     }
     io_sync(c.ctl, io);
-    if (first_item) mark(c, io, 2);
-    // every wavefront: maximum and sum of exponentials over the item's scores
-    float m = -INFINITY;
-    for (int i = lane_id(); i < n; i += kWave) m = fmaxf(m, l.sc[i]);
-    m = wave_max(m);
-    float lsum = 0.0f;
-    for (int i = lane_id(); i < n; i += kWave) lsum += expf(l.sc[i] - m);
-    lsum = wave_sum(lsum);
+    if (first_item) mark(c, io, 1);
+    float qv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[e] = lane_live ? l.qkv[off + e] : 0.0f;
+    const float* kc = l.qkv + kMaxHeadPad + off;
+    const float* vc = l.qkv + 2 * kMaxHeadPad + off;
 
+    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
+    float run_max = -INFINITY, run_sum = 0.0f;
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+    int parity = 0;
+    for (int b0 = t_begin; b0 < t_end; b0 += kSub) {
+        const int n = min(kSub, t_end - b0);
+        float* sc = l.sc + parity * kAttScoreFloats;  // two score areas take turns: one barrier per sub-block is enough
+        float score[kRounds];
 #pragma unroll
-    for (int j = 0; j < kRounds; ++j) {
-        const int t = t_begin + grp + j * ngroups;
-        if (t < t_end) {
-            const float p = expf(score[j] - m);
-            const half8_t vh = as_half8(vrow[j]);
+        for (int j = 0; j < kRounds; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            const half8_t kh = as_half8(krow[j]);
+            float s = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = fmaf((t == current) ? vc[e] : static_cast<float>(vh[e]), p, acc[e]);
+            for (int e = 0; e < 8; ++e) s = fmaf((t == current) ? kc[e] : static_cast<float>(kh[e]), qv[e], s);
+            s = group_sum<kGroup>(s) * scale;
+            score[j] = s;
+            if (t < t_end && sub == 0) sc[t - b0] = s;
         }
+        if (b0 + kSub < t_end) request_rows(krow, kbase, b0 + kSub);
+        io_sync(c.ctl, io);
+        if (first_item && b0 == t_begin) mark(c, io, 2);
+        // every wavefront: the sub-block's maximum and sum of exponentials
+        float m = -INFINITY;
+        for (int i = lane_id(); i < n; i += kWave) m = fmaxf(m, sc[i]);
+        m = fmaxf(wave_max(m), run_max);
+        float lsum = 0.0f;
+        for (int i = lane_id(); i < n; i += kWave) lsum += expf(sc[i] - m);
+        lsum = wave_sum(lsum);
+        const float corr = (run_max == -INFINITY) ? 0.0f : expf(run_max - m);
+        run_sum = run_sum * corr + lsum;
+        run_max = m;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] *= corr;
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            if (t < t_end) {
+                const float p = expf(score[j] - m);
+                const half8_t vh = as_half8(vrow[j]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] = fmaf((t == current) ? vc[e] : static_cast<float>(vh[e]), p, acc[e]);
+            }
+        }
+        if (b0 + kSub < t_end) request_rows(vrow, vbase, b0 + kSub);
+        parity ^= 1;
     }
     // groups of one wavefront by lane exchange, wavefronts through LDS
 #pragma unroll
@@ -715,17 +766,16 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
 #pragma unroll
         for (int w = 0; w < kIoWaves; ++w) o += l.red[w * kMaxHeadPad + io.it];
         if (nsplits == 1) {
-            publish(c.t.xb + static_cast<size_t>(h) * hs + io.it, o / lsum, tag_out);
+            publish(c.t.xb + static_cast<size_t>(h) * hs + io.it, o / run_sum, tag_out);
         } else {
             u64* part = c.t.part + (static_cast<size_t>(h) * c.t.splits_cap + split) * (hs + 2);
             publish(part + io.it, o, tag_out);
             if (io.it == 0) {
-                publish(part + hs, m, tag_out);
-                publish(part + hs + 1, lsum, tag_out);
+                publish(part + hs, run_max, tag_out);
+                publish(part + hs + 1, run_sum, tag_out);
             }
         }
     }
-    (void)hs_pad;
 }
 
 // Combine the context splits of head h: collect every split's (output, max,
@@ -769,10 +819,8 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
     mark(c, io, 0);
     for (int item = c.wg; item < items; item += c.nwg) {
         const int h = item / nsplits, split = item - h * nsplits;
-        if (hs <= 8) att_item<1>(c, io, l, layer, h, split, nsplits, npos, first);
-        else if (hs <= 16) att_item<2>(c, io, l, layer, h, split, nsplits, npos, first);
-        else if (hs <= 32) att_item<4>(c, io, l, layer, h, split, nsplits, npos, first);
-        else if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first);
+        // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
+        if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first);
         else att_item<16>(c, io, l, layer, h, split, nsplits, npos, first);
         first = false;
     }
@@ -962,14 +1010,25 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
 template <bool kF16>
 __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
     const DecodeArgs& a = c.a;
+    // The thread index is made opaque before every phase: per-thread addresses are then formed
+    // where they are used instead of once for the whole token, where they would occupy (and
+    // overflow) the register file for the length of the layer loop.
+    auto fresh = [&]() { asm volatile("" : "+v"(io.it)); };
     for (int layer = 0; layer < a.n_layers; ++layer) {
+        fresh();
         io_qkv(c, io, l, layer);
+        fresh();
         io_attention(c, io, l, layer);
+        fresh();
         io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.t.xb, c.seq(layer, kAtt), c.seq(layer, kOproj));
+        fresh();
         io_gateup(c, io, l, layer);
+        fresh();
         io_proj(c, io, l, 4 * layer + kGDown, c.b.down, a.hidden, c.t.hb, c.seq(layer, kGateUp), c.seq(layer, kDown));
     }
+    fresh();
     io_classify_sample(c, io, l);
+    if (io.it == 0 && lds_peek(&c.ctl.error) != 0u) a.step->error = 2;
 }
 
 // ---------------------------------------------------------------------------
@@ -988,7 +1047,8 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.xs = l.xraw + dim_pad;
     l.results = l.xs + b.xs_floats;
     l.sc = l.results + b.results_floats;
-    l.red = l.sc + kItemPositions;
+    l.qkv = l.sc + 2 * kAttScoreFloats;
+    l.red = l.qkv + 3 * kMaxHeadPad;
     l.gather = l.red + kIoWaves * kMaxHeadPad;
     for (unsigned i = threadIdx.x; i < sizeof(Control) / sizeof(unsigned); i += blockDim.x)
         reinterpret_cast<unsigned*>(&ctl)[i] = 0u;
@@ -996,11 +1056,10 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     const int wave = wave_index();
     if (wave < kGemvWaves) {
         gemv_role<kF16>(a, ctl, row_lists + static_cast<size_t>(wg * kGemvWaves + wave) * row_list_stride, wave, l.xs,
-                        l.results, (wg == 0 && wave == 0) ? a.trace : nullptr);
+                        l.results, wg == 0 && wave == 0 && a.trace != nullptr);
     } else {
-        const StepParams* sp = a.step;
         Ctx c{a, t, b, ctl, t.base, (wg == 0) ? a.trace : nullptr, 0u,
-              sp->token, sp->pos, sp->history_len, sp->temperature, sp->penalty, step_uniform(a), wg, nwg};
+              __builtin_amdgcn_readfirstlane(a.step->token), t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg};
         Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
         if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
         io_role<kF16>(c, io, l);
@@ -1049,8 +1108,8 @@ Plan plan_for(const lpp_model* m) {
     if (b.cls > rows) rows = b.cls;
     b.results_floats = (rows + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
-    p.lds_bytes = static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + df::kItemPositions +
-                                      df::kIoWaves * df::kMaxHeadPad + b.gather_floats) * sizeof(float);
+    p.lds_bytes = static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
+                                      (df::kIoWaves + 3) * df::kMaxHeadPad + b.gather_floats) * sizeof(float);
     return p;
 }
 
@@ -1060,7 +1119,7 @@ size_t tagged_count(const lpp_model* m, int grid_cap) {
            static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2) + 4u * grid_cap;
 }
 
-df::Tagged tagged_of(const lpp_model* m) {
+df::Tagged tagged_of(const lpp_model* m, bool generating) {
     const lpp_config& c = m->cfg;
     df::Tagged t;
     df::u64* p = static_cast<df::u64*>(m->tagged);
@@ -1073,6 +1132,12 @@ df::Tagged tagged_of(const lpp_model* m) {
     t.part = p;         p += static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2);
     t.stats = p;
     t.splits_cap = splits_cap_for(m);
+    t.pos = m->df_pos;
+    t.history_len = m->df_history_len;
+    t.temperature = m->df_temperature;
+    t.penalty = m->df_penalty;
+    // model.cpp:291: one draw per step; a generate call brings them as an array (absent: zeros)
+    t.r = generating ? (m->df_uniforms_host ? m->df_uniforms_host[m->df_step_index] : 0.0f) : m->df_r;
     t.base = m->df_base;
     t.abort = m->sync_words + 65;
     t.spin_limit = m->spin_limit;
@@ -1081,14 +1146,19 @@ df::Tagged tagged_of(const lpp_model* m) {
 
 constexpr int kGridCap = 1024;  // workgroups the statistics table has room for
 
-// Row lists of the streaming wavefronts: [workgroup][wavefront][stride] entries,
-// each list closed by two entries without kRowValid that point at a readable row.
-lpp_status build_row_lists(lpp_model* m, const Plan& p) {
+// Step lists of the streaming wavefronts: [workgroup][wavefront][stride]
+// entries.  After a wavefront's last step the list continues with entries
+// without kStepValid that point at a readable row: the wavefront requests up to
+// a ring of steps past its last one and reads whole batches of entries.
+lpp_status build_step_lists(lpp_model* m, const Plan& p) {
     const lpp_config& c = m->cfg;
     const df::Blocks& b = p.blocks;
     const int L = c.n_layers, dim = c.dim, hidden = c.hidden_dim, kv = m->kv_dim;
     const size_t wb = c.weight_precision == LPP_WEIGHT_FP16 ? 2 : 4;
     const size_t rb_dim = static_cast<size_t>(dim) * wb, rb_hidden = static_cast<size_t>(hidden) * wb;
+    const size_t step_bytes = static_cast<size_t>(df::kStepLoads) * 1024;
+    const int nseg_dim = static_cast<int>((rb_dim + step_bytes - 1) / step_bytes);
+    const int nseg_hidden = static_cast<int>((rb_hidden + step_bytes - 1) / step_bytes);
     auto base = [&](int t) { return reinterpret_cast<unsigned long long>(m->w[t]); };
     auto block_rows = [](int total, int block, int wg) {
         const int n = total - wg * block;
@@ -1098,29 +1168,36 @@ lpp_status build_row_lists(lpp_model* m, const Plan& p) {
     int longest = 0;
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
-            const int n = L * (own(block_rows(dim + 2 * kv, b.qkv, wg), j) + own(block_rows(dim, b.o, wg), j) +
-                               own(block_rows(2 * hidden, 2 * b.gu, wg), j) + own(block_rows(dim, b.down, wg), j)) +
-                          own(block_rows(c.vocab_size, b.cls, wg), j);
+            const int n = L * ((own(block_rows(dim + 2 * kv, b.qkv, wg), j) + own(block_rows(dim, b.o, wg), j) +
+                                own(block_rows(2 * hidden, 2 * b.gu, wg), j)) * nseg_dim +
+                               own(block_rows(dim, b.down, wg), j) * nseg_hidden) +
+                          own(block_rows(c.vocab_size, b.cls, wg), j) * nseg_dim;
             if (n > longest) longest = n;
         }
-    const int stride = longest + 2;
-    LPP_REQUIRE(4 * L + 1 <= static_cast<int>(df::kRowPhaseMask), "persistent decode: too many layers for the row lists");
-    LPP_REQUIRE(b.cls <= static_cast<int>(df::kRowLocalMask) && 2 * b.gu <= static_cast<int>(df::kRowLocalMask),
-                "persistent decode: row block too large for the row lists");
-    std::vector<df::RowEntry> host(static_cast<size_t>(p.grid) * df::kGemvWaves * stride);
+    // whole batches, plus the three batches a wavefront may request past its last step
+    const int stride = ((longest + df::kDepth + df::kStepBatch - 1) / df::kStepBatch + 3) * df::kStepBatch;
+    LPP_REQUIRE(4 * L + 1 <= static_cast<int>(df::kStepPhaseMask), "persistent decode: too many layers for the step lists");
+    LPP_REQUIRE(b.cls <= static_cast<int>(df::kStepLocalMask) && 2 * b.gu <= static_cast<int>(df::kStepLocalMask),
+                "persistent decode: row block too large for the step lists");
+    std::vector<df::StepEntry> host(static_cast<size_t>(p.grid) * df::kGemvWaves * stride);
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
-            df::RowEntry* out = host.data() + (static_cast<size_t>(wg) * df::kGemvWaves + j) * stride;
+            df::StepEntry* out = host.data() + (static_cast<size_t>(wg) * df::kGemvWaves + j) * stride;
             int n = 0;
             auto phase_rows = [&](int phase, int nrows, bool wide, auto row_address) {
                 const int mine = own(nrows, j);
+                const int nseg = wide ? nseg_hidden : nseg_dim;
                 for (int i = 0; i < mine; ++i) {
                     const int r = j + i * df::kGemvWaves;
-                    out[n].ptr = row_address(r);
-                    out[n].meta = static_cast<unsigned>(r) | (static_cast<unsigned>(phase) << df::kRowPhaseShift) |
-                                  (wide ? df::kRowWide : 0u) | (i + 1 == mine ? df::kRowLast : 0u) | df::kRowValid;
-                    out[n].pad = 0;
-                    ++n;
+                    for (int s = 0; s < nseg; ++s) {
+                        out[n].ptr = row_address(r) + static_cast<size_t>(s) * step_bytes;
+                        out[n].meta = static_cast<unsigned>(r) | (static_cast<unsigned>(phase) << df::kStepPhaseShift) |
+                                      (wide ? df::kStepWide : 0u) | (s + 1 == nseg ? df::kStepLastSeg : 0u) |
+                                      (static_cast<size_t>(s + 1) * step_bytes > (wide ? rb_hidden : rb_dim) ? df::kStepPartial : 0u) |
+                                      ((s + 1 == nseg && i + 1 == mine) ? df::kStepLastRow : 0u) | df::kStepValid;
+                        out[n].seg = static_cast<unsigned>(s);
+                        ++n;
+                    }
                 }
             };
             for (int l = 0; l < L; ++l) {
@@ -1142,20 +1219,19 @@ lpp_status build_row_lists(lpp_model* m, const Plan& p) {
             }
             phase_rows(4 * L, block_rows(c.vocab_size, b.cls, wg), false,
                        [&](int r) { return base(LPP_T_WCLS) + (static_cast<size_t>(wg) * b.cls + r) * rb_dim; });
-            for (int k = 0; k < 2; ++k) {
+            for (; n < stride; ++n) {
                 out[n].ptr = base(LPP_T_WCLS);
                 out[n].meta = 0;
-                out[n].pad = 0;
-                ++n;
+                out[n].seg = 0;
             }
         }
     lpp_free(m->df_rows);
     m->df_rows = nullptr;
     void* d = nullptr;
-    LPP_TRY(lpp_malloc(&d, host.size() * sizeof(df::RowEntry)));
+    LPP_TRY(lpp_malloc(&d, host.size() * sizeof(df::StepEntry)));
     m->df_rows = d;
     m->df_row_stride = stride;
-    LPP_TRY(lpp_memcpy_h2d(d, host.data(), host.size() * sizeof(df::RowEntry)));
+    LPP_TRY(lpp_memcpy_h2d(d, host.data(), host.size() * sizeof(df::StepEntry)));
     for (int t = 0; t < LPP_T_COUNT; ++t) m->df_rows_key[t] = m->w[t];
     return LPP_OK;
 }
@@ -1186,12 +1262,18 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     for (int t = 0; t < LPP_T_COUNT && !stale; ++t) stale = m->df_rows_key[t] != m->w[t];
     if (stale) {
         LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the old lists
-        LPP_TRY(build_row_lists(m, p));
+        LPP_TRY(build_step_lists(m, p));
     }
     hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a,
-                       tagged_of(m), p.blocks, static_cast<const uint4*>(m->df_rows), m->df_row_stride);
+                       tagged_of(m, a.uniforms != nullptr), p.blocks, static_cast<const uint4*>(m->df_rows),
+                       m->df_row_stride);
     LPP_CHECK_LAUNCH("k_decode_dataflow");
     m->df_base += df::phases_per_token(m->cfg.n_layers);
+    if (!m->df_freeze) {  // what finish_token does to the device's record
+        if (m->df_history_cap > 0 && m->df_history_len < m->df_history_cap) m->df_history_len += 1;
+        m->df_pos += 1;
+        m->df_step_index += 1;
+    }
     return LPP_OK;
 }
 

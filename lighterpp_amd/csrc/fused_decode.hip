@@ -365,6 +365,15 @@ static lpp_status begin_run(lpp_model* m, const StepParams& init, hipStream_t s)
     sp = init;
     sp.epoch = 0;
     sp.error = 0;
+    m->df_pos = sp.pos;
+    m->df_history_len = sp.history_len;
+    m->df_history_cap = sp.history_cap;
+    m->df_step_index = sp.step_index;
+    m->df_freeze = sp.freeze;
+    m->df_temperature = sp.temperature;
+    m->df_penalty = sp.penalty;
+    m->df_r = sp.r;
+    m->df_uniforms_host = nullptr;
     LPP_HIP(hipMemcpyAsync(m->step, &sp, sizeof sp, hipMemcpyHostToDevice, s));
     if (m->path == LPP_PATH_PERSISTENT) LPP_TRY(lpp_memset(m->sync_words + 64, 0, 2 * sizeof(unsigned)));
     return LPP_OK;
@@ -425,6 +434,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     else
         LPP_TRY(lpp_memset(m->gen_uniforms, 0, static_cast<size_t>(n_steps) * sizeof(float)));
     for (int i = 0; i < n_steps; ++i) m->pinned_tokens[i] = kNoToken;
+    m->df_uniforms_host = uniforms;
     if (m->path != LPP_PATH_PERSISTENT) {
         hipGraphExec_t exec = nullptr;
         LPP_TRY(token_graph(m, true, &exec));  // record outside the timed loop
@@ -446,6 +456,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     }
     LPP_TRY(await_token(m, n_steps - 1, s));
     out_tokens[n_steps - 1] = m->pinned_tokens[n_steps - 1];
+    m->df_uniforms_host = nullptr;
     const auto t1 = std::chrono::steady_clock::now();
     LPP_HIP(hipEventRecord(m->ev_b, s));
     LPP_HIP(hipEventSynchronize(m->ev_b));

@@ -57,6 +57,11 @@ struct lpp_model {
     void* df_rows = nullptr;                 // row lists of the persistent kernel's streaming wavefronts
     int df_row_stride = 0;
     const void* df_rows_key[12] = {};        // weight addresses the lists were built from
+    // Host's own count of the step record for the persistent path: everything but the token id
+    // is known before a launch and travels as kernel arguments.
+    int df_pos = 0, df_history_len = 0, df_history_cap = 0, df_step_index = 0, df_freeze = 0;
+    float df_temperature = 0.0f, df_penalty = 1.0f, df_r = 0.0f;
+    const float* df_uniforms_host = nullptr; // per-step draws of the generate call in progress (host memory)
     unsigned df_base = 0;                    // sequence-number base of the next persistent launch
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
     unsigned spin_limit = 1u << 20;          // polls a grid-barrier wait may take before giving up
