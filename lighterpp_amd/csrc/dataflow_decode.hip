@@ -98,6 +98,7 @@ struct Blocks {
     int gu;     // hidden units (one gate row and one up row each)
     int down;   // rows of W2
     int cls;    // rows of the classifier
+    int ns_dim, ns_hidden;  // column slices of a dim-column / hidden-column matrix (slice_count)
     int xs_floats;
     int results_floats;
     int gather_floats;
@@ -184,24 +185,45 @@ enum { kGQkv = 0, kGO = 1, kGGateUp = 2, kGDown = 3, kGCls = 4 };
 
 // The order in which a streaming wavefront needs its weights is fixed by the
 // model's shape, so the host lists it once: for every (workgroup, wavefront) the
-// 2-KiB steps it will request, in order, across all GEMV phases of a token.
+// 4-KiB steps it will request, in order, across all GEMV phases of a token.
+// A step is one row of the workgroup's block restricted to one column slice of
+// at most kStepLoads chunks; in any one phase a wavefront works on a single
+// slice, so it takes its part of the activation vector from LDS into registers
+// once per phase and every step after that is multiply-adds between registers.
+// (Reading the activations from LDS for every row instead makes the phase
+// LDS-bandwidth bound: 8 bytes of activations for every 2 bytes of weights.)
+// A row cut into several slices yields one partial sum per slice, added up by
+// the exchange wavefronts in slice order.
+//
 // The wavefront reads its list 64 entries at a time (one entry per lane, one
 // coalesced load that travels in the same in-order stream as the weights and
 // is requested a whole batch ahead) and picks the entry of a step with a lane
 // read.  Scalar loads would not do: they share a completion counter with LDS,
 // so every wait for activations would also wait for the list.
 struct StepEntry {
-    unsigned long long ptr;  // first byte of the step: row + segment * 2 KiB
-    unsigned meta;           // local row | phase << 16 | flags
-    unsigned seg;            // segment of the row
+    unsigned long long ptr;  // first byte of the step: row start + first column of the slice
+    unsigned meta;           // result slot | phase << 16 | flags
+    unsigned cols;           // first column of the slice | columns of it that exist << 16
 };
-constexpr unsigned kStepPartial = 1u << 26;  // the row ends inside this step: some lanes have no column
-constexpr unsigned kStepWide = 1u << 27;     // columns = hidden_dim (down projection), else dim
-constexpr unsigned kStepLastSeg = 1u << 28;  // last segment of its row
-constexpr unsigned kStepLastRow = 1u << 29;  // ... of this wavefront's last row of the phase
+constexpr unsigned kStepLastRow = 1u << 29;  // this wavefront's last step of the phase
 constexpr unsigned kStepValid = 1u << 31;    // cleared in the terminating entries
-constexpr unsigned kStepPhaseShift = 16, kStepPhaseMask = 0x3ffu, kStepLocalMask = 0xffffu;
-constexpr int kStepBatch = 64;
+constexpr unsigned kStepPhaseShift = 16, kStepPhaseMask = 0x3ffu, kStepSlotMask = 0xffffu;
+constexpr int kStepBatch = 64;  // entries per batch: a multiple of kDepth, at most one per lane
+constexpr int kMaxSlices = kGemvWaves;
+
+// Column slices of a d-column matrix: a power of two, at most one per streaming
+// wavefront, each at most kStepLoads chunks wide.
+__host__ __device__ inline int slice_count(int d, int chunk_cols) {
+    const int step_cols = kStepLoads * chunk_cols;
+    int n = 1;
+    while (n * step_cols < d && n < kMaxSlices) n *= 2;
+    return n;
+}
+__host__ __device__ inline int slice_width(int d, int chunk_cols) {
+    const int n = slice_count(d, chunk_cols);
+    const int per = (d + n - 1) / n;
+    return (per + chunk_cols - 1) / chunk_cols * chunk_cols;
+}
 
 template <bool kF16>
 __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, const uint4* __restrict__ steps, int j,
@@ -209,12 +231,10 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     constexpr int kPer = WTraits<kF16>::kPerLoad;
     constexpr int kBytes = WTraits<kF16>::kBytes;
     constexpr int kChunkCols = kWave * kPer;
-    constexpr int kStepCols = kStepLoads * kChunkCols;
     static_assert(kStepBatch % kDepth == 0, "batches change between rounds of the ring");
     typedef const char __attribute__((address_space(1)))* GlobalBytes;  // not generic pointers: plain global loads
     typedef const uintx4 __attribute__((address_space(1)))* GlobalVec;
     const int lane = lane_id();
-    const int dim = a.dim, hidden = a.hidden;
     const unsigned n_phases = 4u * static_cast<unsigned>(a.n_layers) + 1u;
     const GlobalVec list = reinterpret_cast<GlobalVec>(reinterpret_cast<unsigned long long>(steps));
 
@@ -222,26 +242,24 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     uintx4 batch_b = list[kStepBatch + lane];  // the batch after it, requested a whole batch ahead
     uintx4 w[kDepth][kStepLoads];
     unsigned meta[kDepth];  // StepEntry::meta of the step held in w[k]
-    unsigned segs[kDepth];  // its segment
+    unsigned cols[kDepth];  // StepEntry::cols
 
-    // request step number (round * kDepth + k) of the list into w[k]
     auto request = [&](int k, const uintx4& batch, int slot) {
         const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[0]), slot));
         const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[1]), slot));
         const unsigned mt = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot));
-        const unsigned sg = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[3]), slot));
+        const unsigned cl = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[3]), slot));
         const GlobalBytes ptr =
             reinterpret_cast<GlobalBytes>(static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
-        const int d = (mt & kStepWide) ? hidden : dim;
+        const int width = static_cast<int>(cl >> 16);
 #pragma unroll
         for (int u = 0; u < kStepLoads; ++u) {
-            const int local = u * kChunkCols + lane * kPer;  // column inside the step
-            const int col = static_cast<int>(sg) * kStepCols + local;
-            const int safe = (col < d) ? local : 0;
+            const int local = u * kChunkCols + lane * kPer;  // column inside the slice
+            const int safe = (local < width) ? local : 0;    // lanes past the slice re-read its start; their activations are 0
             w[k][u] = __builtin_nontemporal_load(reinterpret_cast<GlobalVec>(ptr + static_cast<size_t>(safe) * kBytes));
         }
         meta[k] = mt;
-        segs[k] = sg;
+        cols[k] = cl;
     };
 #pragma unroll
     for (int k = 0; k < kDepth; ++k) request(k, batch_a, k);
@@ -251,8 +269,7 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     }
 
     unsigned cur_p = 0xffffffffu;
-    float acc = 0.0f;
-    const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    floatx4 xr[kStepLoads][kF16 ? 2 : 1];  // this wavefront's slice of the staged activations
     bool more = true;
     // One pass through the ring: multiply the kDepth steps in flight and request
     // the steps whose entries sit in lanes slot0 .. slot0 + kDepth - 1 of `batch`.
@@ -261,58 +278,43 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
         for (int k = 0; k < kDepth; ++k) {
             const unsigned mt = meta[k];
             if (more && (mt & kStepValid)) {
-                const int sg = static_cast<int>(segs[k]);
-                const int d = (mt & kStepWide) ? hidden : dim;
                 const unsigned p = (mt >> kStepPhaseShift) & kStepPhaseMask;
-                if (p != cur_p) {  // first step of a phase: its activations must be staged
+                if (p != cur_p) {  // first step of a phase: wait for its activations, take this wavefront's slice
                     cur_p = p;
                     const unsigned need = static_cast<unsigned>(kIoWaves) * (p + 1u);
                     lds_wait(&ctl.error, [&]() { return static_cast<int>(lds_peek(&ctl.staged) - need) >= 0; });
                     compiler_fence();
                     if (trace_on && lane == 0) ctl.gemv_mark[0] = wall_clock64();
-                }
-                const float* xrow = xs + sg * kStepCols + lane * kPer;
-                if (!(mt & kStepPartial)) {  // the usual case: every lane has columns in every chunk
+                    const int begin = static_cast<int>(cols[k] & 0xffffu), width = static_cast<int>(cols[k] >> 16);
+                    const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int u = 0; u < kStepLoads; ++u) {
+                        const int local = u * kChunkCols + lane * kPer;
+                        const bool live = local < width;
+                        const float* src = xs + begin + (live ? local : 0);
+                        xr[u][0] = *reinterpret_cast<const floatx4*>(src);
+                        xr[u][0] = live ? xr[u][0] : zero;
                         if constexpr (kF16) {
-                            const floatx4 xa = *reinterpret_cast<const floatx4*>(xrow + u * kChunkCols);
-                            const floatx4 xb = *reinterpret_cast<const floatx4*>(xrow + u * kChunkCols + 4);
-                            acc = dot8(w[k][u], xa, xb, acc);
-                        } else {
-                            acc = dot4(w[k][u], *reinterpret_cast<const floatx4*>(xrow + u * kChunkCols), acc);
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int u = 0; u < kStepLoads; ++u) {
-                        const int col = (sg * kStepLoads + u) * kChunkCols + lane * kPer;
-                        const bool live = col < d;
-                        const int safe_col = live ? col : 0;
-                        if constexpr (kF16) {
-                            floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
-                            floatx4 xb = *reinterpret_cast<const floatx4*>(xs + safe_col + 4);
-                            xa = live ? xa : zero;
-                            xb = live ? xb : zero;
-                            acc = dot8(w[k][u], xa, xb, acc);
-                        } else {
-                            floatx4 xa = *reinterpret_cast<const floatx4*>(xs + safe_col);
-                            xa = live ? xa : zero;
-                            acc = dot4(w[k][u], xa, acc);
+                            xr[u][1] = *reinterpret_cast<const floatx4*>(src + 4);
+                            xr[u][1] = live ? xr[u][1] : zero;
                         }
                     }
                 }
-                if (mt & kStepLastSeg) {
-                    const float sum = wave_sum(acc);
-                    if (lane == 0) results[mt & kStepLocalMask] = sum;
-                    acc = 0.0f;
-                    if (mt & kStepLastRow) {  // everything before the next step's phase is complete
-                        const unsigned nm = meta[(k + 1) % kDepth];
-                        const unsigned next_p = (nm & kStepValid) ? ((nm >> kStepPhaseShift) & kStepPhaseMask) : n_phases;
-                        compiler_fence();
-                        if (lane == 0) lds_poke(&ctl.progress[j], next_p);
-                        if (trace_on && lane == 0) ctl.gemv_mark[1] = wall_clock64();
-                    }
+                float part[kStepLoads];  // one chain of multiply-adds per chunk: they overlap instead of queueing up
+#pragma unroll
+                for (int u = 0; u < kStepLoads; ++u) {
+                    if constexpr (kF16) part[u] = dot8(w[k][u], xr[u][0], xr[u][1], 0.0f);
+                    else part[u] = dot4(w[k][u], xr[u][0], 0.0f);
+                }
+                static_assert(kStepLoads == 4, "the partial sums are added pairwise");
+                const float sum = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
+                if (lane == 0) results[mt & kStepSlotMask] = sum;
+                if (mt & kStepLastRow) {  // everything before the next step's phase is complete
+                    const unsigned nm = meta[(k + 1) % kDepth];
+                    const unsigned next_p = (nm & kStepValid) ? ((nm >> kStepPhaseShift) & kStepPhaseMask) : n_phases;
+                    compiler_fence();
+                    if (lane == 0) lds_poke(&ctl.progress[j], next_p);
+                    if (trace_on && lane == 0) ctl.gemv_mark[1] = wall_clock64();
                 }
             } else {
                 more = false;
@@ -402,7 +404,7 @@ __device__ __forceinline__ void wait_gemv(Control& ctl, const Io& io, int p) {
 __device__ __forceinline__ void mark(Ctx& c, const Io& io, int which) {
     if (c.trace && io.it == 0) {
         c.trace[kTraceMarks * c.phase_index + which] = wall_clock64();
-        if (which == 4) {  // the streaming wavefront's marks of this phase are final by now
+        if (which == 4 && c.phase_index % 5u != 1u) {  // the streaming wavefront's marks of this phase are final by now
             c.trace[kTraceMarks * c.phase_index + 5] = c.ctl.gemv_mark[0];
             c.trace[kTraceMarks * c.phase_index + 6] = c.ctl.gemv_mark[1];
         }
@@ -502,11 +504,13 @@ struct Lds {
     float* gather;   // [gather_floats] attention split partials
 };
 
-// xs = the tagged vector itself, zero padded to a multiple of 8.
+// xs = the tagged vector itself, zero padded to a multiple of 8.  (The streaming
+// wavefronts are done with the previous contents: every exchange wavefront waited
+// for all of them before publishing.)
 __device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, int n, unsigned want) {
     const int n_pad = (n + 7) & ~7;
     for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
-    poll_values<2 * kPollBatch>(src, n, want, c, io, [&](int i, float v) { xs[i] = v; });  // 8192 values in one go
+    poll_values<8192 / kIoThreads>(src, n, want, c, io, [&](int i, float v) { xs[i] = v; });  // 8192 values in one go
     mark(c, io, 1);
     signal_staged(c.ctl);
 }
@@ -542,6 +546,24 @@ __device__ __forceinline__ void stage_norm(Ctx& c, Io& io, const Lds& l, const u
 // GEMV phases as the exchange wavefronts see them
 // ---------------------------------------------------------------------------
 
+// Dot product of local row r: its column slices' partial sums, in slice order.
+__device__ __forceinline__ float row_result(const float* results, int r, int nslices) {
+    float v = results[r * nslices];
+    for (int s = 1; s < nslices; ++s) v += results[r * nslices + s];
+    return v;
+}
+
+// Run fn(r) for the local rows r < nrows of GEMV phase `gphase` once the streaming
+// wavefronts have finished it.  (Letting each exchange wavefront go ahead with the
+// rows of "its" streaming wavefronts was tried: it starts the next phase's polling
+// earlier, and the extra polling traffic cost more than the head start gained.)
+template <class RowFn>
+__device__ __forceinline__ void finished_rows(Ctx& c, Io& io, int gphase, int nrows, RowFn fn) {
+    wait_gemv(c.ctl, io, gphase);
+    mark(c, io, 3);
+    for (int r = io.it; r < nrows; r += kIoThreads) fn(r);
+}
+
 __device__ __forceinline__ int block_rows(int total, int block, int wg) {
     const int n = total - wg * block;
     return n < 0 ? 0 : (n > block ? block : n);
@@ -556,15 +578,13 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     stage_norm(c, io, l, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
                a.rms_att + static_cast<size_t>(layer) * dim);
     mark(c, io, 2);
-    wait_gemv(c.ctl, io, 4 * layer + kGQkv);
-    mark(c, io, 3);
     const int row0 = c.wg * c.b.qkv;
     const int nrows = block_rows(dim + 2 * kv_dim, c.b.qkv, c.wg);
     const float2* cs_row = a.rope + static_cast<size_t>(c.pos) * (hs / 2);
     const unsigned tag = c.seq(layer, kQkv);
-    for (int r = io.it; r < nrows; r += kIoThreads) {
+    finished_rows(c, io, 4 * layer + kGQkv, nrows, [&](int r) {
         const int g = row0 + r;
-        const float mine = l.results[r], neighbour = l.results[r ^ 1];
+        const float mine = row_result(l.results, r, c.b.ns_dim), neighbour = row_result(l.results, r ^ 1, c.b.ns_dim);
         float out = mine;
         if (g < dim + kv_dim) {  // ops.cpp:36-52 on the pair (i, i+1)
             const int gi = (g < dim) ? g : g - dim;
@@ -584,22 +604,22 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
             (is_k ? a.k : a.v)[i] = out;
             (is_k ? a.key_cache : a.value_cache)[dst] = f32_to_f16_bits(out);
         }
-    }
+    });
     mark(c, io, 4);
     ++c.phase_index;
 }
 
 // x = xraw + W . src (model.cpp:160,218 and :225-226)
-__device__ __forceinline__ void io_proj(Ctx& c, Io& io, const Lds& l, int gphase, int block, int d, const u64* src,
-                                        unsigned src_tag, unsigned out_tag) {
+__device__ __forceinline__ void io_proj(Ctx& c, Io& io, const Lds& l, int gphase, int block, int d, int nslices,
+                                        const u64* src, unsigned src_tag, unsigned out_tag) {
     mark(c, io, 0);
     stage_tagged(c, io, l.xs, src, d, src_tag);
     mark(c, io, 2);
-    wait_gemv(c.ctl, io, gphase);
-    mark(c, io, 3);
     const int row0 = c.wg * block;
     const int nrows = block_rows(c.a.dim, block, c.wg);
-    for (int r = io.it; r < nrows; r += kIoThreads) publish(c.t.x + row0 + r, l.xraw[row0 + r] + l.results[r], out_tag);
+    finished_rows(c, io, gphase, nrows, [&](int r) {
+        publish(c.t.x + row0 + r, l.xraw[row0 + r] + row_result(l.results, r, nslices), out_tag);
+    });
     mark(c, io, 4);
     ++c.phase_index;
 }
@@ -610,16 +630,16 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
     mark(c, io, 0);
     stage_norm(c, io, l, c.t.x, nullptr, a.dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * a.dim);
     mark(c, io, 2);
-    wait_gemv(c.ctl, io, 4 * layer + kGGateUp);
-    mark(c, io, 3);
     const int unit0 = c.wg * c.b.gu;
     const int units = block_rows(a.hidden, c.b.gu, c.wg);
     const unsigned tag = c.seq(layer, kGateUp);
-    for (int u = io.it; u < units; u += kIoThreads) {
-        const float gate = l.results[2 * u], up = l.results[2 * u + 1];
+    finished_rows(c, io, 4 * layer + kGGateUp, 2 * units, [&](int r) {
+        if (r & 1) return;  // the gate row's thread finishes the unit
+        const int u = r >> 1;
+        const float gate = row_result(l.results, r, c.b.ns_dim), up = row_result(l.results, r + 1, c.b.ns_dim);
         const float sigma = 1.0f / (1.0f + expf(-gate));  // ops.cpp:80-85
         publish(c.t.hb + unit0 + u, (gate * sigma) * up, tag);
-    }
+    });
     mark(c, io, 4);
     ++c.phase_index;
 }
@@ -678,24 +698,46 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
     const unsigned tag_in = c.seq(layer, kQkv);
     if (!first_item) io_sync(c.ctl, io);  // the previous item's readers have left the LDS areas
     {
-        const int wanted = has_current ? 3 * hs : hs;
+        const int wanted = has_current ? 3 * hs : hs;  // at most 2 * kIoThreads
         if (io.it < wanted) {
-            const int which = io.it / hs, e = io.it - which * hs;
-            const u64* src = which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
-                                        : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
-            float in[1];
-            poll_n<1>([&](int) -> const u64* { return src; }, in, tag_in, c);
-            // k and v as the cache will hold them
-            l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[0] : f16_bits_to_f32(f32_to_f16_bits(in[0]));
+            auto source = [&](int idx) -> const u64* {
+                const int which = idx / hs, e = idx - which * hs;
+                return which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
+                                  : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
+            };
+            const int second = io.it + kIoThreads < wanted ? io.it + kIoThreads : io.it;
+            float in[2];
+            poll_n<2>([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
+            for (int j = 0; j < 2; ++j) {
+                const int idx = j == 0 ? io.it : second;
+                const int which = idx / hs, e = idx - which * hs;
+                // k and v as the cache will hold them
+                l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[j] : f16_bits_to_f32(f32_to_f16_bits(in[j]));
+            }
         }
     }
+    if (first_item) mark(c, io, 5);
     io_sync(c.ctl, io);
     if (first_item) mark(c, io, 1);
     float qv[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) qv[e] = lane_live ? l.qkv[off + e] : 0.0f;
-    const float* kc = l.qkv + kMaxHeadPad + off;
-    const float* vc = l.qkv + 2 * kMaxHeadPad + off;
+    // the current position's row as the cache will hold it, ready to stand in for a loaded row
+    // (a register select: a conditional LDS read per element costs a branch each)
+    uintx4 cur_k = uintx4{0u, 0u, 0u, 0u}, cur_v = uintx4{0u, 0u, 0u, 0u};
+    if (has_current && lane_live) {
+        union {
+            half8_t h;
+            uintx4 u;
+        } pk, pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pk.h[e] = static_cast<half_t>(l.qkv[kMaxHeadPad + off + e]);
+            pv.h[e] = static_cast<half_t>(l.qkv[2 * kMaxHeadPad + off + e]);
+        }
+        cur_k = pk.u;
+        cur_v = pv.u;
+    }
 
     const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
     float run_max = -INFINITY, run_sum = 0.0f;
@@ -710,15 +752,16 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
 #pragma unroll
         for (int j = 0; j < kRounds; ++j) {
             const int t = b0 + grp + j * ngroups;
-            const half8_t kh = as_half8(krow[j]);
+            const half8_t kh = as_half8((t == current) ? cur_k : krow[j]);
             float s = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf((t == current) ? kc[e] : static_cast<float>(kh[e]), qv[e], s);
+            for (int e = 0; e < 8; ++e) s = fmaf(static_cast<float>(kh[e]), qv[e], s);
             s = group_sum<kGroup>(s) * scale;
             score[j] = s;
             if (t < t_end && sub == 0) sc[t - b0] = s;
         }
         if (b0 + kSub < t_end) request_rows(krow, kbase, b0 + kSub);
+        if (first_item && b0 == t_begin) mark(c, io, 6);
         io_sync(c.ctl, io);
         if (first_item && b0 == t_begin) mark(c, io, 2);
         // every wavefront: the sub-block's maximum and sum of exponentials
@@ -738,9 +781,9 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
             const int t = b0 + grp + j * ngroups;
             if (t < t_end) {
                 const float p = expf(score[j] - m);
-                const half8_t vh = as_half8(vrow[j]);
+                const half8_t vh = as_half8((t == current) ? cur_v : vrow[j]);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[e] = fmaf((t == current) ? vc[e] : static_cast<float>(vh[e]), p, acc[e]);
+                for (int e = 0; e < 8; ++e) acc[e] = fmaf(static_cast<float>(vh[e]), p, acc[e]);
             }
         }
         if (b0 + kSub < t_end) request_rows(vrow, vbase, b0 + kSub);
@@ -758,6 +801,7 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
 #pragma unroll
         for (int e = 0; e < 8; ++e) l.red[io.iw * kMaxHeadPad + sub * 8 + e] = acc[e];
     }
+    if (first_item) mark(c, io, 7);
     io_sync(c.ctl, io);
     if (first_item) mark(c, io, 3);
     const unsigned tag_out = c.seq(layer, kAtt);
@@ -857,8 +901,11 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     const int r0 = min(vocab, wg * c.b.cls);
     const int n = block_rows(vocab, c.b.cls, wg);
     const int r1 = r0 + n;
-    float* lg = l.results;
-    for (int i = it; i < n; i += kIoThreads) a.logits[r0 + i] = lg[i];  // raw logits stay readable after the token
+    float* lg = l.xs + 4 * nwg;  // beside the sampler tables; the streaming wavefronts are done with xs
+    for (int i = it; i < n; i += kIoThreads) {
+        lg[i] = row_result(l.results, i, c.b.ns_dim);
+        a.logits[r0 + i] = lg[i];  // raw logits stay readable after the token
+    }
     mark(c, io, 4);
     ++c.phase_index;
 
@@ -1020,11 +1067,12 @@ __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
         fresh();
         io_attention(c, io, l, layer);
         fresh();
-        io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.t.xb, c.seq(layer, kAtt), c.seq(layer, kOproj));
+        io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.b.ns_dim, c.t.xb, c.seq(layer, kAtt), c.seq(layer, kOproj));
         fresh();
         io_gateup(c, io, l, layer);
         fresh();
-        io_proj(c, io, l, 4 * layer + kGDown, c.b.down, a.hidden, c.t.hb, c.seq(layer, kGateUp), c.seq(layer, kDown));
+        io_proj(c, io, l, 4 * layer + kGDown, c.b.down, a.hidden, c.b.ns_hidden, c.t.hb, c.seq(layer, kGateUp),
+                c.seq(layer, kDown));
     }
     fresh();
     io_classify_sample(c, io, l);
@@ -1099,14 +1147,17 @@ Plan plan_for(const lpp_model* m) {
     const int dim_pad = (c.dim + 7) & ~7;
     int xs = (c.hidden_dim + 7) & ~7;
     if (dim_pad > xs) xs = dim_pad;
-    if (4 * p.grid > xs) xs = 4 * p.grid;  // sampler tables
+    if (4 * p.grid + b.cls > xs) xs = (4 * p.grid + b.cls + 7) & ~7;  // sampler tables and the workgroup's logits
     b.xs_floats = xs;
-    int rows = b.qkv;
-    if (b.o > rows) rows = b.o;
-    if (2 * b.gu > rows) rows = 2 * b.gu;
-    if (b.down > rows) rows = b.down;
-    if (b.cls > rows) rows = b.cls;
-    b.results_floats = (rows + 7) & ~7;
+    const int chunk_cols = c.weight_precision == LPP_WEIGHT_FP16 ? 512 : 256;
+    b.ns_dim = df::slice_count(c.dim, chunk_cols);
+    b.ns_hidden = df::slice_count(c.hidden_dim, chunk_cols);
+    int slots = b.qkv * b.ns_dim;  // one partial sum per row and column slice
+    if (b.o * b.ns_dim > slots) slots = b.o * b.ns_dim;
+    if (2 * b.gu * b.ns_dim > slots) slots = 2 * b.gu * b.ns_dim;
+    if (b.down * b.ns_hidden > slots) slots = b.down * b.ns_hidden;
+    if (b.cls * b.ns_dim > slots) slots = b.cls * b.ns_dim;
+    b.results_floats = (slots + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
     p.lds_bytes = static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
                                       (df::kIoWaves + 3) * df::kMaxHeadPad + b.gather_floats) * sizeof(float);
@@ -1155,74 +1206,76 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
     const df::Blocks& b = p.blocks;
     const int L = c.n_layers, dim = c.dim, hidden = c.hidden_dim, kv = m->kv_dim;
     const size_t wb = c.weight_precision == LPP_WEIGHT_FP16 ? 2 : 4;
+    const int chunk_cols = static_cast<int>(1024 / wb);
     const size_t rb_dim = static_cast<size_t>(dim) * wb, rb_hidden = static_cast<size_t>(hidden) * wb;
-    const size_t step_bytes = static_cast<size_t>(df::kStepLoads) * 1024;
-    const int nseg_dim = static_cast<int>((rb_dim + step_bytes - 1) / step_bytes);
-    const int nseg_hidden = static_cast<int>((rb_hidden + step_bytes - 1) / step_bytes);
     auto base = [&](int t) { return reinterpret_cast<unsigned long long>(m->w[t]); };
     auto block_rows = [](int total, int block, int wg) {
         const int n = total - wg * block;
         return n < 0 ? 0 : (n > block ? block : n);
     };
-    auto own = [](int nrows, int j) { return nrows > j ? (nrows - j + df::kGemvWaves - 1) / df::kGemvWaves : 0; };
+    // steps of wavefront j in a phase of nrows rows and d columns: it works on slice j % nslices
+    // and, of the wavefronts sharing that slice, takes every (kGemvWaves / nslices)-th row
+    auto own = [&](int nrows, int d, int j) {
+        const int share = df::kGemvWaves / df::slice_count(d, chunk_cols), rank = j / df::slice_count(d, chunk_cols);
+        return nrows > rank ? (nrows - rank + share - 1) / share : 0;
+    };
     int longest = 0;
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
-            const int n = L * ((own(block_rows(dim + 2 * kv, b.qkv, wg), j) + own(block_rows(dim, b.o, wg), j) +
-                                own(block_rows(2 * hidden, 2 * b.gu, wg), j)) * nseg_dim +
-                               own(block_rows(dim, b.down, wg), j) * nseg_hidden) +
-                          own(block_rows(c.vocab_size, b.cls, wg), j) * nseg_dim;
+            const int n = L * (own(block_rows(dim + 2 * kv, b.qkv, wg), dim, j) + own(block_rows(dim, b.o, wg), dim, j) +
+                               own(block_rows(2 * hidden, 2 * b.gu, wg), dim, j) +
+                               own(block_rows(dim, b.down, wg), hidden, j)) +
+                          own(block_rows(c.vocab_size, b.cls, wg), dim, j);
             if (n > longest) longest = n;
         }
     // whole batches, plus the three batches a wavefront may request past its last step
     const int stride = ((longest + df::kDepth + df::kStepBatch - 1) / df::kStepBatch + 3) * df::kStepBatch;
     LPP_REQUIRE(4 * L + 1 <= static_cast<int>(df::kStepPhaseMask), "persistent decode: too many layers for the step lists");
-    LPP_REQUIRE(b.cls <= static_cast<int>(df::kStepLocalMask) && 2 * b.gu <= static_cast<int>(df::kStepLocalMask),
-                "persistent decode: row block too large for the step lists");
+    LPP_REQUIRE(b.results_floats <= static_cast<int>(df::kStepSlotMask) + 1 && dim < 65536 && hidden < 65536,
+                "persistent decode: shape too large for the step lists");
     std::vector<df::StepEntry> host(static_cast<size_t>(p.grid) * df::kGemvWaves * stride);
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
             df::StepEntry* out = host.data() + (static_cast<size_t>(wg) * df::kGemvWaves + j) * stride;
             int n = 0;
-            auto phase_rows = [&](int phase, int nrows, bool wide, auto row_address) {
-                const int mine = own(nrows, j);
-                const int nseg = wide ? nseg_hidden : nseg_dim;
+            auto phase_rows = [&](int phase, int nrows, int d, auto row_address) {
+                const int nslices = df::slice_count(d, chunk_cols), width = df::slice_width(d, chunk_cols);
+                const int slice = j % nslices, rank = j / nslices, share = df::kGemvWaves / nslices;
+                const int begin = slice * width;
+                const int exist = d - begin < 0 ? 0 : (d - begin > width ? width : d - begin);
+                const int mine = exist > 0 ? own(nrows, d, j) : 0;
                 for (int i = 0; i < mine; ++i) {
-                    const int r = j + i * df::kGemvWaves;
-                    for (int s = 0; s < nseg; ++s) {
-                        out[n].ptr = row_address(r) + static_cast<size_t>(s) * step_bytes;
-                        out[n].meta = static_cast<unsigned>(r) | (static_cast<unsigned>(phase) << df::kStepPhaseShift) |
-                                      (wide ? df::kStepWide : 0u) | (s + 1 == nseg ? df::kStepLastSeg : 0u) |
-                                      (static_cast<size_t>(s + 1) * step_bytes > (wide ? rb_hidden : rb_dim) ? df::kStepPartial : 0u) |
-                                      ((s + 1 == nseg && i + 1 == mine) ? df::kStepLastRow : 0u) | df::kStepValid;
-                        out[n].seg = static_cast<unsigned>(s);
-                        ++n;
-                    }
+                    const int r = rank + i * share;
+                    out[n].ptr = row_address(r) + static_cast<size_t>(begin) * wb;
+                    out[n].meta = static_cast<unsigned>(r * nslices + slice) | (static_cast<unsigned>(phase) << df::kStepPhaseShift) |
+                                  (i + 1 == mine ? df::kStepLastRow : 0u) | df::kStepValid;
+                    out[n].cols = static_cast<unsigned>(begin) | (static_cast<unsigned>(exist) << 16);
+                    ++n;
                 }
             };
             for (int l = 0; l < L; ++l) {
-                phase_rows(4 * l + df::kGQkv, block_rows(dim + 2 * kv, b.qkv, wg), false, [&](int r) {
+                phase_rows(4 * l + df::kGQkv, block_rows(dim + 2 * kv, b.qkv, wg), dim, [&](int r) {
                     const int g = wg * b.qkv + r;
                     if (g < dim) return base(LPP_T_WQ) + (static_cast<size_t>(l) * dim + g) * rb_dim;
                     if (g < dim + kv) return base(LPP_T_WK) + (static_cast<size_t>(l) * kv + (g - dim)) * rb_dim;
                     return base(LPP_T_WV) + (static_cast<size_t>(l) * kv + (g - dim - kv)) * rb_dim;
                 });
-                phase_rows(4 * l + df::kGO, block_rows(dim, b.o, wg), false,
+                phase_rows(4 * l + df::kGO, block_rows(dim, b.o, wg), dim,
                            [&](int r) { return base(LPP_T_WO) + (static_cast<size_t>(l) * dim + wg * b.o + r) * rb_dim; });
                 // local row 2u = gate row of hidden unit u, 2u + 1 = its up row
-                phase_rows(4 * l + df::kGGateUp, block_rows(2 * hidden, 2 * b.gu, wg), false, [&](int r) {
+                phase_rows(4 * l + df::kGGateUp, block_rows(2 * hidden, 2 * b.gu, wg), dim, [&](int r) {
                     return base((r & 1) ? LPP_T_W3 : LPP_T_W1) + (static_cast<size_t>(l) * hidden + wg * b.gu + (r >> 1)) * rb_dim;
                 });
-                phase_rows(4 * l + df::kGDown, block_rows(dim, b.down, wg), true, [&](int r) {
+                phase_rows(4 * l + df::kGDown, block_rows(dim, b.down, wg), hidden, [&](int r) {
                     return base(LPP_T_W2) + (static_cast<size_t>(l) * dim + wg * b.down + r) * rb_hidden;
                 });
             }
-            phase_rows(4 * L, block_rows(c.vocab_size, b.cls, wg), false,
+            phase_rows(4 * L, block_rows(c.vocab_size, b.cls, wg), dim,
                        [&](int r) { return base(LPP_T_WCLS) + (static_cast<size_t>(wg) * b.cls + r) * rb_dim; });
             for (; n < stride; ++n) {
                 out[n].ptr = base(LPP_T_WCLS);
                 out[n].meta = 0;
-                out[n].seg = 0;
+                out[n].cols = 0;
             }
         }
     lpp_free(m->df_rows);
