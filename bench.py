@@ -125,7 +125,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--config", default="c3_llama32_1b_fp16", choices=list(WORKLOADS))
-    ap.add_argument("--path", default="fused", choices=["ops", "fused", "persistent"])
+    ap.add_argument("--path", default="persistent", choices=["ops", "fused", "persistent"])
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time bound of the CPU baseline sample (0 = skip)")
     ap.add_argument("--parity-steps", type=int, default=3)
     ap.add_argument("--profile-reps", type=int, default=20)

@@ -415,14 +415,24 @@ def test_sample_categorical(lib, vocab, temp, pen):
     hist[10] = hist[11] = hist[12]
     draws = np.concatenate([capi.synth_uniform_f32(60, vocab), np.array([0.0, 1.0, 0.99999994, 1e-7, 0.5], F)])
     _, want_probs = ob.orc_sample(lg, temp, 1.0, pen, hist, 0.5)
+    # the exact CDF (fp64) of the penalised, tempered logits: the device's token must sit where
+    # the draw falls in it, to within the rounding of an fp32 sum over the vocabulary
+    z = ob.orc_sample(lg, 0.0, 1.0, pen, hist, 0.0)[1].astype(np.float64) / temp
+    p64 = np.exp(z - z.max())
+    c64 = np.cumsum(p64 / p64.sum())
     near = 0
     for r in draws:
         want, lo, hi = ob.orc_sample_cdf(lg, temp, pen, hist, float(r))
         got, probs = sample_gpu(lib, lg, temp, pen, hist, float(r))
+        below = c64[got - 1] if got > 0 else 0.0
+        assert below - 2e-6 <= float(r) < c64[got] + 2e-6 or got == vocab - 1, (float(r), got, below, c64[got])
         if got != want:
             near += 1
             assert min(abs(float(r) - lo), abs(float(r) - hi)) < 1e-4, (float(r), want, got, lo, hi)
-    assert near <= 3
+    # With 128256 buckets of ~8e-6 each, the drift of the CPU's running fp32 sum (up to ~1e-5 by the
+    # end of the vocabulary) moves a fair share of draws into a neighbouring bucket; with few
+    # buckets it must not happen more than occasionally.
+    assert near <= (3 if vocab < 50000 else len(draws) // 2)
     # the buffer is left holding probabilities, as on the CPU (model.cpp:290)
     # (the CPU's running fp32 sum over the vocabulary drifts by up to ~n ulp, the
     # device's tree sum does not: compare loosely with the oracle, tightly with fp64)
