@@ -98,7 +98,7 @@ struct Blocks {
     int gu;     // hidden units (one gate row and one up row each)
     int down;   // rows of W2
     int cls;    // rows of the classifier
-    int ns_dim, ns_hidden;  // column slices of a dim-column / hidden-column matrix (slice_count)
+    int ns_dim, ns_hidden;  // partial sums per row of a dim-column / hidden-column matrix (slices_used)
     int xs_floats;
     int results_floats;
     int gather_floats;
@@ -222,7 +222,13 @@ __host__ __device__ inline int slice_count(int d, int chunk_cols) {
 __host__ __device__ inline int slice_width(int d, int chunk_cols) {
     const int n = slice_count(d, chunk_cols);
     const int per = (d + n - 1) / n;
-    return (per + chunk_cols - 1) / chunk_cols * chunk_cols;
+    return (per + 255) / 256 * 256;  // a slice starts on a multiple of 256 columns (pack_cols)
+}
+// Slices that actually hold columns (rounding the width up can leave the last ones empty): a
+// row's partial sums are results[row * slices_used + slice].
+__host__ __device__ inline int slices_used(int d, int chunk_cols) {
+    const int width = slice_width(d, chunk_cols);
+    return (d + width - 1) / width;
 }
 
 template <bool kF16>
@@ -912,11 +918,17 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     const float temperature = c.temperature, penalty = c.penalty;
     const int history_len = c.history_len;
     if (penalty > 1.0f && history_len > 0) {  // model.cpp:258-270, once per occurrence
+        // the window is scanned once per entry: bring it into LDS first (the attention score area is idle)
+        int* window = reinterpret_cast<int*>(l.sc);
+        const bool window_fits = history_len <= 2 * kAttScoreFloats;
+        if (window_fits)
+            for (int i = it; i < history_len; i += kIoThreads) window[i] = a.history[i];
         io_sync(ctl, io);
+        const int* hist = window_fits ? window : a.history;
         for (int i = it; i < history_len; i += kIoThreads) {
-            const int tok = a.history[i];
+            const int tok = hist[i];
             if (tok < r0 || tok >= r1) continue;
-            const int count = smp::owned_count(a.history, history_len, i);
+            const int count = smp::owned_count(hist, history_len, i);
             if (count > 0) lg[tok - r0] = smp::penalise(lg[tok - r0], penalty, count);
         }
         io_sync(ctl, io);
@@ -973,18 +985,14 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     io_sync(ctl, io);
     mark(c, io, 2);
     if (temperature == 0.0f) {  // model.cpp:272-283: first maximum wins
-        if (it == 0) {
+        if (io.iw == 0) {  // one wavefront, a few workgroups per lane
             ArgMax g{-INFINITY, 0x7fffffff};
-            int target = 0;
-            for (int w = 0; w < nwg; ++w) {
-                const ArgMax cand{st_max[w], __float_as_int(st_arg[w])};
-                if (cand.v > g.v || (cand.v == g.v && cand.i < g.i)) {
-                    g = cand;
-                    target = w;
-                }
+            for (int w = lane_id(); w < nwg; w += kWave) g = argmax_better(g, ArgMax{st_max[w], __float_as_int(st_arg[w])});
+            g = wave_argmax(g);
+            if (lane_id() == 0) {
+                ctl.token = (g.i == 0x7fffffff) ? 0 : g.i;
+                ctl.target = (g.i == 0x7fffffff) ? 0 : g.i / c.b.cls;  // the workgroup that owns the winning row
             }
-            ctl.target = target;
-            ctl.token = (g.i == 0x7fffffff) ? 0 : g.i;
         }
         io_sync(ctl, io);
     } else {
@@ -999,18 +1007,27 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
         }
         const float total = io_sum(ctl, io, mass);
         const float r = c.r;
-        if (it == 0) {
-            // sequential in workgroup order = index order of the CDF (model.cpp:294-301)
-            float cum = 0.0f;
-            int target = -1;
-            for (int w = 0; w < nwg; ++w) {
+        if (io.iw == 0) {
+            // Running mass in workgroup order = index order of the CDF (model.cpp:294-301): every
+            // lane takes a run of consecutive workgroups, a scan across the lanes gives each run's start.
+            const int per_lane = (nwg + kWave - 1) / kWave;
+            const int w0 = lane_id() * per_lane, w1 = min(nwg, w0 + per_lane);
+            float run = 0.0f;
+            for (int w = w0; w < w1; ++w) run += st_cum[w] / total;
+            float cum = wave_inclusive_scan(run) - run;
+            int target = 0x7fffffff;
+            for (int w = w0; w < w1; ++w) {
                 const float before = cum;
                 cum += st_cum[w] / total;
                 st_cum[w] = before;
-                if (target < 0 && r < cum) target = w;
+                if (target == 0x7fffffff && r < cum) target = w;
             }
-            ctl.target = target;
-            ctl.token = vocab - 1;  // model.cpp:302 when no bucket is reached
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) target = min(target, __shfl_xor(target, o));
+            if (lane_id() == 0) {
+                ctl.target = target == 0x7fffffff ? -1 : target;
+                ctl.token = vocab - 1;  // model.cpp:302 when no bucket is reached
+            }
         }
         io_sync(ctl, io);
         if (lds_ld(&ctl.target) == wg) {
@@ -1150,8 +1167,8 @@ Plan plan_for(const lpp_model* m) {
     if (4 * p.grid + b.cls > xs) xs = (4 * p.grid + b.cls + 7) & ~7;  // sampler tables and the workgroup's logits
     b.xs_floats = xs;
     const int chunk_cols = c.weight_precision == LPP_WEIGHT_FP16 ? 512 : 256;
-    b.ns_dim = df::slice_count(c.dim, chunk_cols);
-    b.ns_hidden = df::slice_count(c.hidden_dim, chunk_cols);
+    b.ns_dim = df::slices_used(c.dim, chunk_cols);
+    b.ns_hidden = df::slices_used(c.hidden_dim, chunk_cols);
     int slots = b.qkv * b.ns_dim;  // one partial sum per row and column slice
     if (b.o * b.ns_dim > slots) slots = b.o * b.ns_dim;
     if (2 * b.gu * b.ns_dim > slots) slots = 2 * b.gu * b.ns_dim;
@@ -1213,11 +1230,12 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
         const int n = total - wg * block;
         return n < 0 ? 0 : (n > block ? block : n);
     };
-    // steps of wavefront j in a phase of nrows rows and d columns: it works on slice j % nslices
-    // and, of the wavefronts sharing that slice, takes every (kGemvWaves / nslices)-th row
+    // steps of a wavefront in a phase of nrows rows and d columns: it works on one slice and, of the
+    // wavefronts sharing that slice, takes one row of every (kGemvWaves / nslices)
     auto own = [&](int nrows, int d, int j) {
-        const int share = df::kGemvWaves / df::slice_count(d, chunk_cols), rank = j / df::slice_count(d, chunk_cols);
-        return nrows > rank ? (nrows - rank + share - 1) / share : 0;
+        const int share = df::kGemvWaves / df::slice_count(d, chunk_cols);
+        (void)j;
+        return (nrows + share - 1) / share;  // an upper bound for every wavefront
     };
     int longest = 0;
     for (int wg = 0; wg < p.grid; ++wg)
@@ -1243,15 +1261,23 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
                 const int slice = j % nslices, rank = j / nslices, share = df::kGemvWaves / nslices;
                 const int begin = slice * width;
                 const int exist = d - begin < 0 ? 0 : (d - begin > width ? width : d - begin);
-                const int mine = exist > 0 ? own(nrows, d, j) : 0;
-                for (int i = 0; i < mine; ++i) {
-                    const int r = rank + i * share;
+                if (exist == 0) return;
+                // Of every `share` consecutive rows this wavefront takes one, and not always the same
+                // one: with a fixed residue its rows would sit at a fixed stride in memory.  (Which of a
+                // workgroup's wavefronts streams which rows does not change how long a bandwidth-bound
+                // phase takes: the wavefront launched first on each SIMD runs ahead of its neighbour,
+                // but handing it more rows only widens its lead; the phase ends when the bytes are in.)
+                const int first = n;
+                for (int i = 0; i * share < nrows; ++i) {
+                    const int r = i * share + (rank + i) % share;
+                    if (r >= nrows) continue;
                     out[n].ptr = row_address(r) + static_cast<size_t>(begin) * wb;
-                    out[n].meta = static_cast<unsigned>(r * nslices + slice) | (static_cast<unsigned>(phase) << df::kStepPhaseShift) |
-                                  (i + 1 == mine ? df::kStepLastRow : 0u) | df::kStepValid;
+                    out[n].meta = static_cast<unsigned>(r * df::slices_used(d, chunk_cols) + slice) |
+                                  (static_cast<unsigned>(phase) << df::kStepPhaseShift) | df::kStepValid;
                     out[n].cols = static_cast<unsigned>(begin) | (static_cast<unsigned>(exist) << 16);
                     ++n;
                 }
+                if (n > first) out[n - 1].meta |= df::kStepLastRow;
             };
             for (int l = 0; l < L; ++l) {
                 phase_rows(4 * l + df::kGQkv, block_rows(dim + 2 * kv, b.qkv, wg), dim, [&](int r) {

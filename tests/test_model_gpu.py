@@ -32,6 +32,11 @@ SMALL_SHAPES = {
     "gqa4_fp16": Shape(256, 512, 3, 8, 2, 2048, 160, 500000.0, fp16=True, tied=True),
     "gqa8_fp16_untied": Shape(512, 1408, 2, 8, 1, 1500, 96, 10000.0, fp16=True, tied=False),
     "hs128_fp16": Shape(512, 1024, 2, 4, 2, 777, 48, 500000.0, fp16=True, tied=False),
+    # rows wider than one 4-KiB weight step: the persistent kernel cuts them into column slices
+    # (dim 2560 -> 2 slices of 1280, hidden 7168 -> 4 of 1792) and adds per-slice partial sums
+    "sliced_fp16": Shape(2560, 7168, 1, 20, 4, 640, 24, 500000.0, fp16=True, tied=False),
+    # fp32 rows: dim 1536 -> 2 slices of 768; hidden 2304 -> width 768, 3 slices used of 4 (one idle)
+    "sliced_fp32_idle_slice": Shape(1536, 2304, 2, 12, 4, 500, 24, 10000.0, fp16=False, tied=True),
 }
 
 
