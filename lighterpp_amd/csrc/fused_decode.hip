@@ -547,7 +547,7 @@ lpp_status profile_impl(lpp_model* m, int pos, int reps, lpp_kernel_time* out, i
         LPP_HIP(hipEventSynchronize(m->ev_b));
         float total = 0.0f;
         LPP_HIP(hipEventElapsedTime(&total, m->ev_a, m->ev_b));
-        add("k_decode_token", 1, static_cast<double>(total) / reps, token_bytes);
+        add("k_decode_dataflow", 1, static_cast<double>(total) / reps, token_bytes);
         *count = n < capacity ? n : capacity;
         return LPP_OK;
     }
