@@ -528,6 +528,17 @@ __device__ __forceinline__ void stage_norm(Ctx& c, Io& io, const Lds& l, const u
 #pragma clang fp contract(off)
     float* xraw = l.xraw;
     float* xs = l.xs;
+    // The gains do not depend on anything: request this thread's first few before polling, so that
+    // their memory latency is spent while the inputs are still on their way (the fence keeps the
+    // requests from being moved down to their first use).
+    constexpr int kEarly = 8;
+    float early_gain[kEarly];
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int i = io.it + e * kIoThreads;
+        early_gain[e] = (i < n) ? gain[i] : 0.0f;
+    }
+    compiler_fence();
     if (plain_x != nullptr) {
         for (int i = io.it; i < n; i += kIoThreads) xraw[i] = plain_x[i];
     } else {
@@ -544,7 +555,12 @@ __device__ __forceinline__ void stage_norm(Ctx& c, Io& io, const Lds& l, const u
     ss += 1e-5f;
     const float scale = 1.0f / sqrtf(ss);
     const int n_pad = (n + 7) & ~7;
-    for (int i = io.it; i < n_pad; i += kIoThreads) xs[i] = (i < n) ? xraw[i] * scale * gain[i] : 0.0f;
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int i = io.it + e * kIoThreads;
+        if (i < n_pad) xs[i] = (i < n) ? xraw[i] * scale * early_gain[e] : 0.0f;
+    }
+    for (int i = io.it + kEarly * kIoThreads; i < n_pad; i += kIoThreads) xs[i] = (i < n) ? xraw[i] * scale * gain[i] : 0.0f;
     signal_staged(c.ctl);
 }
 
@@ -588,13 +604,20 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     const int nrows = block_rows(dim + 2 * kv_dim, c.b.qkv, c.wg);
     const float2* cs_row = a.rope + static_cast<size_t>(c.pos) * (hs / 2);
     const unsigned tag = c.seq(layer, kQkv);
+    // (cos, sin) of this thread's first row: requested while the streaming wavefronts still multiply
+    float2 cs_first = make_float2(1.0f, 0.0f);
+    {
+        const int g = row0 + io.it;
+        if (io.it < nrows && g < dim + kv_dim) cs_first = cs_row[((((g < dim) ? g : g - dim) & ~1) % hs) >> 1];
+    }
+    compiler_fence();
     finished_rows(c, io, 4 * layer + kGQkv, nrows, [&](int r) {
         const int g = row0 + r;
         const float mine = row_result(l.results, r, c.b.ns_dim), neighbour = row_result(l.results, r ^ 1, c.b.ns_dim);
         float out = mine;
         if (g < dim + kv_dim) {  // ops.cpp:36-52 on the pair (i, i+1)
             const int gi = (g < dim) ? g : g - dim;
-            const float2 cs = cs_row[((gi & ~1) % hs) >> 1];
+            const float2 cs = (r == io.it) ? cs_first : cs_row[((gi & ~1) % hs) >> 1];
             out = (gi & 1) ? neighbour * cs.y + mine * cs.x : mine * cs.x - neighbour * cs.y;
         }
         if (g < dim) {
