@@ -246,9 +246,11 @@ lpp_status lpp_profile_kernels(lpp_model *m, int pos, int reps, lpp_kernel_time 
 /* Timeline of one token on LPP_PATH_PERSISTENT at position `pos`, as seen by
  * workgroup 0: out[marks * i + k] is mark k of phase i in 10 ns ticks from the
  * kernel's start (0 = mark not taken).  Phase order per layer: qkv, attention,
- * o-projection, gate/up, down; then classifier and sampler.  Marks: 0 phase
- * entered, 1 own inputs received, 2 inputs staged, 3 row results ready,
- * 4 outputs published, 5 first weight step multiplied, 6 last row finished.
+ * o-projection, gate/up, down; then classifier and sampler.  Marks of a GEMV
+ * phase: 0 phase entered, 1 own inputs received, 2 inputs staged, 3 row results
+ * ready, 4 outputs published, 5 first weight step multiplied, 6 last row
+ * finished.  Attention: 0 entered, 5 q/k/v received, 1 shared, 6 scores
+ * computed, 2 scores exchanged, 7 values accumulated, 3 reduced, 4 published.
  * *count = marks * phases, *marks_per_phase = marks. */
 lpp_status lpp_trace_token(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count,
                            int *marks_per_phase);

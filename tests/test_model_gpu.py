@@ -265,3 +265,26 @@ def test_benchmark_shapes_first_steps(cfg, steps, start):
     assert agree == steps
     m.close()
     o.close()
+
+
+def test_persistent_timeline_is_ordered():
+    """lpp_trace_token: every phase of the persistent kernel reports its marks, in order, and the
+    phases follow one another (the timeline is what DESIGN.md's per-phase figures come from)."""
+    import ctypes as C
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m, o = build(shape, 4)
+    arr = (C.c_ulonglong * 4096)()
+    n, marks = C.c_int(), C.c_int()
+    capi.check(m.lib.lpp_trace_token(m.handle, 5, arr, 4096, C.byref(n), C.byref(marks)))
+    phases = 5 * shape.n_layers + 2
+    assert marks.value == 8 and n.value == 8 * phases
+    t = np.array(arr[:n.value], dtype=np.int64).reshape(phases, 8)
+    published = t[:, 4]
+    assert np.all(np.diff(published) > 0), "phases out of order"
+    gemv = [i for i in range(5 * shape.n_layers) if i % 5 != 1] + [5 * shape.n_layers]
+    for i in gemv:
+        e, polled, staged, rows, pub = t[i, 0], t[i, 1], t[i, 2], t[i, 3], t[i, 4]
+        assert 0 < e <= polled <= staged <= rows <= pub, (i, t[i])
+    assert published[-1] < 100_000_00, "a tiny model's token takes far less than a second (10 ns ticks)"
+    m.close()
+    o.close()
