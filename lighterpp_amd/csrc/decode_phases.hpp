@@ -11,17 +11,17 @@
 //   lmhead   rmsnorm(x)        -> classifier GEMV -> logits                   (fuses :357-358)
 //   sample   four short steps over vocabulary chunks + one bookkeeping step   (:366-370)
 //
-// Each phase is a __device__ function of (workgroup index, workgroup count), so
-// the same code runs as one launch per phase (a HIP graph of kernels) or inside
-// one persistent kernel with grid barriers in between.  GEMV phases issue their
-// first weight loads BEFORE calling the `pre` hook that waits for the previous
-// phase and stages the activations in LDS: weights never depend on activations,
-// so HBM keeps streaming across the phase boundary.
+// Each phase is a __device__ function of (workgroup index, workgroup count); the
+// kernels of fused_decode.hip run one phase per launch (a HIP graph of kernels).
+// GEMV phases issue their first weight loads BEFORE calling the `pre` hook and
+// staging the activations in LDS: weights never depend on activations.
+// (dataflow_decode.hip, the one-kernel-per-token schedule, shares DecodeArgs, the
+// sampler helpers and finish_token with this file but has its own phase code.)
 //
-// kCoh = true is the persistent kernel: whatever one phase hands to the next
-// (q, k, v, x, xb, hb, logits, sampler tables) is written and read with
-// device-coherent accesses (dev::Mem<true>), because producer and consumer may
-// sit on different XCDs and no cache-wide fence is issued at the barriers.
+// kCoh selects dev::Mem<kCoh> for whatever one phase hands to the next; the
+// kernels here pass false (their inputs are complete before the launch).  Values
+// that cross workgroups inside ONE launch (the attention split partials) always
+// use dev::Mem<true>: producer and consumer may sit on different XCDs.
 #pragma once
 
 #include "lpp_device.hpp"
@@ -69,7 +69,7 @@ struct DecodeArgs {
     int* out_tokens;       // per-step results (may be pinned host memory), or null
     int* sampled;          // [1]
     smp::SampleScratch sample_scratch;
-    unsigned long long* trace;  // optional: timestamps of workgroup 0 at every grid barrier
+    unsigned long long* trace;  // optional: timeline of workgroup 0 (one-kernel-per-token schedule only)
 };
 
 // ---------------------------------------------------------------------------

@@ -3,16 +3,14 @@
 //
 //   LPP_PATH_FUSED       one launch per phase (5 per layer + classifier + sampler
 //                        steps), recorded once into a HIP graph, replayed per token;
-//   LPP_PATH_PERSISTENT  one kernel per token that walks all phases itself, with
-//                        a grid barrier between phases.  A workgroup requests the
-//                        first weights of the next phase before it waits at the
-//                        barrier, so HBM keeps streaming while the grid
-//                        synchronises.
+//   LPP_PATH_PERSISTENT  one kernel per token (dataflow_decode.hip); this file
+//                        holds its host side: launch, generation loop, timing.
 //
 // All per-token scalars (token, position, penalty window, uniform draw) live in
-// device memory, so neither schedule is patched between tokens; the sampled id is
-// fed back on the device and written straight into pinned host memory, 4 bytes
-// per token.
+// device memory, so the graph is not patched between tokens (the persistent
+// kernel takes everything but the token id as launch arguments); the sampled id
+// is fed back on the device and written straight into pinned host memory, 4
+// bytes per token.
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -329,7 +327,7 @@ lpp_status fused_prepare(lpp_model* m) {
     m->att_partial = static_cast<float*>(p);
     LPP_TRY(lpp_malloc(&p, static_cast<size_t>(c.vocab_size) * sizeof(float)));
     m->work_logits = static_cast<float*>(p);
-    // words 0..63: attention split counters per KV head; 64: grid-barrier arrivals; 65: abort flag
+    // words 0..63: attention split counters per KV head; 64: unused; 65: abort flag of the persistent kernel
     LPP_REQUIRE(c.n_kv_heads <= 64 || !m->fused_ok, "more than 64 KV heads");
     LPP_TRY(lpp_malloc(&p, 128 * sizeof(unsigned)));
     m->sync_words = static_cast<unsigned*>(p);
@@ -358,7 +356,7 @@ lpp_status fused_release(lpp_model* m) {
     return LPP_OK;
 }
 
-// Bring the device-side step record (and the persistent kernel's barrier state)
+// Bring the device-side step record (and the persistent kernel's abort flag)
 // to a known start.
 static lpp_status begin_run(lpp_model* m, const StepParams& init, hipStream_t s) {
     StepParams& sp = *m->step_host;
@@ -404,7 +402,7 @@ lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, fl
     LPP_HIP(hipStreamSynchronize(s));
     if (m->path == LPP_PATH_PERSISTENT) {
         LPP_HIP(hipMemcpy(m->step_host, m->step, sizeof(StepParams), hipMemcpyDeviceToHost));
-        if (m->step_host->error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up at a grid barrier");
+        if (m->step_host->error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up waiting for its inputs");
     }
     return LPP_OK;
 }
@@ -464,7 +462,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     // Hand the penalty window back in the reference's order (oldest first).
     StepParams done{};
     LPP_HIP(hipMemcpy(&done, m->step, sizeof done, hipMemcpyDeviceToHost));
-    if (done.error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up at a grid barrier");
+    if (done.error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up waiting for its inputs");
     if (history_cap > 0) {
         std::vector<int> ring(static_cast<size_t>(history_cap));
         LPP_HIP(hipMemcpy(ring.data(), m->history, ring.size() * sizeof(int), hipMemcpyDeviceToHost));

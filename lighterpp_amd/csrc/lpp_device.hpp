@@ -243,13 +243,12 @@ __device__ __forceinline__ void wave_rows_dot(const char* const (&rows)[kRows], 
     for (int r = 0; r < kRows; ++r) result[r] = wave_sum(acc[r]);
 }
 
-// Accessors for values that cross workgroups INSIDE one kernel (the persistent
-// decode kernel).  The eight XCDs of the device have separate L2 caches, and
-// whole-cache acquire/release fences cost tens of microseconds per grid barrier
-// here; instead, every such value is written through and read around the
-// non-coherent cache levels with device-scope accesses (sc1), which is all a
-// consumer needs once the barrier has ordered the two sides.  kCoherent = false
-// is the ordinary access for kernels whose inputs were complete before launch.
+// Accessors for values that cross workgroups INSIDE one kernel.  The eight XCDs
+// of the device have separate L2 caches, and whole-cache acquire/release fences
+// cost tens of microseconds here; instead, every such value is written through
+// and read around the non-coherent cache levels with device-scope accesses
+// (sc1).  kCoherent = false is the ordinary access for kernels whose inputs were
+// complete before launch.
 template <bool kCoherent>
 struct Mem {
     static __device__ __forceinline__ float ld(const float* p) {

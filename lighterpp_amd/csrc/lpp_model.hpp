@@ -49,7 +49,7 @@ struct lpp_model {
     int* pinned_tokens_dev = nullptr;        // the same memory as the device addresses it
     float* att_partial = nullptr;            // split-context attention partials
     float* work_logits = nullptr;            // sampler working copy of the logits
-    unsigned* sync_words = nullptr;          // arrival counters (attention combine, grid barrier)
+    unsigned* sync_words = nullptr;          // arrival counters of the attention combine; abort flag
     float* sample_scratch = nullptr;         // 4 x kMaxChunks words
     float* gen_uniforms = nullptr;           // device copy of the per-step draws
     int gen_cap = 0;
@@ -64,7 +64,7 @@ struct lpp_model {
     const float* df_uniforms_host = nullptr; // per-step draws of the generate call in progress (host memory)
     unsigned df_base = 0;                    // sequence-number base of the next persistent launch
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
-    unsigned spin_limit = 1u << 20;          // polls a grid-barrier wait may take before giving up
+    unsigned spin_limit = 1u << 20;          // polls a wait for tagged inputs may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
     int max_splits = 1;
     bool fused_ok = false;                   // shape supported by the fused kernels
@@ -88,8 +88,8 @@ struct StepParams {
     float temperature;
     float penalty;
     float r;           // uniform draw when no uniforms[] array is attached
-    unsigned epoch;    // grid-barrier generation base of the persistent kernel
-    int error;         // set by a kernel that gave up (bounded barrier wait)
+    unsigned epoch;    // unused (kept so the record's layout stays put)
+    int error;         // set by a kernel that gave up (bounded waits)
     int freeze;        // nonzero: a step leaves token/position/window as they are (timing replays)
 };
 
