@@ -99,6 +99,7 @@ struct Blocks {
     int down;   // rows of W2
     int cls;    // rows of the classifier
     int ns_dim, ns_hidden;  // partial sums per row of a dim-column / hidden-column matrix (slices_used)
+    float dim_as_float;
     int xs_floats;
     int results_floats;
     int gather_floats;
@@ -132,6 +133,21 @@ __device__ __forceinline__ void lds_poke(unsigned* p, unsigned v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 __device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory"); }
+// A load that stays where it is written.  (An ordinary load whose value is first used behind
+// a wait loop is moved down to that use by the optimiser; fencing it in place with a memory
+// clobber instead makes the compiler wait for it on the spot and park it in private memory.)
+// The request is issued here and waited for at the first use of the value.
+__device__ __forceinline__ float pinned_load(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+}
+// (two plain floats, not a float2: an object of class type that meets another one in a
+// conditional expression is selected by address and has to live in private memory for that)
+__device__ __forceinline__ void pinned_load(const float2* p, float& x, float& y) {
+    const unsigned long long bits =
+        __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    x = __uint_as_float(static_cast<unsigned>(bits));
+    y = __uint_as_float(static_cast<unsigned>(bits >> 32));
+}
 
 // Waits on LDS words are satisfied by construction (neither kind of wavefront
 // ever waits for global memory before raising them); the bound only makes sure a
@@ -277,53 +293,96 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     unsigned cur_p = 0xffffffffu;
     floatx4 xr[kStepLoads][kF16 ? 2 : 1];  // this wavefront's slice of the staged activations
     bool more = true;
+    // Multiply the step held in ring slot k; next_meta = StepEntry::meta of the step after it.
+    auto multiply = [&](int k, unsigned next_meta) {
+        const unsigned mt = meta[k];
+        float part[kStepLoads];  // one chain of multiply-adds per chunk: they overlap instead of queueing up
+#pragma unroll
+        for (int u = 0; u < kStepLoads; ++u) {
+            if constexpr (kF16) part[u] = dot8(w[k][u], xr[u][0], xr[u][1], 0.0f);
+            else part[u] = dot4(w[k][u], xr[u][0], 0.0f);
+        }
+        static_assert(kStepLoads == 4, "the partial sums are added pairwise");
+        const float sum = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
+        if (lane == 0) results[mt & kStepSlotMask] = sum;
+        if (mt & kStepLastRow) {  // everything before the next step's phase is complete
+            const unsigned nm = next_meta;
+            const unsigned next_p = (nm & kStepValid) ? ((nm >> kStepPhaseShift) & kStepPhaseMask) : n_phases;
+            compiler_fence();
+            if (lane == 0) lds_poke(&ctl.progress[j], next_p);
+            if (trace_on && lane == 0) ctl.gemv_mark[1] = wall_clock64();
+        }
+    };
     // One pass through the ring: multiply the kDepth steps in flight and request
     // the steps whose entries sit in lanes slot0 .. slot0 + kDepth - 1 of `batch`.
+    //
+    // When a phase's activations arrive, the ring usually holds several steps of that
+    // phase whose weights came in while the wavefront was waiting.  All of them are
+    // multiplied before anything new is requested: a compute unit accepts a 4-KiB
+    // request only every hundred cycles or so, with eight wavefronts asking at once a
+    // request waits its turn for the better part of a microsecond, and rows that only
+    // need multiplying would otherwise queue behind requests for later phases.
+    unsigned ahead = 0u;  // bit k: the step in slot k has been multiplied already
+    unsigned pace = 0u;
+    constexpr int kPaceSleep = 15;
     auto run_round = [&](const uintx4& batch, int slot0) {
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) {
             const unsigned mt = meta[k];
             if (more && (mt & kStepValid)) {
-                const unsigned p = (mt >> kStepPhaseShift) & kStepPhaseMask;
-                if (p != cur_p) {  // first step of a phase: wait for its activations, take this wavefront's slice
-                    cur_p = p;
-                    const unsigned need = static_cast<unsigned>(kIoWaves) * (p + 1u);
-                    lds_wait(&ctl.error, [&]() { return static_cast<int>(lds_peek(&ctl.staged) - need) >= 0; });
-                    compiler_fence();
-                    if (trace_on && lane == 0) ctl.gemv_mark[0] = wall_clock64();
-                    const int begin = static_cast<int>(cols[k] & 0xffffu), width = static_cast<int>(cols[k] >> 16);
-                    const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (((ahead >> k) & 1u) == 0u) {
+                    const unsigned p = (mt >> kStepPhaseShift) & kStepPhaseMask;
+                    const bool phase_start = p != cur_p;
+                    if (phase_start) {  // first step of a phase: wait for its activations, take this wavefront's slice
+                        cur_p = p;
+                        const unsigned need = static_cast<unsigned>(kIoWaves) * (p + 1u);
+                        lds_wait(&ctl.error, [&]() { return static_cast<int>(lds_peek(&ctl.staged) - need) >= 0; });
+                        compiler_fence();
+                        if (trace_on && lane == 0) ctl.gemv_mark[0] = wall_clock64();
+                        const int begin = static_cast<int>(cols[k] & 0xffffu), width = static_cast<int>(cols[k] >> 16);
+                        const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                    for (int u = 0; u < kStepLoads; ++u) {
-                        const int local = u * kChunkCols + lane * kPer;
-                        const bool live = local < width;
-                        const float* src = xs + begin + (live ? local : 0);
-                        xr[u][0] = *reinterpret_cast<const floatx4*>(src);
-                        xr[u][0] = live ? xr[u][0] : zero;
-                        if constexpr (kF16) {
-                            xr[u][1] = *reinterpret_cast<const floatx4*>(src + 4);
-                            xr[u][1] = live ? xr[u][1] : zero;
+                        for (int u = 0; u < kStepLoads; ++u) {
+                            const int local = u * kChunkCols + lane * kPer;
+                            const bool live = local < width;
+                            const float* src = xs + begin + (live ? local : 0);
+                            xr[u][0] = *reinterpret_cast<const floatx4*>(src);
+                            xr[u][0] = live ? xr[u][0] : zero;
+                            if constexpr (kF16) {
+                                xr[u][1] = *reinterpret_cast<const floatx4*>(src + 4);
+                                xr[u][1] = live ? xr[u][1] : zero;
+                            }
+                        }
+                    }
+                    multiply(k, meta[(k + 1) % kDepth]);
+                    if (phase_start) {  // the steps of this phase behind it in the ring, oldest first
+                        pace |= 1u << k;
+                        bool same = true;
+#pragma unroll
+                        for (int i = 1; i < kDepth; ++i) {
+                            const int kk = (k + i) % kDepth;
+                            const unsigned m2 = meta[kk];
+                            same = same && (m2 & kStepValid) && ((m2 >> kStepPhaseShift) & kStepPhaseMask) == p;
+                            if (same) {
+                                // (the step after the newest one in the ring is the one slot k is about to request)
+                                const unsigned after =
+                                    (i + 1 < kDepth)
+                                        ? meta[(kk + 1) % kDepth]
+                                        : static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot0 + k));
+                                multiply(kk, after);
+                                ahead |= 1u << kk;
+                                pace |= 1u << kk;
+                            }
                         }
                     }
                 }
-                float part[kStepLoads];  // one chain of multiply-adds per chunk: they overlap instead of queueing up
-#pragma unroll
-                for (int u = 0; u < kStepLoads; ++u) {
-                    if constexpr (kF16) part[u] = dot8(w[k][u], xr[u][0], xr[u][1], 0.0f);
-                    else part[u] = dot4(w[k][u], xr[u][0], 0.0f);
-                }
-                static_assert(kStepLoads == 4, "the partial sums are added pairwise");
-                const float sum = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
-                if (lane == 0) results[mt & kStepSlotMask] = sum;
-                if (mt & kStepLastRow) {  // everything before the next step's phase is complete
-                    const unsigned nm = meta[(k + 1) % kDepth];
-                    const unsigned next_p = (nm & kStepValid) ? ((nm >> kStepPhaseShift) & kStepPhaseMask) : n_phases;
-                    compiler_fence();
-                    if (lane == 0) lds_poke(&ctl.progress[j], next_p);
-                    if (trace_on && lane == 0) ctl.gemv_mark[1] = wall_clock64();
-                }
+                ahead &= ~(1u << k);
             } else {
                 more = false;
+            }
+            if (kPaceSleep > 0 && ((pace >> k) & 1u)) {
+                __builtin_amdgcn_s_sleep(kPaceSleep);
+                pace &= ~(1u << k);
             }
             request(k, batch, slot0 + k);
         }
@@ -346,6 +405,18 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
 // ---------------------------------------------------------------------------
 // Exchange wavefronts: synchronisation among themselves
 // ---------------------------------------------------------------------------
+
+// Index of the calling thread among the exchange threads, computed from scratch (two
+// instructions the optimiser can neither hoist nor share).  Code that needs the index forms
+// it where it is needed: a copy kept in a register from phase to phase does not survive the
+// busiest stretches, and every reload from spill memory is a wait for all of the wavefront's
+// outstanding memory operations -- the publishing stores' acknowledgements among them, which
+// take microseconds.
+__device__ __forceinline__ int exchange_thread_index(int iw) {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return iw * kWave + lane;
+}
 
 struct Io {
     int it;        // thread index among the exchange threads
@@ -433,14 +504,15 @@ __device__ __forceinline__ bool poll_give_up(const Ctx& c, unsigned& spins) {
 }
 
 // Fetch n tagged values carrying sequence number `want` and hand each to
-// sink(i, value); the exchange threads share the range.  A thread requests up
+// sink(i, value, j, first_round), where i = thread index + (round * kBatch + j) *
+// kIoThreads and j is a constant of the unrolled code; the exchange threads share
+// the range.  A thread requests up
 // to kPollBatch values, then re-requests only those that were not there yet.
 template <int kBatch = kPollBatch, class Sink>
 __device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want, const Ctx& c, const Io& io, Sink sink) {
     // (opaque to the optimiser: otherwise the addresses of every poll in the layer loop are
     // computed once, ahead of the loop, and occupy registers for the whole token)
-    int lane_first = io.it;
-    asm volatile("" : "+v"(lane_first));
+    const int lane_first = exchange_thread_index(io.iw);
     for (int first = lane_first; first < n; first += kIoThreads * kBatch) {
         u64 got[kBatch];
         unsigned pending = 0u;
@@ -467,7 +539,7 @@ __device__ __forceinline__ void poll_values(const u64* src, int n, unsigned want
 #pragma unroll
         for (int j = 0; j < kBatch; ++j) {
             const int i = first + j * kIoThreads;
-            if (i < n) sink(i, value_of(got[j]));
+            if (i < n) sink(i, value_of(got[j]), j, first == lane_first);
         }
     }
 }
@@ -516,52 +588,59 @@ struct Lds {
 __device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, int n, unsigned want) {
     const int n_pad = (n + 7) & ~7;
     for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
-    poll_values<8192 / kIoThreads>(src, n, want, c, io, [&](int i, float v) { xs[i] = v; });  // 8192 values in one go
+    poll_values<8192 / kIoThreads>(src, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });  // 8192 values in one go
     mark(c, io, 1);
     signal_staged(c.ctl);
 }
 
 // xraw = the input vector (tagged x, or the embedding row for layer 0);
-// xs = rmsnorm(xraw) * gain, ops.cpp:20-32.
-__device__ __forceinline__ void stage_norm(Ctx& c, Io& io, const Lds& l, const u64* tagged_x, const float* plain_x, int n,
-                                           unsigned want, const float* gain) {
+// xs = xraw * gain, and the return value is 1 / sqrt(mean(xraw^2) + 1e-5): the rows of
+// the GEMV that follows are those of ops.cpp:20-32 once multiplied by it.  (W.(s.g.x) =
+// s.(W.(g.x)): the streaming wavefronts can start the moment the last value is in,
+// without waiting for a sum over all of them, a reduction across the exchange
+// wavefronts that would otherwise sit in every layer's dependency chain twice; it
+// now runs while they multiply.)
+__device__ __forceinline__ float stage_norm(Ctx& c, Io& io, const Lds& l, const u64* tagged_x, const float* plain_x, int n,
+                                            unsigned want, const float* gain) {
 #pragma clang fp contract(off)
     float* xraw = l.xraw;
     float* xs = l.xs;
+    const int it = exchange_thread_index(io.iw);
     // The gains do not depend on anything: request this thread's first few before polling, so that
-    // their memory latency is spent while the inputs are still on their way (the fence keeps the
-    // requests from being moved down to their first use).
+    // their memory latency is spent while the inputs are still on their way.
     constexpr int kEarly = 8;
     float early_gain[kEarly];
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
-        const int i = io.it + e * kIoThreads;
-        early_gain[e] = (i < n) ? gain[i] : 0.0f;
+        const int i = it + e * kIoThreads;
+        early_gain[e] = (i < n) ? pinned_load(gain + i) : 0.0f;
     }
-    compiler_fence();
+    const int n_pad = (n + 7) & ~7;
+    for (int i = n + it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
+    float ss = 0.0f;
+    auto take = [&](int i, float v, float g) {
+        xraw[i] = v;
+        xs[i] = v * g;
+        ss += v * v;
+    };
     if (plain_x != nullptr) {
-        for (int i = io.it; i < n; i += kIoThreads) xraw[i] = plain_x[i];
+#pragma unroll
+        for (int e = 0; e < kEarly; ++e) {
+            const int i = it + e * kIoThreads;
+            if (i < n) take(i, plain_x[i], early_gain[e]);
+        }
+        for (int i = it + kEarly * kIoThreads; i < n; i += kIoThreads) take(i, plain_x[i], gain[i]);
     } else {
-        poll_values(tagged_x, n, want, c, io, [&](int i, float v) { xraw[i] = v; });
+        static_assert(kEarly == kPollBatch, "the first round of polls covers exactly the values whose gains were requested early");
+        poll_values(tagged_x, n, want, c, io,
+                    [&](int i, float v, int j, bool first_round) { take(i, v, first_round ? early_gain[j] : gain[i]); });
     }
     mark(c, io, 1);
-    float ss = 0.0f;
-    for (int i = io.it; i < n; i += kIoThreads) {  // the index set this thread wrote
-        const float v = xraw[i];
-        ss += v * v;
-    }
-    ss = io_sum(c.ctl, io, ss);
-    ss /= static_cast<float>(n);
-    ss += 1e-5f;
-    const float scale = 1.0f / sqrtf(ss);
-    const int n_pad = (n + 7) & ~7;
-#pragma unroll
-    for (int e = 0; e < kEarly; ++e) {
-        const int i = io.it + e * kIoThreads;
-        if (i < n_pad) xs[i] = (i < n) ? xraw[i] * scale * early_gain[e] : 0.0f;
-    }
-    for (int i = io.it + kEarly * kIoThreads; i < n_pad; i += kIoThreads) xs[i] = (i < n) ? xraw[i] * scale * gain[i] : 0.0f;
     signal_staged(c.ctl);
+    ss = io_sum(c.ctl, io, ss);
+    ss /= c.b.dim_as_float;  // n, converted on the host: here the conversion's result would be kept in (and spilled from) a vector register
+    ss += 1e-5f;
+    return 1.0f / sqrtf(ss);
 }
 
 // ---------------------------------------------------------------------------
@@ -583,7 +662,7 @@ template <class RowFn>
 __device__ __forceinline__ void finished_rows(Ctx& c, Io& io, int gphase, int nrows, RowFn fn) {
     wait_gemv(c.ctl, io, gphase);
     mark(c, io, 3);
-    for (int r = io.it; r < nrows; r += kIoThreads) fn(r);
+    for (int r = exchange_thread_index(io.iw); r < nrows; r += kIoThreads) fn(r);
 }
 
 __device__ __forceinline__ int block_rows(int total, int block, int wg) {
@@ -597,28 +676,38 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     const int dim = a.dim, kv_dim = a.kv_dim, hs = a.head_size;
     const float* emb_row = (layer == 0) ? a.emb + static_cast<size_t>(c.token) * dim : nullptr;
     mark(c, io, 0);
-    stage_norm(c, io, l, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
-               a.rms_att + static_cast<size_t>(layer) * dim);
+    const float scale = stage_norm(c, io, l, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
+                                   a.rms_att + static_cast<size_t>(layer) * dim);
     mark(c, io, 2);
     const int row0 = c.wg * c.b.qkv;
     const int nrows = block_rows(dim + 2 * kv_dim, c.b.qkv, c.wg);
     const float2* cs_row = a.rope + static_cast<size_t>(c.pos) * (hs / 2);
     const unsigned tag = c.seq(layer, kQkv);
     // (cos, sin) of this thread's first row: requested while the streaming wavefronts still multiply
-    float2 cs_first = make_float2(1.0f, 0.0f);
-    {
-        const int g = row0 + io.it;
-        if (io.it < nrows && g < dim + kv_dim) cs_first = cs_row[((((g < dim) ? g : g - dim) & ~1) % hs) >> 1];
-    }
-    compiler_fence();
-    finished_rows(c, io, 4 * layer + kGQkv, nrows, [&](int r) {
+    const int first_row = io.it;
+    const int first_g = row0 + first_row;
+    const bool first_rotates = first_row < nrows && first_g < dim + kv_dim;
+    // (a valid address either way, so that the request does not sit behind a branch)
+    float first_cos, first_sin;
+    pinned_load(cs_row + (first_rotates ? ((((first_g < dim) ? first_g : first_g - dim) & ~1) % hs) >> 1 : 0), first_cos, first_sin);
+    // (a plain loop, not finished_rows with a closure: a local captured by reference is kept in
+    // private memory across the wait, and private memory shares the load counter)
+    wait_gemv(c.ctl, io, 4 * layer + kGQkv);
+    mark(c, io, 3);
+    for (int r = exchange_thread_index(io.iw); r < nrows; r += kIoThreads) {
         const int g = row0 + r;
-        const float mine = row_result(l.results, r, c.b.ns_dim), neighbour = row_result(l.results, r ^ 1, c.b.ns_dim);
+        const float mine = row_result(l.results, r, c.b.ns_dim) * scale,
+                    neighbour = row_result(l.results, r ^ 1, c.b.ns_dim) * scale;
         float out = mine;
         if (g < dim + kv_dim) {  // ops.cpp:36-52 on the pair (i, i+1)
             const int gi = (g < dim) ? g : g - dim;
-            const float2 cs = (r == io.it) ? cs_first : cs_row[((gi & ~1) % hs) >> 1];
-            out = (gi & 1) ? neighbour * cs.y + mine * cs.x : mine * cs.x - neighbour * cs.y;
+            float cos_t = first_cos, sin_t = first_sin;
+            if (r != first_row) {
+                const float2 cs = cs_row[((gi & ~1) % hs) >> 1];
+                cos_t = cs.x;
+                sin_t = cs.y;
+            }
+            out = (gi & 1) ? neighbour * sin_t + mine * cos_t : mine * cos_t - neighbour * sin_t;
         }
         if (g < dim) {
             publish(c.t.q + g, out, tag);
@@ -633,7 +722,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
             (is_k ? a.k : a.v)[i] = out;
             (is_k ? a.key_cache : a.value_cache)[dst] = f32_to_f16_bits(out);
         }
-    });
+    }
     mark(c, io, 4);
     ++c.phase_index;
 }
@@ -657,7 +746,8 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
 #pragma clang fp contract(off)
     const DecodeArgs& a = c.a;
     mark(c, io, 0);
-    stage_norm(c, io, l, c.t.x, nullptr, a.dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * a.dim);
+    const float scale =
+        stage_norm(c, io, l, c.t.x, nullptr, a.dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * a.dim);
     mark(c, io, 2);
     const int unit0 = c.wg * c.b.gu;
     const int units = block_rows(a.hidden, c.b.gu, c.wg);
@@ -665,7 +755,7 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
     finished_rows(c, io, 4 * layer + kGGateUp, 2 * units, [&](int r) {
         if (r & 1) return;  // the gate row's thread finishes the unit
         const int u = r >> 1;
-        const float gate = row_result(l.results, r, c.b.ns_dim), up = row_result(l.results, r + 1, c.b.ns_dim);
+        const float gate = row_result(l.results, r, c.b.ns_dim) * scale, up = row_result(l.results, r + 1, c.b.ns_dim) * scale;
         const float sigma = 1.0f / (1.0f + expf(-gate));  // ops.cpp:80-85
         publish(c.t.hb + unit0 + u, (gate * sigma) * up, tag);
     });
@@ -861,7 +951,7 @@ __device__ __forceinline__ void att_combine(Ctx& c, Io& io, const Lds& l, int la
     const unsigned tag_out = c.seq(layer, kAtt);
     io_sync(c.ctl, io);  // earlier readers of gather have left
     const u64* src = c.t.part + static_cast<size_t>(h) * c.t.splits_cap * stride;
-    poll_values(src, nsplits * stride, tag_out, c, io, [&](int i, float v) { l.gather[i] = v; });
+    poll_values(src, nsplits * stride, tag_out, c, io, [&](int i, float v, int, bool) { l.gather[i] = v; });
     io_sync(c.ctl, io);
     if (io.it < hs) {
         float top = -INFINITY;
@@ -892,6 +982,7 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
     mark(c, io, 0);
     for (int item = c.wg; item < items; item += c.nwg) {
         const int h = item / nsplits, split = item - h * nsplits;
+        io.it = exchange_thread_index(io.iw);
         // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
         if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first);
         else att_item<16>(c, io, l, layer, h, split, nsplits, npos, first);
@@ -900,6 +991,7 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
     if (nsplits > 1) {
         for (int item = c.wg; item < items; item += c.nwg) {
             const int h = item / nsplits, split = item - h * nsplits;
+            io.it = exchange_thread_index(io.iw);
             if (split == 0) att_combine(c, io, l, layer, h, nsplits);
         }
     }
@@ -923,7 +1015,7 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     const int vocab = a.vocab, dim = a.dim, wg = c.wg, nwg = c.nwg;
     const int it = io.it;
     mark(c, io, 0);
-    stage_norm(c, io, l, c.t.x, nullptr, dim, c.seq(a.n_layers - 1, kDown), a.rms_final);
+    const float scale = stage_norm(c, io, l, c.t.x, nullptr, dim, c.seq(a.n_layers - 1, kDown), a.rms_final);
     mark(c, io, 2);
     wait_gemv(ctl, io, 4 * a.n_layers);
     mark(c, io, 3);
@@ -932,7 +1024,7 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     const int r1 = r0 + n;
     float* lg = l.xs + 4 * nwg;  // beside the sampler tables; the streaming wavefronts are done with xs
     for (int i = it; i < n; i += kIoThreads) {
-        lg[i] = row_result(l.results, i, c.b.ns_dim);
+        lg[i] = row_result(l.results, i, c.b.ns_dim) * scale;
         a.logits[r0 + i] = lg[i];  // raw logits stay readable after the token
     }
     mark(c, io, 4);
@@ -999,7 +1091,7 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     float* st_sum = l.xs + nwg;      // [nwg]
     float* st_arg = l.xs + 2 * nwg;  // [nwg] (int bits)
     float* st_cum = l.xs + 3 * nwg;  // [nwg] mass before the workgroup
-    poll_values(c.t.stats, nwg * 4, tag, c, io, [&](int i, float v) {
+    poll_values(c.t.stats, nwg * 4, tag, c, io, [&](int i, float v, int, bool) {
         const int w = i >> 2, f = i & 3;
         if (f == 0) st_max[w] = v;
         else if (f == 1) st_sum[w] = v;
@@ -1100,7 +1192,7 @@ __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
     // The thread index is made opaque before every phase: per-thread addresses are then formed
     // where they are used instead of once for the whole token, where they would occupy (and
     // overflow) the register file for the length of the layer loop.
-    auto fresh = [&]() { asm volatile("" : "+v"(io.it)); };
+    auto fresh = [&]() { io.it = exchange_thread_index(io.iw); };
     for (int layer = 0; layer < a.n_layers; ++layer) {
         fresh();
         io_qkv(c, io, l, layer);
@@ -1192,6 +1284,7 @@ Plan plan_for(const lpp_model* m) {
     const int chunk_cols = c.weight_precision == LPP_WEIGHT_FP16 ? 512 : 256;
     b.ns_dim = df::slices_used(c.dim, chunk_cols);
     b.ns_hidden = df::slices_used(c.hidden_dim, chunk_cols);
+    b.dim_as_float = static_cast<float>(c.dim);
     int slots = b.qkv * b.ns_dim;  // one partial sum per row and column slice
     if (b.o * b.ns_dim > slots) slots = b.o * b.ns_dim;
     if (2 * b.gu * b.ns_dim > slots) slots = 2 * b.gu * b.ns_dim;
