@@ -356,7 +356,12 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
                     }
                     multiply(k, meta[(k + 1) % kDepth]);
                     if (phase_start) {  // the steps of this phase behind it in the ring, oldest first
-                        pace |= 1u << k;
+                        // The refills are spaced out only when this burst was all the wavefront had to do in
+                        // the phase: the exchange wavefronts publish next, and their stores should not queue
+                        // behind eight wavefronts' requests.  In a longer phase the requests are this phase's
+                        // own rows and go out at once.
+                        unsigned burst = 1u << k;
+                        bool ended = (mt & kStepLastRow) != 0u;
                         bool same = true;
 #pragma unroll
                         for (int i = 1; i < kDepth; ++i) {
@@ -371,9 +376,11 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
                                         : static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot0 + k));
                                 multiply(kk, after);
                                 ahead |= 1u << kk;
-                                pace |= 1u << kk;
+                                burst |= 1u << kk;
+                                ended = ended || (m2 & kStepLastRow) != 0u;
                             }
                         }
+                        if (ended) pace |= burst;
                     }
                 }
                 ahead &= ~(1u << k);
