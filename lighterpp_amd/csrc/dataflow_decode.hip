@@ -16,15 +16,18 @@
 // therefore split into two kinds of wavefronts:
 //
 //   streaming wavefronts  walk their fixed list of weight rows across ALL phases
-//       and layers of the token with kDepth 2-KiB steps always in flight in
+//       and layers of the token with kDepth 4-KiB steps always in flight in
 //       registers.  They never touch global memory otherwise: activations come
 //       from LDS, results go to LDS, and they only ever wait on an LDS flag.
 //       While the dependency chain is stalled they already hold the next
 //       phases' weights.
-//   exchange wavefronts   poll the tagged inputs of a phase (their loads never
-//       queue behind weight traffic), normalise and stage them in LDS, raise the
-//       flag, later pick up the row results, apply the phase's epilogue (RoPE,
-//       SwiGLU, residual) and publish.  They also run attention and the sampler.
+//   exchange wavefronts   poll the tagged inputs of a phase, stage them in LDS
+//       (times the norm gain where a norm precedes the GEMV), raise the flag,
+//       later pick up the row results, apply the phase's epilogue (the norm's
+//       1/rms, RoPE, SwiGLU, residual) and publish.  They also run attention and
+//       the sampler.  What they send and poll does queue behind weight requests
+//       already in flight: the streaming wavefronts hold their refills back for
+//       a moment when the exchange wavefronts are about to publish.
 //
 // Sequence numbers grow monotonically for the life of a model (the host hands
 // every launch its base and advances it by the number of phases), so a stale
