@@ -14,6 +14,8 @@
  * reference's src/kernels.cuh:24-36 (the operator surface src/model.cpp calls).
  * Section B replaces the model-level functions of src/model.h:117-164.
  * Section C is plumbing the reference gets from the CUDA runtime directly.
+ * Section D is what sits either side of the path in the reference: the llama2.c
+ * checkpoint reader (src/loader.cpp) and the driver loop (src/main.cpp).
  */
 #ifndef LPP_H
 #define LPP_H
@@ -228,6 +230,52 @@ lpp_status lpp_generate(lpp_model *m, int first_token, int start_pos, int n_step
                         float temperature, float topp, float penalty, int *history,
                         int *history_len, int history_cap, const float *uniforms,
                         int *out_tokens, lpp_gen_stats *stats);
+
+/* ===================================================================== */
+/* D. The callers either side of the path (src/main.cpp, src/loader.cpp)  */
+/* ===================================================================== */
+
+/* A llama2.c checkpoint mapped into host memory: seven-int header (dim,
+ * hidden_dim, n_layers, n_heads, n_kv_heads, vocab_size, seq_len) followed by fp32
+ * tensors in the order of LPP_T_TOKEN_EMBEDDING .. LPP_T_RMS_FINAL, classifier tied
+ * to the embedding.  Host code only; needs no GPU. */
+typedef struct lpp_checkpoint lpp_checkpoint;
+/* load_model_file (loader.cpp:134-172): maps the file, reads the header, sets
+ * rope_base 10000; weight_precision is LPP_WEIGHT_FP32.  Unlike the reference it
+ * checks that every field is positive and that the file holds all its tensors. */
+lpp_status lpp_checkpoint_open(lpp_checkpoint **out, const char *path);
+/* free_model_file (loader.cpp:174-177). */
+lpp_status lpp_checkpoint_close(lpp_checkpoint *ck);
+lpp_status lpp_checkpoint_config(const lpp_checkpoint *ck, lpp_config *cfg);
+/* Where checkpoint_init_weights (loader.cpp:18-66) points the named tensor:
+ * host address inside the mapping and number of floats.  LPP_T_WCLS answers with
+ * the embedding table (:66). */
+lpp_status lpp_checkpoint_tensor(const lpp_checkpoint *ck, int tensor, const float **host,
+                                 size_t *count);
+/* lpp_model_create + the upload half of checkpoint_init_weights (loader.cpp:73-131)
+ * + lpp_model_tie_classifier. */
+lpp_status lpp_model_load_checkpoint(lpp_model **out, const lpp_checkpoint *ck);
+
+typedef struct lpp_run_result {
+    int n_tokens;        /* ids generated before the stop (what main.cpp prints)          */
+    int final_pos;
+    int stopped_by_eos;  /* an id of main.cpp:211-213 (2, 128001, 128009) ended the loop  */
+    int reported_count;  /* "Tokens generated" as main.cpp:229 counts: final_pos - n_prompt */
+    int history_len;     /* the penalty window as the loop left it                        */
+    int history[64];
+    double wall_seconds; /* steady_clock around the generation loop (main.cpp:196-226)    */
+} lpp_run_result;
+
+/* The driver loop of main.cpp:139-232 without text: prefill by decode of
+ * prompt[0 .. n_prompt-1) (penalty 1.1, sampled ids dropped), then generation from
+ * the last prompt id (penalty 1.05) until position `steps` or an end-of-sequence
+ * id; 64-entry sliding penalty window.  prompt == NULL stands for the single id 1
+ * (main.cpp:147-151).  uniforms[pos] is the draw of the forward at position pos
+ * (the reference draws inside every forward, prefill included).  Positions beyond
+ * seq_len are an error here (the reference overruns its cache). */
+lpp_status lpp_run(lpp_model *m, const int *prompt, int n_prompt, int steps, float temperature,
+                   float topp, const float *uniforms, int *out_tokens, int out_capacity,
+                   lpp_run_result *res);
 
 /* Per-kernel timing of the fused path, measured with HIP events on the launch
  * stream: each kernel class is recorded n_layers times (one launch per layer,

@@ -47,6 +47,13 @@ class LppGenStats(C.Structure):
                 ("kernel_launches", C.c_int), ("tokens", C.c_int)]
 
 
+class LppRunResult(C.Structure):
+    """lpp_run_result: what the driver loop of src/main.cpp:139-232 leaves behind."""
+    _fields_ = [("n_tokens", C.c_int), ("final_pos", C.c_int), ("stopped_by_eos", C.c_int),
+                ("reported_count", C.c_int), ("history_len", C.c_int), ("history", C.c_int * 64),
+                ("wall_seconds", C.c_double)]
+
+
 class LppKernelTime(C.Structure):
     _fields_ = [("name", C.c_char * 32), ("launches_per_token", C.c_int), ("avg_ms", C.c_double),
                 ("bytes_per_launch", C.c_double)]
@@ -91,6 +98,13 @@ SIGNATURES = {
     "lpp_generate": (_i, [_vp, _i, _i, _i, _f, _f, _f, _vp, _ip, _i, _vp, _vp, C.POINTER(LppGenStats)]),
     "lpp_profile_kernels": (_i, [_vp, _i, _i, C.POINTER(LppKernelTime), _i, _ip]),
     "lpp_trace_token": (_i, [_vp, _i, C.POINTER(C.c_ulonglong), _i, _ip, _ip]),
+    # D. checkpoint reader and driver loop
+    "lpp_checkpoint_open": (_i, [C.POINTER(_vp), C.c_char_p]),
+    "lpp_checkpoint_close": (_i, [_vp]),
+    "lpp_checkpoint_config": (_i, [_vp, C.POINTER(LppConfig)]),
+    "lpp_checkpoint_tensor": (_i, [_vp, _i, C.POINTER(_vp), C.POINTER(_sz)]),
+    "lpp_model_load_checkpoint": (_i, [C.POINTER(_vp), _vp]),
+    "lpp_run": (_i, [_vp, _vp, _i, _i, _f, _f, _vp, _vp, _i, C.POINTER(LppRunResult)]),
     # C. runtime
     "lpp_last_error": (C.c_char_p, []),
     "lpp_version": (C.c_char_p, []),

@@ -475,7 +475,7 @@ __device__ __forceinline__ void signal_staged(Control& ctl) {
 }
 
 // Wait until every streaming wavefront has completed GEMV phase p.
-__device__ __forceinline__ void wait_gemv(Control& ctl, const Io& io, int p) {
+__device__ __forceinline__ void wait_gemv(Control& ctl, int p) {
     const unsigned need = static_cast<unsigned>(p + 1);
     static_assert(kGemvWaves == 8, "progress is read as two 16-byte vectors");
     lds_wait(&ctl.error, [&]() {
@@ -670,7 +670,7 @@ __device__ __forceinline__ float row_result(const float* results, int r, int nsl
 // earlier, and the extra polling traffic cost more than the head start gained.)
 template <class RowFn>
 __device__ __forceinline__ void finished_rows(Ctx& c, Io& io, int gphase, int nrows, RowFn fn) {
-    wait_gemv(c.ctl, io, gphase);
+    wait_gemv(c.ctl, gphase);
     mark(c, io, 3);
     for (int r = exchange_thread_index(io.iw); r < nrows; r += kIoThreads) fn(r);
 }
@@ -702,7 +702,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     pinned_load(cs_row + (first_rotates ? ((((first_g < dim) ? first_g : first_g - dim) & ~1) % hs) >> 1 : 0), first_cos, first_sin);
     // (a plain loop, not finished_rows with a closure: a local captured by reference is kept in
     // private memory across the wait, and private memory shares the load counter)
-    wait_gemv(c.ctl, io, 4 * layer + kGQkv);
+    wait_gemv(c.ctl, 4 * layer + kGQkv);
     mark(c, io, 3);
     for (int r = exchange_thread_index(io.iw); r < nrows; r += kIoThreads) {
         const int g = row0 + r;
@@ -1027,7 +1027,7 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     mark(c, io, 0);
     const float scale = stage_norm(c, io, l, c.t.x, nullptr, dim, c.seq(a.n_layers - 1, kDown), a.rms_final);
     mark(c, io, 2);
-    wait_gemv(ctl, io, 4 * a.n_layers);
+    wait_gemv(ctl, 4 * a.n_layers);
     mark(c, io, 3);
     const int r0 = min(vocab, wg * c.b.cls);
     const int n = block_rows(vocab, c.b.cls, wg);

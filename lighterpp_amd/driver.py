@@ -1,0 +1,59 @@
+"""Command-line driver over liblpp_hip.so: what src/main.cpp does with a llama2.c
+checkpoint, minus the tokenizer (ids in, ids out).
+
+    python -m lighterpp_amd.driver model.bin [--prompt-ids 1,15,7] [--steps 200]
+                                   [--temperature 0.8] [--seed 1] [--path persistent]
+
+Prefill by decode, 64-entry sliding penalty window (1.1 while reading the prompt,
+1.05 while generating), stop at position --steps or at an end-of-sequence id, then the
+statistics block of main.cpp:228-232.
+"""
+from __future__ import annotations
+
+import argparse
+import sys
+
+import numpy as np
+
+from . import capi
+from .model import Checkpoint, Model
+
+PATHS = {"ops": capi.PATH_OPS, "fused": capi.PATH_FUSED, "persistent": capi.PATH_PERSISTENT}
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="lighterpp_amd.driver", description=__doc__.split("\n\n")[0])
+    ap.add_argument("checkpoint", help="llama2.c .bin file")
+    ap.add_argument("--prompt-ids", default="", help="comma-separated token ids (default: the single id 1)")
+    ap.add_argument("--steps", type=int, default=200, help="last position + 1 (main.cpp:155)")
+    ap.add_argument("--temperature", type=float, default=0.8)
+    ap.add_argument("--seed", type=int, default=1, help="seed of the per-step uniform draws")
+    ap.add_argument("--path", default="persistent", choices=list(PATHS))
+    args = ap.parse_args(argv)
+
+    capi.init(0)
+    ck = Checkpoint(args.checkpoint)
+    c = ck.config
+    print("--- Model Configuration ---")
+    print(f"Dim: {c.dim}\nHidden Dim: {c.hidden_dim}\nLayers: {c.n_layers}\nHeads: {c.n_heads}\nKV Heads: {c.n_kv_heads}")
+    print(f"Vocab: {c.vocab_size}\nSeq Len: {c.seq_len}\nRoPE Base: {c.rope_base:.0f}\nTemperature: {args.temperature:.2f}")
+    model = Model.from_checkpoint(ck)
+    model.set_path(PATHS[args.path])
+    prompt = [int(t) for t in args.prompt_ids.split(",") if t.strip()] or None
+    steps = min(args.steps, c.seq_len)
+    uniforms = capi.synth_uniform_f32(steps, args.seed)
+    print("\n--- Running Inference ---")
+    tokens, res = model.run(prompt, steps, args.temperature, 1.0, uniforms)
+    print(" ".join(str(int(t)) for t in tokens))
+    print("\n--- Statistics ---")
+    print(f"Tokens generated: {res.reported_count}")
+    print(f"Elapsed time: {res.wall_seconds:.2f} s")
+    if res.wall_seconds > 0:
+        print(f"Tokens per second: {res.reported_count / res.wall_seconds:.2f} tok/s")
+    model.close()
+    ck.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -94,10 +94,66 @@ def synth_tensor(shape: Shape, t: int, seed: int) -> np.ndarray:
     return capi.synth_normal_f32(n, stream, 0.02).reshape(dims)
 
 
+def write_checkpoint(path, shape: Shape, tensors: dict) -> None:
+    """Writes a llama2.c checkpoint as the reference reads it (src/loader.cpp:134-172,
+    18-66): seven ints, then the eleven fp32 tensors back to back, classifier tied."""
+    assert not shape.fp16 and shape.tied, "the format holds fp32 tensors and a tied classifier"
+    with open(path, "wb") as f:
+        f.write(np.array([shape.dim, shape.hidden_dim, shape.n_layers, shape.n_heads, shape.n_kv_heads,
+                          shape.vocab_size, shape.seq_len], dtype=np.int32).tobytes())
+        for t in range(capi.T_WCLS):
+            a = np.ascontiguousarray(tensors[t], dtype=np.float32)
+            assert a.shape == shape.tensor_shape(t), (t, a.shape)
+            f.write(a.tobytes())
+
+
+class Checkpoint:
+    """A llama2.c checkpoint mapped by lpp_checkpoint_open (host code, no GPU)."""
+
+    def __init__(self, path):
+        self.lib = capi.load()
+        h = C.c_void_p()
+        capi.check(self.lib.lpp_checkpoint_open(C.byref(h), str(path).encode()))
+        self.handle = h
+        cfg = capi.LppConfig()
+        capi.check(self.lib.lpp_checkpoint_config(self.handle, C.byref(cfg)))
+        self.config = cfg
+        self.shape = Shape(cfg.dim, cfg.hidden_dim, cfg.n_layers, cfg.n_heads, cfg.n_kv_heads, cfg.vocab_size,
+                           cfg.seq_len, cfg.rope_base, fp16=cfg.weight_precision == capi.WEIGHT_FP16, tied=True)
+
+    def tensor(self, t: int) -> np.ndarray:
+        """Copy of the named tensor, shaped."""
+        p, n = C.c_void_p(), C.c_size_t()
+        capi.check(self.lib.lpp_checkpoint_tensor(self.handle, t, C.byref(p), C.byref(n)))
+        flat = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_float)), shape=(n.value,))
+        return flat.reshape(self.shape.tensor_shape(t)).copy()
+
+    def tensor_offset(self, t: int) -> int:
+        """Floats between the first weight of the file and the named tensor."""
+        p, n, p0 = C.c_void_p(), C.c_size_t(), C.c_void_p()
+        capi.check(self.lib.lpp_checkpoint_tensor(self.handle, t, C.byref(p), C.byref(n)))
+        capi.check(self.lib.lpp_checkpoint_tensor(self.handle, capi.T_TOKEN_EMBEDDING, C.byref(p0), C.byref(n)))
+        return (p.value - p0.value) // 4
+
+    def close(self) -> None:
+        if self.handle:
+            self.lib.lpp_checkpoint_close(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Model:
-    def __init__(self, shape: Shape):
+    def __init__(self, shape: Shape, _handle=None):
         self.shape = shape
         lib = capi.load()
+        if _handle is not None:
+            self.handle, self.lib = _handle, lib
+            return
         cfg = capi.LppConfig(shape.dim, shape.hidden_dim, shape.n_layers, shape.n_heads, shape.n_kv_heads,
                              shape.vocab_size, shape.seq_len, shape.rope_base,
                              capi.WEIGHT_FP16 if shape.fp16 else capi.WEIGHT_FP32)
@@ -105,6 +161,13 @@ class Model:
         capi.check(lib.lpp_model_create(C.byref(h), C.byref(cfg)))
         self.handle = h
         self.lib = lib
+
+    @classmethod
+    def from_checkpoint(cls, ck: "Checkpoint") -> "Model":
+        """lpp_model_load_checkpoint: create, upload every tensor, tie the classifier."""
+        h = C.c_void_p()
+        capi.check(ck.lib.lpp_model_load_checkpoint(C.byref(h), ck.handle))
+        return cls(ck.shape, _handle=h)
 
     def close(self) -> None:
         if self.handle:
@@ -181,6 +244,23 @@ class Model:
                                          C.c_void_p(hist.ctypes.data), C.byref(hlen), history_cap, up,
                                          C.c_void_p(out.ctypes.data), C.byref(stats)))
         return out, hist[:hlen.value].tolist(), stats
+
+    def run(self, prompt, steps: int, temperature: float = 0.0, topp: float = 1.0, uniforms=None):
+        """lpp_run, the driver loop of src/main.cpp:139-232.  Returns (generated ids, LppRunResult)."""
+        out = np.empty(max(steps, 1), dtype=np.int32)
+        pp, pn = None, 0
+        if prompt is not None and len(prompt) > 0:
+            pr = np.ascontiguousarray(prompt, dtype=np.int32)
+            pp, pn = C.c_void_p(pr.ctypes.data), int(pr.size)
+        up = None
+        if uniforms is not None:
+            u = np.ascontiguousarray(uniforms, dtype=np.float32)
+            assert u.size >= steps
+            up = C.c_void_p(u.ctypes.data)
+        res = capi.LppRunResult()
+        capi.check(self.lib.lpp_run(self.handle, pp, pn, steps, temperature, topp, up, C.c_void_p(out.ctypes.data),
+                                    int(out.size), C.byref(res)))
+        return out[:res.n_tokens].copy(), res
 
     def profile_kernels(self, pos: int, reps: int = 20) -> list:
         """[(name, launches_per_token, avg_ms, bytes_per_launch)] for the fused path."""

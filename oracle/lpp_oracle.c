@@ -434,3 +434,104 @@ void orc_history_push(int *history, int *len, int capacity, int token)
         history[capacity - 1] = token;
     }
 }
+
+/* main.cpp:139-232 without text.  One uniform per forward() call, in call order
+ * (the reference draws rand() inside sample(), model.cpp:291, also for the
+ * prefill forwards whose result it discards, and only when temperature != 0):
+ * uniforms[pos]. */
+int orc_run(const int *prompt, int n_prompt, int steps, float temperature, float topp,
+            const float *uniforms, orc_state *s, const orc_weights *w, const orc_config *p,
+            int *out_tokens, int out_capacity, orc_run_result *res)
+{
+    enum { HISTORY_LEN = 64 };                     /* main.cpp:158 */
+    int history[HISTORY_LEN];
+    int current_history_len = 0;
+    int bos = 1;                                   /* main.cpp:147-151 */
+    if (prompt == NULL || n_prompt <= 0) {
+        prompt = &bos;
+        n_prompt = 1;
+    }
+    int pos = 0;
+    int n_out = 0;
+    /* 1. prefill, main.cpp:163-180: penalty 1.1f, sampled token discarded */
+    for (int i = 0; i < n_prompt - 1; i++) {
+        orc_history_push(history, &current_history_len, HISTORY_LEN, prompt[i]);
+        (void)orc_forward(prompt[i], pos, s, w, p, temperature, topp, 1.1f, history, current_history_len,
+                          uniforms ? uniforms[pos] : 0.0f);
+        pos++;
+    }
+    /* 2. main.cpp:182-190 */
+    int token = prompt[n_prompt - 1];
+    orc_history_push(history, &current_history_len, HISTORY_LEN, token);
+    /* 3. generation, main.cpp:199-223: penalty 1.05f; the end-of-sequence ids stop the loop
+     *    after they entered the window and before pos advances */
+    int stopped = 0;
+    for (; pos < steps; pos++) {
+        token = orc_forward(token, pos, s, w, p, temperature, topp, 1.05f, history, current_history_len,
+                            uniforms ? uniforms[pos] : 0.0f);
+        orc_history_push(history, &current_history_len, HISTORY_LEN, token);
+        if (token == 2 || token == 128001 || token == 128009) {  /* main.cpp:211-213, the id half of each test */
+            stopped = 1;
+            break;
+        }
+        if (n_out < out_capacity) out_tokens[n_out] = token;
+        n_out++;
+    }
+    if (res) {
+        res->n_tokens = n_out;
+        res->final_pos = pos;
+        res->stopped_by_eos = stopped;
+        res->reported_count = pos - n_prompt;      /* main.cpp:229 */
+        res->history_len = current_history_len;
+        memcpy(res->history, history, sizeof(history));
+    }
+    return 0;
+}
+
+/* load_model_file (loader.cpp:134-172) + checkpoint_init_weights (loader.cpp:18-66):
+ * seven ints, then fp32 tensors back to back in the order below; the classifier is
+ * the embedding table.  Offsets and counts are in floats from the first weight. */
+int orc_checkpoint_parse(const void *file_bytes, size_t file_size, orc_config *cfg,
+                         size_t offsets[12], size_t counts[12])
+{
+    if (file_size < 28) return -1;
+    int header[7];
+    memcpy(header, file_bytes, sizeof(header));
+    cfg->dim = header[0];
+    cfg->hidden_dim = header[1];
+    cfg->n_layers = header[2];
+    cfg->n_heads = header[3];
+    cfg->n_kv_heads = header[4];
+    cfg->vocab_size = header[5];
+    cfg->seq_len = header[6];
+    cfg->rope_base = 10000.0f;                     /* loader.cpp:163 */
+    if (cfg->dim <= 0 || cfg->hidden_dim <= 0 || cfg->n_layers <= 0 || cfg->n_heads <= 0 ||
+        cfg->n_kv_heads <= 0 || cfg->vocab_size <= 0 || cfg->seq_len <= 0)
+        return -2;
+    const size_t dim = (size_t)cfg->dim, hidden = (size_t)cfg->hidden_dim, L = (size_t)cfg->n_layers;
+    const size_t head_size = dim / (size_t)cfg->n_heads;           /* loader.cpp:19 */
+    const size_t q_cols = (size_t)cfg->n_heads * head_size, kv_cols = (size_t)cfg->n_kv_heads * head_size;
+    const size_t n[11] = {
+        (size_t)cfg->vocab_size * dim,  /* token_embedding_table  :22-23 */
+        L * dim,                        /* rms_att_weight         :26-27 */
+        L * dim * q_cols,               /* wq                     :30-31 */
+        L * dim * kv_cols,              /* wk                     :34-35 */
+        L * dim * kv_cols,              /* wv                     :38-39 */
+        L * q_cols * dim,               /* wo                     :42-43 */
+        L * dim,                        /* rms_ffn_weight         :46-47 */
+        L * dim * hidden,               /* w1                     :50-51 */
+        L * hidden * dim,               /* w2                     :54-55 */
+        L * dim * hidden,               /* w3                     :58-59 */
+        dim                             /* rms_final_weight       :62-63 */
+    };
+    size_t at = 0;
+    for (int t = 0; t < 11; t++) {
+        offsets[t] = at;
+        counts[t] = n[t];
+        at += n[t];
+    }
+    offsets[11] = offsets[0];                      /* w_cls = token_embedding_table, :66 */
+    counts[11] = counts[0];
+    if (28 + at * sizeof(float) > file_size) return -3;
+    return 0;
+}

@@ -20,12 +20,21 @@
  *                     force on tiny shapes, hand-built sampler cases, golden
  *                     vectors written from the compiled reference
  *                     (tests/golden) and live bit-equality with oracle/_ref
+ *   orc_run           golden token sequences written from the reference's own
+ *                     executable (oracle/_ref/lighterpp_ref, built from main.cpp
+ *                     and the six files it needs) on a tiny synthetic checkpoint
+ *                     with a one-character-per-id tokenizer, greedy, with and
+ *                     without a prompt (tests/golden/ref_driver.json)
+ *   orc_checkpoint_parse  live equality with the compiled reference's
+ *                     load_model_file + checkpoint_init_weights (oracle/_ref) and
+ *                     the same golden run (the executable reads the file itself)
  *   orc_f16_to_f32    exhaustive over all 65536 half bit patterns against the
  *                     IEEE definition (numpy float16) and _ref-independent
  */
 #ifndef LPP_ORACLE_H
 #define LPP_ORACLE_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -119,6 +128,26 @@ int  orc_forward(int token, int pos, orc_state *s, const orc_weights *w,
 /* Sliding repetition-penalty window of src/main.cpp:158-208 (append, or shift
  * left by one when full). */
 void orc_history_push(int *history, int *len, int capacity, int token);
+
+/* The driver loop of src/main.cpp:139-232 without text: prefill-by-decode of all
+ * but the last prompt id (penalty 1.1, results discarded), generation from the
+ * last one (penalty 1.05) until position `steps` or an end-of-sequence id (2,
+ * 128001, 128009), 64-entry sliding window.  prompt == NULL: the single id 1. */
+typedef struct {
+    int n_tokens;        /* ids the reference would have printed during generation */
+    int final_pos;
+    int stopped_by_eos;
+    int reported_count;  /* "Tokens generated", main.cpp:229: final_pos - n_prompt */
+    int history_len;
+    int history[64];
+} orc_run_result;
+int orc_run(const int *prompt, int n_prompt, int steps, float temperature, float topp,
+            const float *uniforms, orc_state *s, const orc_weights *w, const orc_config *p,
+            int *out_tokens, int out_capacity, orc_run_result *res);
+
+/* llama2.c checkpoint (src/loader.cpp:134-172 header, :18-66 tensor order). */
+int orc_checkpoint_parse(const void *file_bytes, size_t file_size, orc_config *cfg,
+                         size_t offsets[12], size_t counts[12]);
 
 #ifdef __cplusplus
 }

@@ -11,6 +11,7 @@
 #include <string.h>
 
 #include "model.h"
+#include "loader.h"
 #include "ops.h"
 
 // model.h still declares the old 4-argument sample(); the definition in
@@ -127,4 +128,26 @@ float* ref_state_buffer(void* h, int which) {
     }
 }
 
+
+// load_model_file + checkpoint_init_weights (loader.cpp:134-172, 18-66) on a file on
+// disk: the header fields as the reference reads them and where it points each
+// tensor, in floats from the first weight.  Returns 0, or -1 when the file cannot
+// be opened.
+int ref_checkpoint_layout(const char* path, int* header7, float* rope_base, long long* offsets12) {
+    Config cfg;
+    size_t file_size = 0;
+    float* data = load_model_file(path, &cfg, &file_size);
+    if (!data) return -1;
+    transformerWeights w;
+    memset(&w, 0, sizeof(w));
+    checkpoint_init_weights(&w, &cfg, data);
+    header7[0] = cfg.dim; header7[1] = cfg.hidden_dim; header7[2] = cfg.n_layers; header7[3] = cfg.n_heads;
+    header7[4] = cfg.n_kv_heads; header7[5] = cfg.vocab_size; header7[6] = cfg.seq_len;
+    *rope_base = cfg.rope_base;
+    float* t[12] = {w.token_embedding_table, w.rms_att_weight, w.wq, w.wk, w.wv, w.wo, w.rms_ffn_weight,
+                    w.w1, w.w2, w.w3, w.rms_final_weight, w.w_cls};
+    for (int i = 0; i < 12; ++i) offsets12[i] = (long long)(t[i] - data);
+    free_model_file(data, file_size);
+    return 0;
+}
 }  // extern "C"

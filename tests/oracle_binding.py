@@ -35,6 +35,13 @@ class OrcState(C.Structure):
                [("kv_round_f16", C.c_int)]
 
 
+class OrcRunResult(C.Structure):
+    _fields_ = [("n_tokens", C.c_int), ("final_pos", C.c_int), ("stopped_by_eos", C.c_int),
+                ("reported_count", C.c_int), ("history_len", C.c_int), ("history", C.c_int * 64)]
+
+
+REF_EXE = ORACLE_DIR / "_ref" / "lighterpp_ref"
+
 _oracle = None
 _ref = None
 
@@ -75,6 +82,12 @@ def oracle() -> C.CDLL:
                                 C.c_float, C.c_float, C.c_float, C.c_void_p, C.c_int, C.c_float]
     lib.orc_forward.restype = C.c_int
     lib.orc_history_push.argtypes = [_i32p, C.POINTER(C.c_int), C.c_int, C.c_int]
+    lib.orc_run.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_float, C.c_void_p, C.POINTER(OrcState),
+                            C.POINTER(OrcWeights), C.POINTER(OrcConfig), C.c_void_p, C.c_int, C.POINTER(OrcRunResult)]
+    lib.orc_run.restype = C.c_int
+    lib.orc_checkpoint_parse.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(OrcConfig), C.POINTER(C.c_size_t),
+                                         C.POINTER(C.c_size_t)]
+    lib.orc_checkpoint_parse.restype = C.c_int
     _oracle = lib
     return lib
 
@@ -106,6 +119,9 @@ def ref() -> C.CDLL:
     lib.ref_transformer_block.argtypes = [C.c_void_p, C.c_int, C.c_int]
     lib.ref_state_buffer.argtypes = [C.c_void_p, C.c_int]
     lib.ref_state_buffer.restype = C.POINTER(C.c_float)
+    lib.ref_checkpoint_layout.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.POINTER(C.c_float),
+                                          C.POINTER(C.c_longlong)]
+    lib.ref_checkpoint_layout.restype = C.c_int
     _ref = lib
     return lib
 
@@ -177,6 +193,44 @@ class OracleModel:
             hp, hl = None, 0
         return self.lib.orc_forward(token, pos, C.byref(self.s), C.byref(self.w), C.byref(self.cfg), temperature,
                                     topp, penalty, hp, hl, r)
+
+
+    def run(self, prompt, steps: int, temperature: float = 0.0, topp: float = 1.0, uniforms=None):
+        """orc_run, the driver loop of main.cpp:139-232.  Returns (generated ids, OrcRunResult)."""
+        out = np.empty(max(steps, 1), dtype=np.int32)
+        pp, pn = None, 0
+        if prompt is not None and len(prompt) > 0:
+            pr = np.ascontiguousarray(prompt, dtype=np.int32)
+            pp, pn = pr.ctypes.data, int(pr.size)
+        up = None
+        if uniforms is not None:
+            u = np.ascontiguousarray(uniforms, dtype=np.float32)
+            up = u.ctypes.data
+        res = OrcRunResult()
+        rc = self.lib.orc_run(pp, pn, steps, temperature, topp, up, C.byref(self.s), C.byref(self.w),
+                              C.byref(self.cfg), out.ctypes.data, int(out.size), C.byref(res))
+        assert rc == 0
+        return out[:res.n_tokens].copy(), res
+
+
+def orc_checkpoint_parse(data: bytes):
+    """(status, OrcConfig, offsets[12], counts[12]) of a llama2.c checkpoint held in memory."""
+    cfg = OrcConfig()
+    off = (C.c_size_t * 12)()
+    cnt = (C.c_size_t * 12)()
+    buf = C.create_string_buffer(data, len(data))
+    rc = oracle().orc_checkpoint_parse(buf, len(data), C.byref(cfg), off, cnt)
+    return rc, cfg, list(off), list(cnt)
+
+
+def ref_checkpoint_layout(path):
+    """(header[7], rope_base, offsets[12]) as the compiled reference reads the file."""
+    hdr = (C.c_int * 7)()
+    rb = C.c_float()
+    off = (C.c_longlong * 12)()
+    rc = ref().ref_checkpoint_layout(str(path).encode(), hdr, C.byref(rb), off)
+    assert rc == 0
+    return list(hdr), rb.value, list(off)
 
 
 def orc_sample(logits: np.ndarray, temperature, topp, penalty, history, r) -> tuple:
