@@ -15,7 +15,7 @@
  * Section B replaces the model-level functions of src/model.h:117-164.
  * Section C is plumbing the reference gets from the CUDA runtime directly.
  * Section D is what sits either side of the path in the reference: the llama2.c
- * checkpoint reader (src/loader.cpp) and the driver loop (src/main.cpp).
+ * and GGUF readers (src/loader.cpp, src/gguf.cpp) and the driver loop (src/main.cpp).
  */
 #ifndef LPP_H
 #define LPP_H
@@ -255,6 +255,36 @@ lpp_status lpp_checkpoint_tensor(const lpp_checkpoint *ck, int tensor, const flo
 /* lpp_model_create + the upload half of checkpoint_init_weights (loader.cpp:73-131)
  * + lpp_model_tie_classifier. */
 lpp_status lpp_model_load_checkpoint(lpp_model **out, const lpp_checkpoint *ck);
+
+/* A GGUF file (versions 2 and 3) mapped into host memory; src/gguf.cpp.  Host code
+ * only; needs no GPU.  Tensor types read: F32 and F16 (gguf.h:10-17). */
+typedef struct lpp_gguf lpp_gguf;
+enum { LPP_GGML_F32 = 0, LPP_GGML_F16 = 1 };
+/* gguf_open (gguf.cpp:125-266): header, key/value index, tensor descriptions, data
+ * section at the next multiple of 32.  Unlike the reference it bounds every read,
+ * every tensor's data and the number of dimensions by the file. */
+lpp_status lpp_gguf_open(lpp_gguf **out, const char *path);
+/* gguf_close (gguf.cpp:268-290). */
+lpp_status lpp_gguf_close(lpp_gguf *g);
+/* gguf_extract_config (loader.cpp:213-339): "<arch>.embedding_length",
+ * ".feed_forward_length", ".block_count", ".attention.head_count",
+ * ".attention.head_count_kv" (default: head_count), ".context_length" (capped at
+ * 16384), ".rope.freq_base" (default 10000); vocab_size = number of entries of
+ * "tokenizer.ggml.tokens".  weight_precision as gguf_init_weights detects it
+ * (loader.cpp:426-433): FP16 iff blk.0.attn_q.weight is F16. */
+lpp_status lpp_gguf_config(const lpp_gguf *g, lpp_config *cfg);
+/* gguf_find_tensor + gguf_tensor_data (gguf.cpp:292-303): host address inside the
+ * mapping, ggml type and number of elements of a named tensor. */
+lpp_status lpp_gguf_tensor(const lpp_gguf *g, const char *name, const void **data, int *ggml_type,
+                           size_t *nelements);
+/* lpp_model_create + gguf_init_weights (loader.cpp:423-641): token_embd, output_norm,
+ * blk.N.{attn_norm, attn_q, attn_k, attn_v, attn_output, ffn_norm, ffn_gate, ffn_down,
+ * ffn_up}.weight into the stacked per-layer tensors, output.weight or the tied
+ * classifier.  F16 matrices of an FP16 model are uploaded as they are; F16 data
+ * destined for an fp32 tensor is widened exactly.  A tensor of another type, or an
+ * F32 matrix in an FP16 file, is LPP_ERR_UNSUPPORTED (the reference zero-fills the
+ * former and mis-sizes the latter). */
+lpp_status lpp_model_load_gguf(lpp_model **out, const lpp_gguf *g);
 
 typedef struct lpp_run_result {
     int n_tokens;        /* ids generated before the stop (what main.cpp prints)          */

@@ -33,6 +33,7 @@ TENSOR_NAMES = ["token_embedding", "rms_att", "wq", "wk", "wv", "wo", "rms_ffn",
 (B_X, B_XB, B_XB2, B_HB, B_HE, B_Q, B_K, B_V, B_ATT, B_LOGITS, B_KEY_CACHE, B_VALUE_CACHE) = range(12)
 
 PATH_OPS, PATH_FUSED, PATH_PERSISTENT = 0, 1, 2
+GGML_F32, GGML_F16 = 0, 1
 
 
 class LppConfig(C.Structure):
@@ -105,6 +106,11 @@ SIGNATURES = {
     "lpp_checkpoint_tensor": (_i, [_vp, _i, C.POINTER(_vp), C.POINTER(_sz)]),
     "lpp_model_load_checkpoint": (_i, [C.POINTER(_vp), _vp]),
     "lpp_run": (_i, [_vp, _vp, _i, _i, _f, _f, _vp, _vp, _i, C.POINTER(LppRunResult)]),
+    "lpp_gguf_open": (_i, [C.POINTER(_vp), C.c_char_p]),
+    "lpp_gguf_close": (_i, [_vp]),
+    "lpp_gguf_config": (_i, [_vp, C.POINTER(LppConfig)]),
+    "lpp_gguf_tensor": (_i, [_vp, C.c_char_p, C.POINTER(_vp), _ip, C.POINTER(_sz)]),
+    "lpp_model_load_gguf": (_i, [C.POINTER(_vp), _vp]),
     # C. runtime
     "lpp_last_error": (C.c_char_p, []),
     "lpp_version": (C.c_char_p, []),

@@ -1,7 +1,7 @@
 """Command-line driver over liblpp_hip.so: what src/main.cpp does with a llama2.c
-checkpoint, minus the tokenizer (ids in, ids out).
+checkpoint or a GGUF file (F32 / F16), minus the tokenizer (ids in, ids out).
 
-    python -m lighterpp_amd.driver model.bin [--prompt-ids 1,15,7] [--steps 200]
+    python -m lighterpp_amd.driver model.bin|model.gguf [--prompt-ids 1,15,7] [--steps 200]
                                    [--temperature 0.8] [--seed 1] [--path persistent]
 
 Prefill by decode, 64-entry sliding penalty window (1.1 while reading the prompt,
@@ -16,14 +16,14 @@ import sys
 import numpy as np
 
 from . import capi
-from .model import Checkpoint, Model
+from .model import Checkpoint, Gguf, Model
 
 PATHS = {"ops": capi.PATH_OPS, "fused": capi.PATH_FUSED, "persistent": capi.PATH_PERSISTENT}
 
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="lighterpp_amd.driver", description=__doc__.split("\n\n")[0])
-    ap.add_argument("checkpoint", help="llama2.c .bin file")
+    ap.add_argument("checkpoint", help="llama2.c .bin file or GGUF file")
     ap.add_argument("--prompt-ids", default="", help="comma-separated token ids (default: the single id 1)")
     ap.add_argument("--steps", type=int, default=200, help="last position + 1 (main.cpp:155)")
     ap.add_argument("--temperature", type=float, default=0.8)
@@ -32,12 +32,14 @@ def main(argv=None) -> int:
     args = ap.parse_args(argv)
 
     capi.init(0)
-    ck = Checkpoint(args.checkpoint)
+    with open(args.checkpoint, "rb") as f:
+        is_gguf = f.read(4) == b"GGUF"  # is_gguf_file, loader.cpp:200-211
+    ck = Gguf(args.checkpoint) if is_gguf else Checkpoint(args.checkpoint)
     c = ck.config
     print("--- Model Configuration ---")
     print(f"Dim: {c.dim}\nHidden Dim: {c.hidden_dim}\nLayers: {c.n_layers}\nHeads: {c.n_heads}\nKV Heads: {c.n_kv_heads}")
     print(f"Vocab: {c.vocab_size}\nSeq Len: {c.seq_len}\nRoPE Base: {c.rope_base:.0f}\nTemperature: {args.temperature:.2f}")
-    model = Model.from_checkpoint(ck)
+    model = Model.from_gguf(ck) if is_gguf else Model.from_checkpoint(ck)
     model.set_path(PATHS[args.path])
     prompt = [int(t) for t in args.prompt_ids.split(",") if t.strip()] or None
     steps = min(args.steps, c.seq_len)

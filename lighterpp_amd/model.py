@@ -147,6 +147,49 @@ class Checkpoint:
             pass
 
 
+class Gguf:
+    """A GGUF file mapped by lpp_gguf_open (host code, no GPU)."""
+
+    def __init__(self, path):
+        self.lib = capi.load()
+        h = C.c_void_p()
+        capi.check(self.lib.lpp_gguf_open(C.byref(h), str(path).encode()))
+        self.handle = h
+
+    @property
+    def config(self) -> "capi.LppConfig":
+        cfg = capi.LppConfig()
+        capi.check(self.lib.lpp_gguf_config(self.handle, C.byref(cfg)))
+        return cfg
+
+    def shape(self, tied: bool) -> Shape:
+        c = self.config
+        return Shape(c.dim, c.hidden_dim, c.n_layers, c.n_heads, c.n_kv_heads, c.vocab_size, c.seq_len, c.rope_base,
+                     fp16=c.weight_precision == capi.WEIGHT_FP16, tied=tied)
+
+    def tensor(self, name: str) -> np.ndarray:
+        """Copy of a named tensor, flat: float32, or binary16 bit patterns (uint16)."""
+        p, ty, n = C.c_void_p(), C.c_int(), C.c_size_t()
+        capi.check(self.lib.lpp_gguf_tensor(self.handle, name.encode(), C.byref(p), C.byref(ty), C.byref(n)))
+        ctype, dtype = {capi.GGML_F32: (C.c_float, np.float32), capi.GGML_F16: (C.c_uint16, np.uint16)}[ty.value]
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(ctype)), shape=(n.value,)).astype(dtype, copy=True)
+
+    def has_tensor(self, name: str) -> bool:
+        p, ty, n = C.c_void_p(), C.c_int(), C.c_size_t()
+        return self.lib.lpp_gguf_tensor(self.handle, name.encode(), C.byref(p), C.byref(ty), C.byref(n)) == capi.LPP_OK
+
+    def close(self) -> None:
+        if self.handle:
+            self.lib.lpp_gguf_close(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Model:
     def __init__(self, shape: Shape, _handle=None):
         self.shape = shape
@@ -168,6 +211,13 @@ class Model:
         h = C.c_void_p()
         capi.check(ck.lib.lpp_model_load_checkpoint(C.byref(h), ck.handle))
         return cls(ck.shape, _handle=h)
+
+    @classmethod
+    def from_gguf(cls, g: "Gguf") -> "Model":
+        """lpp_model_load_gguf: create, gather the named tensors into the stacked layout, upload."""
+        h = C.c_void_p()
+        capi.check(g.lib.lpp_model_load_gguf(C.byref(h), g.handle))
+        return cls(g.shape(tied=not g.has_tensor("output.weight")), _handle=h)
 
     def close(self) -> None:
         if self.handle:

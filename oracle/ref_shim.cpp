@@ -150,4 +150,38 @@ int ref_checkpoint_layout(const char* path, int* header7, float* rope_base, long
     free_model_file(data, file_size);
     return 0;
 }
+
+// gguf_open + gguf_extract_config + gguf_init_weights (gguf.cpp:125-266, loader.cpp:213-339,
+// 423-541, CPU build): the reference's own reading of a GGUF file.  config9 receives the
+// nine Config fields (rope_base as its bit pattern); weights12 the host arrays the loader
+// allocated (fp32, stacked per layer).  Returns a handle for ref_gguf_free, or null.
+void* ref_gguf_load(const char* path, int* config9, float** weights12) {
+    GGUFFile* f = gguf_open(path);
+    if (!f) return nullptr;
+    RefModel* m = (RefModel*)calloc(1, sizeof(RefModel));
+    if (!m || !gguf_extract_config(f, &m->cfg) || !gguf_init_weights(f, &m->w, &m->cfg)) {
+        gguf_close(f);
+        free(m);
+        return nullptr;
+    }
+    gguf_close(f);
+    config9[0] = m->cfg.dim; config9[1] = m->cfg.hidden_dim; config9[2] = m->cfg.n_layers;
+    config9[3] = m->cfg.n_heads; config9[4] = m->cfg.n_kv_heads; config9[5] = m->cfg.vocab_size;
+    config9[6] = m->cfg.seq_len; memcpy(&config9[7], &m->cfg.rope_base, 4);
+    config9[8] = (int)m->cfg.weight_precision;
+    float* t[12] = {m->w.token_embedding_table, m->w.rms_att_weight, m->w.wq, m->w.wk, m->w.wv, m->w.wo,
+                    m->w.rms_ffn_weight, m->w.w1, m->w.w2, m->w.w3, m->w.rms_final_weight, m->w.w_cls};
+    for (int i = 0; i < 12; ++i) weights12[i] = t[i];
+    return m;
+}
+
+void ref_gguf_free(void* h) {
+    RefModel* m = (RefModel*)h;
+    if (!m) return;
+    if (m->w.w_cls != m->w.token_embedding_table) free(m->w.w_cls);
+    float* t[11] = {m->w.token_embedding_table, m->w.rms_att_weight, m->w.wq, m->w.wk, m->w.wv, m->w.wo,
+                    m->w.rms_ffn_weight, m->w.w1, m->w.w2, m->w.w3, m->w.rms_final_weight};
+    for (int i = 0; i < 11; ++i) free(t[i]);
+    free(m);
+}
 }  // extern "C"

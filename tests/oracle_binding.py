@@ -122,6 +122,9 @@ def ref() -> C.CDLL:
     lib.ref_checkpoint_layout.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.POINTER(C.c_float),
                                           C.POINTER(C.c_longlong)]
     lib.ref_checkpoint_layout.restype = C.c_int
+    lib.ref_gguf_load.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.POINTER(C.POINTER(C.c_float))]
+    lib.ref_gguf_load.restype = C.c_void_p
+    lib.ref_gguf_free.argtypes = [C.c_void_p]
     _ref = lib
     return lib
 
@@ -231,6 +234,26 @@ def ref_checkpoint_layout(path):
     rc = ref().ref_checkpoint_layout(str(path).encode(), hdr, C.byref(rb), off)
     assert rc == 0
     return list(hdr), rb.value, list(off)
+
+
+def ref_gguf_load(path):
+    """The compiled reference's reading of a GGUF file: (config dict, [12 fp32 arrays]) or None
+    when it refuses the file.  Arrays are copies."""
+    cfg = (C.c_int * 9)()
+    ptrs = (C.POINTER(C.c_float) * 12)()
+    h = ref().ref_gguf_load(str(path).encode(), cfg, ptrs)
+    if not h:
+        return None
+    c = dict(zip(["dim", "hidden_dim", "n_layers", "n_heads", "n_kv_heads", "vocab_size", "seq_len"], list(cfg)[:7]))
+    c["rope_base"] = np.array([cfg[7]], dtype=np.int32).view(np.float32)[0]
+    c["fp16"] = cfg[8] == 1
+    kv = c["dim"] // c["n_heads"] * c["n_kv_heads"]
+    L, d, hd, v = c["n_layers"], c["dim"], c["hidden_dim"], c["vocab_size"]
+    counts = [v * d, L * d, L * d * d, L * kv * d, L * kv * d, L * d * d, L * d, L * hd * d, L * d * hd, L * hd * d, d, v * d]
+    arrays = [np.ctypeslib.as_array(ptrs[i], shape=(counts[i],)).copy() for i in range(12)]
+    tied = C.addressof(ptrs[11].contents) == C.addressof(ptrs[0].contents)
+    ref().ref_gguf_free(h)
+    return c, arrays, tied
 
 
 def orc_sample(logits: np.ndarray, temperature, topp, penalty, history, r) -> tuple:
