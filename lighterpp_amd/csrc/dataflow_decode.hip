@@ -977,15 +977,31 @@ __device__ __forceinline__ void att_combine(Ctx& c, Io& io, const Lds& l, int la
     }
 }
 
-__device__ __forceinline__ int item_splits(int npos, int cap) {
-    int s = (npos + kItemPositions - 1) / kItemPositions;
-    return s < 1 ? 1 : (s > cap ? cap : s);
+// Context splits per query head.  The attention phase lasts as long as its busiest workgroup:
+// (work items per workgroup) x (positions per item), plus, once there is more than one split, the
+// extra hand-over in which the partial results are combined (about what 300 positions cost).  Among
+// the split counts that keep an item within 2 * kItemPositions positions, the cheapest wins and the
+// smaller of equals: at 8193 positions and 32 heads on 256 workgroups that is 8 splits of 1025
+// positions in one round, where 9 splits of 911 would leave 32 workgroups a second item.
+__device__ __forceinline__ int item_splits(int npos, int cap, int n_heads, int nwg) {
+    constexpr int kCombineCost = 300;
+    int best = 1, best_cost = 0x7fffffff;
+    const int first = max(1, (npos + 2 * kItemPositions - 1) / (2 * kItemPositions));
+    for (int s = first; s <= cap; ++s) {
+        const int rounds = (n_heads * s + nwg - 1) / nwg;
+        const int cost = rounds * ((npos + s - 1) / s) + (s > 1 ? kCombineCost : 0);
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = s;
+        }
+    }
+    return best;
 }
 
 __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int layer) {
     const DecodeArgs& a = c.a;
     const int npos = c.pos + 1;
-    const int nsplits = item_splits(npos, c.t.splits_cap);
+    const int nsplits = item_splits(npos, c.t.splits_cap, a.n_heads, c.nwg);
     const int items = a.n_heads * nsplits;
     const int hs = a.head_size;
     bool first = true;
