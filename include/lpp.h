@@ -286,6 +286,29 @@ lpp_status lpp_gguf_tensor(const lpp_gguf *g, const char *name, const void **dat
  * former and mis-sizes the latter). */
 lpp_status lpp_model_load_gguf(lpp_model **out, const lpp_gguf *g);
 
+/* The tokenizer of src/tokenizer.cpp.  Host code only. */
+typedef struct lpp_tokenizer lpp_tokenizer;
+enum { LPP_TOKENIZER_SENTENCEPIECE = 0, LPP_TOKENIZER_BPE = 1 }; /* TokenizerType, tokenizer.h:4-7 */
+/* load_tokenizer (tokenizer.cpp:15-55): the llama2.c tokenizer file -- int maximum
+ * token length, then per id a float score, an int length and the bytes. */
+lpp_status lpp_tokenizer_load(lpp_tokenizer **out, const char *path, int vocab_size);
+/* gguf_init_tokenizer (loader.cpp:648-699): the vocabulary embedded in a GGUF file. */
+lpp_status lpp_tokenizer_from_gguf(lpp_tokenizer **out, const lpp_gguf *g);
+/* free_tokenizer (tokenizer.cpp:237-245). */
+lpp_status lpp_tokenizer_free(lpp_tokenizer *t);
+lpp_status lpp_tokenizer_info(const lpp_tokenizer *t, int *vocab_size, int *kind, int *max_token_len);
+/* encode (tokenizer.cpp:148-235): optional BOS, a blank in front of the text, one id
+ * per byte (space marker / "<0xXX>" fallback; bytes without any entry are dropped),
+ * then greedy merging by score.  Ids beyond max_tokens are dropped, as in the
+ * reference.  An empty result is returned as such (the reference's merge loop
+ * underflows on it). */
+lpp_status lpp_tokenizer_encode(const lpp_tokenizer *t, const char *text, int *tokens, int max_tokens,
+                                int *n_tokens);
+/* decode_token (tokenizer.cpp:61-123): "<0xXX>" entries give their byte, other
+ * "<...>" entries nothing, space (and newline) markers their character; at most
+ * 255 bytes.  An id outside the vocabulary is an error (the reference exits). */
+lpp_status lpp_tokenizer_decode(const lpp_tokenizer *t, int token_id, char *out, size_t capacity);
+
 typedef struct lpp_run_result {
     int n_tokens;        /* ids generated before the stop (what main.cpp prints)          */
     int final_pos;

@@ -34,6 +34,7 @@ TENSOR_NAMES = ["token_embedding", "rms_att", "wq", "wk", "wv", "wo", "rms_ffn",
 
 PATH_OPS, PATH_FUSED, PATH_PERSISTENT = 0, 1, 2
 GGML_F32, GGML_F16 = 0, 1
+TOKENIZER_SENTENCEPIECE, TOKENIZER_BPE = 0, 1
 
 
 class LppConfig(C.Structure):
@@ -111,6 +112,12 @@ SIGNATURES = {
     "lpp_gguf_config": (_i, [_vp, C.POINTER(LppConfig)]),
     "lpp_gguf_tensor": (_i, [_vp, C.c_char_p, C.POINTER(_vp), _ip, C.POINTER(_sz)]),
     "lpp_model_load_gguf": (_i, [C.POINTER(_vp), _vp]),
+    "lpp_tokenizer_load": (_i, [C.POINTER(_vp), C.c_char_p, _i]),
+    "lpp_tokenizer_from_gguf": (_i, [C.POINTER(_vp), _vp]),
+    "lpp_tokenizer_free": (_i, [_vp]),
+    "lpp_tokenizer_info": (_i, [_vp, _ip, _ip, _ip]),
+    "lpp_tokenizer_encode": (_i, [_vp, C.c_char_p, _vp, _i, _ip]),
+    "lpp_tokenizer_decode": (_i, [_vp, _i, C.c_char_p, _sz]),
     # C. runtime
     "lpp_last_error": (C.c_char_p, []),
     "lpp_version": (C.c_char_p, []),

@@ -149,6 +149,38 @@ struct lpp_gguf {
     const void* data(const TensorInfo& t) const { return at(data_start + static_cast<size_t>(t.offset)); }
 };
 
+// The embedded vocabulary as gguf_init_tokenizer reads it (loader.cpp:648-699): kind from
+// "tokenizer.ggml.model" ("gpt2" = byte-pair, anything else or absent = SentencePiece), strings
+// from "tokenizer.ggml.tokens", scores from "tokenizer.ggml.scores" when there is one per token,
+// zeros otherwise.  Used by lpp_tokenizer_from_gguf.
+namespace lpp {
+lpp_status gguf_vocabulary(const lpp_gguf* g, int* kind, std::vector<std::string>* tokens, std::vector<float>* scores) {
+    std::string model;
+    *kind = (g->get_string("tokenizer.ggml.model", &model) && model == "gpt2") ? LPP_TOKENIZER_BPE : LPP_TOKENIZER_SENTENCEPIECE;
+    const size_t n = g->string_array_count("tokenizer.ggml.tokens");
+    if (n == 0) return lpp::fail(LPP_ERR_INVALID_ARG, "lpp_tokenizer_from_gguf: no tokenizer.ggml.tokens");
+    const Meta* m = g->find("tokenizer.ggml.tokens", kArray);
+    size_t pos = m->value_offset + 12;
+    tokens->resize(n);
+    for (size_t i = 0; i < n; ++i) {  // bounds were checked when the file was opened
+        uint64_t len = 0;
+        std::memcpy(&len, g->at(pos), 8);
+        (*tokens)[i].assign(reinterpret_cast<const char*>(g->at(pos + 8)), static_cast<size_t>(len));
+        pos += 8 + static_cast<size_t>(len);
+    }
+    scores->assign(n, 0.0f);
+    const Meta* sm = g->find("tokenizer.ggml.scores", kArray);
+    if (sm != nullptr) {
+        uint32_t elem = 0;
+        uint64_t count = 0;
+        std::memcpy(&elem, g->at(sm->value_offset), 4);
+        std::memcpy(&count, g->at(sm->value_offset + 4), 8);
+        if (elem == kF32 && count == n) std::memcpy(scores->data(), g->at(sm->value_offset + 12), n * sizeof(float));
+    }
+    return LPP_OK;
+}
+}  // namespace lpp
+
 extern "C" {
 
 lpp_status lpp_gguf_open(lpp_gguf** out, const char* path) {

@@ -1,8 +1,12 @@
 """Command-line driver over liblpp_hip.so: what src/main.cpp does with a llama2.c
-checkpoint or a GGUF file (F32 / F16), minus the tokenizer (ids in, ids out).
+checkpoint or a GGUF file (F32 / F16).
 
-    python -m lighterpp_amd.driver model.bin|model.gguf [--prompt-ids 1,15,7] [--steps 200]
-                                   [--temperature 0.8] [--seed 1] [--path persistent]
+    python -m lighterpp_amd.driver model.bin|model.gguf [--tokenizer tokenizer.bin] [--prompt "text"]
+                                   [--prompt-ids 1,15,7] [--steps 200] [--temperature 0.8] [--seed 1]
+                                   [--path persistent]
+
+With a tokenizer (a llama2.c tokenizer file, or the vocabulary inside a GGUF file) text goes
+in and comes out; without one, ids do.
 
 Prefill by decode, 64-entry sliding penalty window (1.1 while reading the prompt,
 1.05 while generating), stop at position --steps or at an end-of-sequence id, then the
@@ -16,7 +20,7 @@ import sys
 import numpy as np
 
 from . import capi
-from .model import Checkpoint, Gguf, Model
+from .model import Checkpoint, Gguf, Model, Tokenizer
 
 PATHS = {"ops": capi.PATH_OPS, "fused": capi.PATH_FUSED, "persistent": capi.PATH_PERSISTENT}
 
@@ -24,6 +28,8 @@ PATHS = {"ops": capi.PATH_OPS, "fused": capi.PATH_FUSED, "persistent": capi.PATH
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="lighterpp_amd.driver", description=__doc__.split("\n\n")[0])
     ap.add_argument("checkpoint", help="llama2.c .bin file or GGUF file")
+    ap.add_argument("--tokenizer", default=None, help="llama2.c tokenizer file (default for GGUF: the embedded vocabulary)")
+    ap.add_argument("--prompt", default=None, help="prompt text (needs a tokenizer)")
     ap.add_argument("--prompt-ids", default="", help="comma-separated token ids (default: the single id 1)")
     ap.add_argument("--steps", type=int, default=200, help="last position + 1 (main.cpp:155)")
     ap.add_argument("--temperature", type=float, default=0.8)
@@ -41,12 +47,30 @@ def main(argv=None) -> int:
     print(f"Vocab: {c.vocab_size}\nSeq Len: {c.seq_len}\nRoPE Base: {c.rope_base:.0f}\nTemperature: {args.temperature:.2f}")
     model = Model.from_gguf(ck) if is_gguf else Model.from_checkpoint(ck)
     model.set_path(PATHS[args.path])
+    tok = None
+    if args.tokenizer:
+        tok = Tokenizer.load(args.tokenizer, c.vocab_size)
+    elif is_gguf:
+        try:
+            tok = Tokenizer.from_gguf(ck)
+        except capi.LppError:
+            tok = None  # main.cpp:78-82: ids are printed instead
     prompt = [int(t) for t in args.prompt_ids.split(",") if t.strip()] or None
+    if args.prompt is not None:
+        if tok is None:
+            ap.error("--prompt needs a tokenizer")
+        prompt = tok.encode(args.prompt, 2048)  # main.cpp:140-146
+        print(f"Encoded {len(prompt)} tokens.")
     steps = min(args.steps, c.seq_len)
     uniforms = capi.synth_uniform_f32(steps, args.seed)
     print("\n--- Running Inference ---")
     tokens, res = model.run(prompt, steps, args.temperature, 1.0, uniforms)
-    print(" ".join(str(int(t)) for t in tokens))
+    if tok is not None:
+        shown = list(prompt or [1]) + [int(t) for t in tokens]  # main.cpp:175-176, 191-192, 215-221
+        sys.stdout.buffer.write(b"".join(tok.decode(t) for t in shown) + b"\n")
+        sys.stdout.flush()
+    else:
+        print(" ".join(str(int(t)) for t in tokens))
     print("\n--- Statistics ---")
     print(f"Tokens generated: {res.reported_count}")
     print(f"Elapsed time: {res.wall_seconds:.2f} s")

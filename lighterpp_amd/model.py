@@ -147,6 +147,52 @@ class Checkpoint:
             pass
 
 
+class Tokenizer:
+    """lpp_tokenizer: the tokenizer of src/tokenizer.cpp (host code, no GPU)."""
+
+    def __init__(self, handle):
+        self.lib = capi.load()
+        self.handle = handle
+        n, kind, mx = C.c_int(), C.c_int(), C.c_int()
+        capi.check(self.lib.lpp_tokenizer_info(handle, C.byref(n), C.byref(kind), C.byref(mx)))
+        self.vocab_size, self.kind, self.max_token_len = n.value, kind.value, mx.value
+
+    @classmethod
+    def load(cls, path, vocab_size: int) -> "Tokenizer":
+        h = C.c_void_p()
+        capi.check(capi.load().lpp_tokenizer_load(C.byref(h), str(path).encode(), vocab_size))
+        return cls(h)
+
+    @classmethod
+    def from_gguf(cls, g: "Gguf") -> "Tokenizer":
+        h = C.c_void_p()
+        capi.check(g.lib.lpp_tokenizer_from_gguf(C.byref(h), g.handle))
+        return cls(h)
+
+    def encode(self, text, max_tokens: int = 2048) -> list:
+        raw = text if isinstance(text, bytes) else text.encode()
+        out = np.empty(max(max_tokens, 1), dtype=np.int32)
+        n = C.c_int()
+        capi.check(self.lib.lpp_tokenizer_encode(self.handle, raw, C.c_void_p(out.ctypes.data), max_tokens, C.byref(n)))
+        return out[:n.value].tolist()
+
+    def decode(self, token_id: int) -> bytes:
+        buf = C.create_string_buffer(256)
+        capi.check(self.lib.lpp_tokenizer_decode(self.handle, token_id, buf, 256))
+        return buf.value
+
+    def close(self) -> None:
+        if self.handle:
+            self.lib.lpp_tokenizer_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Gguf:
     """A GGUF file mapped by lpp_gguf_open (host code, no GPU)."""
 

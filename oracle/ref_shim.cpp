@@ -13,6 +13,7 @@
 #include "model.h"
 #include "loader.h"
 #include "ops.h"
+#include "tokenizer.h"
 
 // model.h still declares the old 4-argument sample(); the definition in
 // model.cpp:256 takes seven.  Declare what is actually defined.
@@ -184,4 +185,35 @@ void ref_gguf_free(void* h) {
     for (int i = 0; i < 11; ++i) free(t[i]);
     free(m);
 }
+
+// The reference's tokenizer (tokenizer.cpp; gguf_init_tokenizer, loader.cpp:648-699).
+// Its string-to-id map is a file-scope static built from the first vocabulary it
+// sees: load this library afresh (from a copy of the file) for every vocabulary.
+void* ref_tokenizer_load(const char* path, int vocab_size) {
+    Tokenizer* t = (Tokenizer*)calloc(1, sizeof(Tokenizer));
+    load_tokenizer(t, path, vocab_size);  // exits the process on a malformed file
+    return t;
+}
+void* ref_tokenizer_from_gguf(const char* path) {
+    GGUFFile* f = gguf_open(path);
+    if (!f) return nullptr;
+    Tokenizer* t = (Tokenizer*)calloc(1, sizeof(Tokenizer));
+    const bool ok = gguf_init_tokenizer(f, t);
+    gguf_close(f);
+    if (!ok) {
+        free(t);
+        return nullptr;
+    }
+    return t;
+}
+int ref_tokenizer_kind(void* h) { return (int)((Tokenizer*)h)->type; }
+int ref_tokenizer_vocab_size(void* h) { return ((Tokenizer*)h)->vocab_size; }
+int ref_tokenizer_max_token_len(void* h) { return ((Tokenizer*)h)->max_token_len; }
+float ref_tokenizer_score(void* h, int i) { return ((Tokenizer*)h)->vocab_scores[i]; }
+int ref_encode(void* h, const char* text, int* tokens, int max_tokens) {
+    int n = 0;
+    encode((Tokenizer*)h, text, tokens, &n, max_tokens);
+    return n;
+}
+const char* ref_decode(void* h, int id) { return decode_token((Tokenizer*)h, id); }
 }  // extern "C"

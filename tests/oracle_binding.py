@@ -236,6 +236,34 @@ def ref_checkpoint_layout(path):
     return list(hdr), rb.value, list(off)
 
 
+def fresh_ref(tmp_dir) -> C.CDLL:
+    """A private copy of the compiled reference, with its own file-scope statics (the
+    tokenizer keeps its string-to-id map in one, built from the first vocabulary it sees)."""
+    import shutil
+    import uuid
+    dst = Path(tmp_dir) / f"liblpp_ref_{uuid.uuid4().hex}.so"
+    shutil.copy(REF_SO, dst)
+    lib = C.CDLL(str(dst))
+    lib.ref_tokenizer_load.argtypes = [C.c_char_p, C.c_int]
+    lib.ref_tokenizer_load.restype = C.c_void_p
+    lib.ref_tokenizer_from_gguf.argtypes = [C.c_char_p]
+    lib.ref_tokenizer_from_gguf.restype = C.c_void_p
+    for f in ("ref_tokenizer_kind", "ref_tokenizer_vocab_size", "ref_tokenizer_max_token_len"):
+        getattr(lib, f).argtypes = [C.c_void_p]
+    lib.ref_tokenizer_score.argtypes = [C.c_void_p, C.c_int]
+    lib.ref_tokenizer_score.restype = C.c_float
+    lib.ref_encode.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int]
+    lib.ref_decode.argtypes = [C.c_void_p, C.c_int]
+    lib.ref_decode.restype = C.c_char_p
+    return lib
+
+
+def ref_encode(lib, handle, text: bytes, max_tokens: int = 4096) -> list:
+    out = np.empty(max_tokens, dtype=np.int32)
+    n = lib.ref_encode(handle, text, out.ctypes.data, max_tokens)
+    return out[:n].tolist()
+
+
 def ref_gguf_load(path):
     """The compiled reference's reading of a GGUF file: (config dict, [12 fp32 arrays]) or None
     when it refuses the file.  Arrays are copies."""

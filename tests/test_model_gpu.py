@@ -269,7 +269,7 @@ def test_benchmark_shapes_first_steps(cfg, steps, start):
 
 def test_persistent_timeline_is_ordered():
     """lpp_trace_token: every phase of the persistent kernel reports its marks, in order, and the
-    phases follow one another (the timeline is what DESIGN.md's per-phase figures come from)."""
+    phases follow one another."""
     import ctypes as C
     shape = SMALL_SHAPES["gqa4_fp16"]
     m, o = build(shape, 4)
