@@ -37,7 +37,7 @@ def main(argv=None) -> int:
     ap.add_argument("--path", default="persistent", choices=list(PATHS))
     args = ap.parse_args(argv)
 
-    capi.init(0)
+    capi.check(capi.load().lpp_init(0))
     with open(args.checkpoint, "rb") as f:
         is_gguf = f.read(4) == b"GGUF"  # is_gguf_file, loader.cpp:200-211
     ck = Gguf(args.checkpoint) if is_gguf else Checkpoint(args.checkpoint)

@@ -177,3 +177,39 @@ def test_model_from_checkpoint_equals_uploaded_model(path, tmp_path):
         assert tok_a == tok_b
     a.close()
     b.close()
+
+
+def test_command_line_driver_text_in_text_out(tmp_path):
+    """python -m lighterpp_amd.driver on a llama2.c checkpoint with a tokenizer file: the text it
+    prints is the prompt's and the generated ids' strings, the ids are lpp_run's."""
+    import struct
+    import subprocess
+    import sys
+    from lighterpp_amd import Tokenizer
+    shape = Shape(64, 96, 2, 4, 2, 40, 200, 10000.0, fp16=False, tied=True)
+    w = weights(shape, 22)
+    ck, tk = tmp_path / "m.bin", tmp_path / "t.bin"
+    write_checkpoint(ck, shape, w)
+    alphabet = "abcdefghijklmnopqrstuvwxyzABCDEFGHIJKLMN"
+    with open(tk, "wb") as f:
+        f.write(struct.pack("<i", 1))
+        for ch in alphabet:
+            f.write(struct.pack("<fi", 0.0, 1) + ch.encode())
+    root = Path(__file__).resolve().parent.parent
+    out = subprocess.run([sys.executable, "-m", "lighterpp_amd.driver", str(ck), "--tokenizer", str(tk), "--prompt", "hello",
+                          "--steps", "60", "--temperature", "0", "--path", "persistent"],
+                         cwd=root, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, out.stderr
+    assert "Encoded 5 tokens." in out.stdout and "Tokens generated: 55" in out.stdout
+    text = out.stdout.split("--- Running Inference ---\n", 1)[1].split("\n\n--- Statistics ---", 1)[0].strip("\n")
+    tok = Tokenizer.load(tk, shape.vocab_size)
+    prompt = tok.encode("hello")
+    assert prompt == [alphabet.index(c) for c in "hello"]
+    m = Model(shape)
+    for t in range(capi.T_WCLS):
+        m.upload(t, w[t])
+    m.tie_classifier()
+    m.set_path(capi.PATH_PERSISTENT)
+    ids, res = m.run(prompt, 60, 0.0)
+    assert text == "".join(alphabet[i] for i in prompt + ids.tolist())
+    m.close()
