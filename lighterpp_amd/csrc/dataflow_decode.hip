@@ -60,6 +60,8 @@ constexpr int kItemPositions = 1024;               // context positions per atte
 constexpr int kAttSubBlock = 256;                  // positions scored between two barriers of an item
 constexpr int kAttScoreFloats = 512;               // one score area (a sub-block never exceeds kIoThreads positions)
 constexpr int kMaxHeadPad = 128;
+constexpr int kMaxAttHeads = 4;                    // query heads of one KV head a long-context work item covers
+constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
 
 typedef unsigned long long u64;
 
@@ -86,6 +88,9 @@ struct Tagged {
     u64* part;   // [n_heads][splits_cap][head_size + 2] attention split partials
     u64* stats;  // [nwg][4]  per-workgroup sampler statistics (max, sum, argmax)
     int splits_cap;
+    unsigned hs_magic;     // floor(2^32 / head_size) + 1: x / head_size == __umulhi(x, hs_magic) for x < 2^25
+    int att_splits;        // context splits per query head at this position (worked out on the host: the search
+    int att_group_splits;  // is a few dozen integer divisions); > 0: items cover two heads of a KV head, this many splits
     // the step record, except the token id (which the previous launch left in device memory)
     int pos, history_len;
     float temperature, penalty, r;
@@ -188,6 +193,11 @@ struct Ctx {
     }
     __device__ __forceinline__ unsigned seq_stats() const { return base + 1u + 5u * static_cast<unsigned>(a.n_layers); }
 };
+
+// x / head_size without the two dozen instructions of a run-time integer division (x < 2^25).
+__device__ __forceinline__ int div_head_size(const Ctx& c, int x) {
+    return static_cast<int>(__umulhi(static_cast<unsigned>(x), c.t.hs_magic));
+}
 
 __host__ __device__ inline unsigned phases_per_token(int n_layers) { return 5u * n_layers + 2u; }
 // Timeline marks per phase (workgroup 0): 0 phase entered, 1 own inputs received,
@@ -428,6 +438,18 @@ __device__ __forceinline__ int exchange_thread_index(int iw) {
     return iw * kWave + lane;
 }
 
+// Lane exchange with an explicitly supplied lane index (byte address of the partner = (lane ^
+// offset) * 4).  __shfl_xor works the index out from a value the optimiser keeps for the whole
+// kernel; callers here pass one made with fresh_lane() where the exchanges happen.
+__device__ __forceinline__ int fresh_lane() {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+__device__ __forceinline__ float lane_xor(float v, int offset, int lane) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ offset) << 2, __float_as_int(v)));
+}
+
 struct Io {
     int it;        // thread index among the exchange threads
     int iw;        // exchange wavefront index
@@ -587,8 +609,8 @@ struct Lds {
     float* xs;       // [xs_floats] staged GEMV input; sampler tables after the classifier
     float* results;  // [results_floats] row results of the current GEMV phase
     float* sc;       // [2][kAttScoreFloats] attention scores of a sub-block, two areas taking turns
-    float* qkv;      // [3][kMaxHeadPad] this token's q, k, v of the head being attended
-    float* red;      // [kIoWaves][kMaxHeadPad] attention cross-wavefront reduction
+    float* qkv;      // [kMaxAttHeads + 2][kMaxHeadPad] this token's q (per head of the item), k, v
+    float* red;      // [kIoWaves][kMaxAttHeads][kRedStride] attention cross-wavefront reduction
     float* gather;   // [gather_floats] attention split partials
 };
 
@@ -684,6 +706,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
 #pragma clang fp contract(off)
     const DecodeArgs& a = c.a;
     const int dim = a.dim, kv_dim = a.kv_dim, hs = a.head_size;
+    auto mod_hs = [&](int x) { return x - div_head_size(c, x) * hs; };
     const float* emb_row = (layer == 0) ? a.emb + static_cast<size_t>(c.token) * dim : nullptr;
     mark(c, io, 0);
     const float scale = stage_norm(c, io, l, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
@@ -699,7 +722,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     const bool first_rotates = first_row < nrows && first_g < dim + kv_dim;
     // (a valid address either way, so that the request does not sit behind a branch)
     float first_cos, first_sin;
-    pinned_load(cs_row + (first_rotates ? ((((first_g < dim) ? first_g : first_g - dim) & ~1) % hs) >> 1 : 0), first_cos, first_sin);
+    pinned_load(cs_row + (first_rotates ? mod_hs(((first_g < dim) ? first_g : first_g - dim) & ~1) >> 1 : 0), first_cos, first_sin);
     // (a plain loop, not finished_rows with a closure: a local captured by reference is kept in
     // private memory across the wait, and private memory shares the load counter)
     wait_gemv(c.ctl, 4 * layer + kGQkv);
@@ -713,7 +736,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
             const int gi = (g < dim) ? g : g - dim;
             float cos_t = first_cos, sin_t = first_sin;
             if (r != first_row) {
-                const float2 cs = cs_row[((gi & ~1) % hs) >> 1];
+                const float2 cs = cs_row[mod_hs(gi & ~1) >> 1];
                 cos_t = cs.x;
                 sin_t = cs.y;
             }
@@ -725,7 +748,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
         } else {  // model.cpp:171-176 / scatter_kv.cu:15-18
             const bool is_k = g < dim + kv_dim;
             const int i = is_k ? g - dim : g - dim - kv_dim;
-            const int head = i / hs, within = i - head * hs;
+            const int head = div_head_size(c, i), within = i - head * hs;
             const size_t dst = static_cast<size_t>(layer) * kv_dim * a.seq_len +
                                static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(c.pos) * hs + within;
             publish((is_k ? c.t.k : c.t.v) + i, out, tag);
@@ -790,9 +813,8 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
 // regrouped).
 template <int kGroup>
 __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer, int h, int split, int nsplits,
-                                         int npos, bool first_item) {
+                                         int npos, bool first_item, int hs) {
     const DecodeArgs& a = c.a;
-    const int hs = a.head_size;
     constexpr int ngroups = kIoThreads / kGroup;
     constexpr int kRounds = (ngroups >= kAttSubBlock) ? 1 : (kAttSubBlock / ngroups > 4 ? 4 : kAttSubBlock / ngroups);
     constexpr int kSub = ngroups * kRounds;  // positions per sub-block, <= max(kAttSubBlock, kIoThreads)
@@ -830,7 +852,7 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
         const int wanted = has_current ? 3 * hs : hs;  // at most 2 * kIoThreads
         if (io.it < wanted) {
             auto source = [&](int idx) -> const u64* {
-                const int which = idx / hs, e = idx - which * hs;
+                const int which = div_head_size(c, idx), e = idx - which * hs;
                 return which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
                                   : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
             };
@@ -839,7 +861,7 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
             poll_n<2>([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
             for (int j = 0; j < 2; ++j) {
                 const int idx = j == 0 ? io.it : second;
-                const int which = idx / hs, e = idx - which * hs;
+                const int which = div_head_size(c, idx), e = idx - which * hs;
                 // k and v as the cache will hold them
                 l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[j] : f16_bits_to_f32(f32_to_f16_bits(in[j]));
             }
@@ -919,11 +941,12 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
         parity ^= 1;
     }
     // groups of one wavefront by lane exchange, wavefronts through LDS
+    const int merge_lane = fresh_lane();
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float v = acc[e];
 #pragma unroll
-        for (int o = kGroup; o < kWave; o <<= 1) v += __shfl_xor(v, o);
+        for (int o = kGroup; o < kWave; o <<= 1) v += lane_xor(v, o, merge_lane);
         acc[e] = v;
     }
     if (lane_id() < kGroup) {
@@ -951,13 +974,218 @@ __device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer
     }
 }
 
+// exp(x) for the long-context items: one hardware exponential.  (About an ulp off expf; the
+// weights it forms are normalised by their own sum.)
+__device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+
+// One long-context work item: kHeads query heads that share a KV head, context split `split` of
+// `nsplits`.  Every K and V row of the split is fetched ONCE and used for all kHeads heads (the
+// per-head item above reads it once per head, which at 8K positions is four times the cache
+// traffic of the Llama-3 shapes).  No score ever goes to LDS and nothing synchronises inside the
+// loop: every lane group keeps its own running maximum, sum and weighted V sum per head and
+// rescales them when the maximum grows; the groups' results are merged at the end, inside a
+// wavefront by lane exchange, across wavefronts through LDS (the same merge the splits undergo
+// later in att_combine).  model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped.
+template <int kGroup, int kHeads>
+__device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int layer, int h0, int split, int nsplits,
+                                               int npos, bool first_item, int hs) {
+    static_assert(kHeads <= kMaxAttHeads, "LDS areas are sized for kMaxAttHeads heads");
+    const DecodeArgs& a = c.a;
+    constexpr int ngroups = kIoThreads / kGroup;
+    constexpr int kRounds = 2;
+    constexpr int kSub = ngroups * kRounds;
+    const int kvh = h0 / a.gqa;
+    const int sub = io.it % kGroup, grp = io.it / kGroup;
+    const bool lane_live = sub * 8 < hs;
+    const int off = lane_live ? sub * 8 : 0;
+
+    const int chunk = (npos + nsplits - 1) / nsplits;
+    const int t_begin = split * chunk;
+    const int t_end = min(npos, t_begin + chunk);
+    const int current = npos - 1;
+    const bool has_current = current >= t_begin && current < t_end;
+    const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
+    const uint16_t* kbase = a.key_cache + head_base;
+    const uint16_t* vbase = a.value_cache + head_base;
+
+    uintx4 krow[kRounds], vrow[kRounds];
+    auto request_rows = [&](uintx4 (&rows)[kRounds], const uint16_t* base, int b0) {
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            rows[j] = uintx4{0u, 0u, 0u, 0u};
+            if (t < t_end && t != current && lane_live) rows[j] = load16(base + static_cast<size_t>(t) * hs + off);
+        }
+    };
+    request_rows(krow, kbase, t_begin);
+    request_rows(vrow, vbase, t_begin);
+
+    // q of the item's heads (and, in the last split, k and v of the current position): LDS rows
+    // 0 .. kHeads-1 hold q, rows kHeads and kHeads+1 hold k and v as the cache will hold them
+    const unsigned tag_in = c.seq(layer, kQkv);
+    if (!first_item) io_sync(c.ctl, io);  // the previous item's readers have left the LDS areas
+    {
+        const int wanted = (kHeads + (has_current ? 2 : 0)) * hs;  // at most 6 * 128 <= 2 * kIoThreads
+        if (io.it < wanted) {
+            auto source = [&](int idx) -> const u64* {
+                const int which = div_head_size(c, idx), e = idx - which * hs;
+                return which < kHeads ? c.t.q + static_cast<size_t>(h0 + which) * hs + e
+                                      : (which == kHeads ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
+            };
+            const int second = io.it + kIoThreads < wanted ? io.it + kIoThreads : io.it;
+            float in[2];
+            poll_n<2>([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
+            for (int j = 0; j < 2; ++j) {
+                const int idx = j == 0 ? io.it : second;
+                const int which = div_head_size(c, idx), e = idx - which * hs;
+                l.qkv[which * kMaxHeadPad + e] = which < kHeads ? in[j] : f16_bits_to_f32(f32_to_f16_bits(in[j]));
+            }
+        }
+    }
+    if (first_item) mark(c, io, 5);
+    io_sync(c.ctl, io);
+    if (first_item) {
+        mark(c, io, 1);
+        mark(c, io, 6);
+        mark(c, io, 2);
+    }
+    uintx4 cur_k = uintx4{0u, 0u, 0u, 0u}, cur_v = uintx4{0u, 0u, 0u, 0u};
+    if (has_current && lane_live) {
+        union {
+            half8_t h;
+            uintx4 u;
+        } pk, pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pk.h[e] = static_cast<half_t>(l.qkv[kHeads * kMaxHeadPad + off + e]);
+            pv.h[e] = static_cast<half_t>(l.qkv[(kHeads + 1) * kMaxHeadPad + off + e]);
+        }
+        cur_k = pk.u;
+        cur_v = pv.u;
+    }
+
+    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
+    float top[kHeads], lsum[kHeads], acc[kHeads][8];
+#pragma unroll
+    for (int h = 0; h < kHeads; ++h) {
+        top[h] = -INFINITY;
+        lsum[h] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
+    }
+    for (int b0 = t_begin; b0 < t_end; b0 += kSub) {
+        float score[kRounds][kHeads];
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            const half8_t kh = as_half8((t == current) ? cur_k : krow[j]);
+#pragma unroll
+            for (int h = 0; h < kHeads; ++h) {
+                // (q comes from LDS every time: lanes with the same `sub` read the same words, and
+                // four heads of q would not fit the register file beside their accumulators)
+                const floatx4 qa = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + off);
+                const floatx4 qb = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + off + 4);
+                float s = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s = fmaf(static_cast<float>(kh[e]), qa[e], s);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s = fmaf(static_cast<float>(kh[4 + e]), qb[e], s);
+                s = lane_live ? s : 0.0f;
+                s = group_sum<kGroup>(s) * scale;
+                score[j][h] = (t < t_end) ? s : -INFINITY;
+            }
+        }
+        if (b0 + kSub < t_end) request_rows(krow, kbase, b0 + kSub);
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int t = b0 + grp + j * ngroups;
+            const half8_t vh = as_half8((t == current) ? cur_v : vrow[j]);
+#pragma unroll
+            for (int h = 0; h < kHeads; ++h) {
+                const float s = score[j][h];
+                const float grown = fmaxf(top[h], s);
+                const float corr = (top[h] == -INFINITY) ? 0.0f : exp_fast(top[h] - grown);
+                const float p = (s == -INFINITY) ? 0.0f : exp_fast(s - grown);
+                top[h] = grown;
+                lsum[h] = lsum[h] * corr + p;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(static_cast<float>(vh[e]), p, acc[h][e] * corr);
+            }
+        }
+        if (b0 + kSub < t_end) request_rows(vrow, vbase, b0 + kSub);
+    }
+    // the lane groups of a wavefront, by lane exchange
+    const int merge_lane = fresh_lane();
+#pragma unroll
+    for (int h = 0; h < kHeads; ++h) {
+        float all = top[h];
+#pragma unroll
+        for (int o = kGroup; o < kWave; o <<= 1) all = fmaxf(all, lane_xor(all, o, merge_lane));
+        const float f = (top[h] == -INFINITY) ? 0.0f : exp_fast(top[h] - all);
+        float ls = lsum[h] * f;
+#pragma unroll
+        for (int o = kGroup; o < kWave; o <<= 1) ls += lane_xor(ls, o, merge_lane);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float v = acc[h][e] * f;
+#pragma unroll
+            for (int o = kGroup; o < kWave; o <<= 1) v += lane_xor(v, o, merge_lane);
+            acc[h][e] = v;
+        }
+        top[h] = all;
+        lsum[h] = ls;
+    }
+    if (lane_id() < kGroup) {
+#pragma unroll
+        for (int h = 0; h < kHeads; ++h) {
+            float* r = l.red + (io.iw * kMaxAttHeads + h) * kRedStride;
+            if (lane_live) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) r[sub * 8 + e] = acc[h][e];
+            }
+            if (sub == 0) {
+                r[kMaxHeadPad] = top[h];
+                r[kMaxHeadPad + 1] = lsum[h];
+            }
+        }
+    }
+    if (first_item) mark(c, io, 7);
+    io_sync(c.ctl, io);
+    if (first_item) mark(c, io, 3);
+    // the wavefronts, through LDS: thread (h, e)
+    const unsigned tag_out = c.seq(layer, kAtt);
+    if (io.it < kHeads * hs) {
+        const int h = div_head_size(c, io.it), e = io.it - h * hs;
+        float all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) all = fmaxf(all, l.red[(w * kMaxAttHeads + h) * kRedStride + kMaxHeadPad]);
+        float o = 0.0f, ls = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) {
+            const float* r = l.red + (w * kMaxAttHeads + h) * kRedStride;
+            const float f = (r[kMaxHeadPad] == -INFINITY) ? 0.0f : exp_fast(r[kMaxHeadPad] - all);
+            o += r[e] * f;
+            ls += r[kMaxHeadPad + 1] * f;
+        }
+        if (nsplits == 1) {
+            publish(c.t.xb + static_cast<size_t>(h0 + h) * hs + e, o / ls, tag_out);
+        } else {
+            u64* part = c.t.part + (static_cast<size_t>(h0 + h) * c.t.splits_cap + split) * (hs + 2);
+            publish(part + e, o, tag_out);
+            if (e == 0) {
+                publish(part + hs, all, tag_out);
+                publish(part + hs + 1, ls, tag_out);
+            }
+        }
+    }
+}
+
 // Combine the context splits of head h: collect every split's (output, max,
 // sum), rescale to the common maximum and normalise.  Runs after the workgroup
 // has published all of its own partials, so a workgroup waiting here never
 // holds back a partial another combiner needs.
-__device__ __forceinline__ void att_combine(Ctx& c, Io& io, const Lds& l, int layer, int h, int nsplits) {
-    const DecodeArgs& a = c.a;
-    const int hs = a.head_size, stride = hs + 2;
+__device__ __forceinline__ void att_combine(Ctx& c, Io& io, const Lds& l, int layer, int h, int nsplits, int hs) {
+    const int stride = hs + 2;
     const unsigned tag_out = c.seq(layer, kAtt);
     io_sync(c.ctl, io);  // earlier readers of gather have left
     const u64* src = c.t.part + static_cast<size_t>(h) * c.t.splits_cap * stride;
@@ -983,10 +1211,11 @@ __device__ __forceinline__ void att_combine(Ctx& c, Io& io, const Lds& l, int la
 // the split counts that keep an item within 2 * kItemPositions positions, the cheapest wins and the
 // smaller of equals: at 8193 positions and 32 heads on 256 workgroups that is 8 splits of 1025
 // positions in one round, where 9 splits of 911 would leave 32 workgroups a second item.
-__device__ __forceinline__ int item_splits(int npos, int cap, int n_heads, int nwg) {
+__host__ __device__ inline int item_splits(int npos, int cap, int n_heads, int nwg) {
     constexpr int kCombineCost = 300;
     int best = 1, best_cost = 0x7fffffff;
-    const int first = max(1, (npos + 2 * kItemPositions - 1) / (2 * kItemPositions));
+    int first = (npos + 2 * kItemPositions - 1) / (2 * kItemPositions);
+    if (first < 1) first = 1;
     for (int s = first; s <= cap; ++s) {
         const int rounds = (n_heads * s + nwg - 1) / nwg;
         const int cost = rounds * ((npos + s - 1) / s) + (s > 1 ? kCombineCost : 0);
@@ -998,27 +1227,79 @@ __device__ __forceinline__ int item_splits(int npos, int cap, int n_heads, int n
     return best;
 }
 
+// Splits for items that cover several heads: as item_splits, with an item's length counted in
+// whole passes of `sub_positions` positions (what one trip round its loop handles).
+__host__ __device__ inline int group_item_splits(int npos, int cap, int n_chunks, int nwg, int sub_positions) {
+    constexpr int kCombineCost = 300;
+    int best = 1, best_cost = 0x7fffffff;
+    for (int s = 1; s <= cap; ++s) {
+        const int rounds = (n_chunks * s + nwg - 1) / nwg;
+        const int passes = ((npos + s - 1) / s + sub_positions - 1) / sub_positions;
+        const int cost = rounds * passes * sub_positions + (s > 1 ? kCombineCost : 0);
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = s;
+        }
+    }
+    return best;
+}
+
 __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int layer) {
     const DecodeArgs& a = c.a;
     const int npos = c.pos + 1;
-    const int nsplits = item_splits(npos, c.t.splits_cap, a.n_heads, c.nwg);
-    const int items = a.n_heads * nsplits;
+    // (Index arithmetic of this phase divides by the head size through a host-made multiplier and by the
+    // split count through an opaque copy: a division by a value that does not change from layer to layer
+    // has its reciprocal worked out once per token otherwise, and kept in a vector register that the busy
+    // stretches of the layer loop then spill.)
     const int hs = a.head_size;
     bool first = true;
     mark(c, io, 0);
+    // Long contexts of grouped-query models: one item covers the heads that share a KV head (four at a
+    // time), so that the cache is read once.  Short contexts keep one item per head and no combine pass.
+    constexpr int heads_per_item = 2;
+    if (c.t.att_group_splits > 0) {
+        const int n_chunks = a.n_heads / heads_per_item;
+        int nsplits = c.t.att_group_splits;
+        asm volatile("" : "+s"(nsplits));
+        const int items = n_chunks * nsplits;
+        for (int item = c.wg; item < items; item += c.nwg) {
+            const int chunk = item / nsplits, split = item - chunk * nsplits;
+            const int h0 = chunk * heads_per_item;
+            io.it = exchange_thread_index(io.iw);
+            if (hs <= 64) att_group_item<8, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
+            else att_group_item<16, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
+            first = false;
+        }
+        if (nsplits > 1) {
+            // the heads of a chunk are combined by the workgroups that held its first splits
+            for (int item = c.wg; item < items; item += c.nwg) {
+                const int chunk = item / nsplits, split = item - chunk * nsplits;
+                for (int j = split; j < heads_per_item; j += nsplits) {
+                    io.it = exchange_thread_index(io.iw);
+                    att_combine(c, io, l, layer, chunk * heads_per_item + j, nsplits, hs);
+                }
+            }
+        }
+        mark(c, io, 4);
+        ++c.phase_index;
+        return;
+    }
+    int nsplits = c.t.att_splits;
+    asm volatile("" : "+s"(nsplits));
+    const int items = a.n_heads * nsplits;
     for (int item = c.wg; item < items; item += c.nwg) {
         const int h = item / nsplits, split = item - h * nsplits;
         io.it = exchange_thread_index(io.iw);
         // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
-        if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first);
-        else att_item<16>(c, io, l, layer, h, split, nsplits, npos, first);
+        if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first, hs);
+        else att_item<16>(c, io, l, layer, h, split, nsplits, npos, first, hs);
         first = false;
     }
     if (nsplits > 1) {
         for (int item = c.wg; item < items; item += c.nwg) {
             const int h = item / nsplits, split = item - h * nsplits;
             io.it = exchange_thread_index(io.iw);
-            if (split == 0) att_combine(c, io, l, layer, h, nsplits);
+            if (split == 0) att_combine(c, io, l, layer, h, nsplits, hs);
         }
     }
     mark(c, io, 4);
@@ -1254,8 +1535,8 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.results = l.xs + b.xs_floats;
     l.sc = l.results + b.results_floats;
     l.qkv = l.sc + 2 * kAttScoreFloats;
-    l.red = l.qkv + 3 * kMaxHeadPad;
-    l.gather = l.red + kIoWaves * kMaxHeadPad;
+    l.red = l.qkv + (kMaxAttHeads + 2) * kMaxHeadPad;
+    l.gather = l.red + kIoWaves * kMaxAttHeads * kRedStride;
     for (unsigned i = threadIdx.x; i < sizeof(Control) / sizeof(unsigned); i += blockDim.x)
         reinterpret_cast<unsigned*>(&ctl)[i] = 0u;
     __syncthreads();  // the only workgroup-wide barrier: the two kinds of wavefronts part ways here
@@ -1281,8 +1562,9 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
 namespace {
 
 int splits_cap_for(const lpp_model* m) {
-    const int s = (m->cfg.seq_len + df::kItemPositions - 1) / df::kItemPositions;
-    return s < 1 ? 1 : s;
+    // enough for long-context items of a few hundred positions each
+    const int s = (m->cfg.seq_len + 127) / 128;
+    return s < 1 ? 1 : (s > 64 ? 64 : s);
 }
 
 struct Plan {
@@ -1319,7 +1601,8 @@ Plan plan_for(const lpp_model* m) {
     b.results_floats = (slots + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
     p.lds_bytes = static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
-                                      (df::kIoWaves + 3) * df::kMaxHeadPad + b.gather_floats) * sizeof(float);
+                                      (df::kMaxAttHeads + 2) * df::kMaxHeadPad + df::kIoWaves * df::kMaxAttHeads * df::kRedStride +
+                                      b.gather_floats) * sizeof(float);
     return p;
 }
 
@@ -1342,7 +1625,17 @@ df::Tagged tagged_of(const lpp_model* m, bool generating) {
     t.part = p;         p += static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2);
     t.stats = p;
     t.splits_cap = splits_cap_for(m);
+    t.hs_magic = static_cast<unsigned>((1ull << 32) / static_cast<unsigned long long>(m->head_size)) + 1u;
     t.pos = m->df_pos;
+    {
+        const int npos = m->df_pos + 1, nwg = m->persist_grid > 0 ? m->persist_grid : compute_units();
+        t.att_splits = df::item_splits(npos, t.splits_cap, c.n_heads, nwg);
+        t.att_group_splits = 0;
+        if (m->gqa % 2 == 0 && t.att_splits > 1) {
+            const int sub_positions = (m->head_size <= 64 ? df::kIoThreads / 8 : df::kIoThreads / 16) * 2;
+            t.att_group_splits = df::group_item_splits(npos, t.splits_cap, c.n_heads / 2, nwg, sub_positions);
+        }
+    }
     t.history_len = m->df_history_len;
     t.temperature = m->df_temperature;
     t.penalty = m->df_penalty;
