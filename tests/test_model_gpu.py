@@ -203,13 +203,24 @@ def test_forward_then_generate_continuation():
     o.close()
 
 
-def test_long_context_attention_matches_oracle():
+LONG_CONTEXT = {
+    # name: (Shape, first position).  The persistent kernel gives grouped-query models work items that
+    # cover two query heads of a KV head once the context is long enough to be split.
+    "gqa4_hs32": (Shape(256, 512, 2, 8, 2, 1000, 4400, 500000.0, fp16=True, tied=True), 4300),
+    "gqa8_hs32": (Shape(256, 512, 2, 8, 1, 1000, 4400, 500000.0, fp16=True, tied=True), 4300),
+    "gqa2_hs128": (Shape(512, 512, 1, 4, 2, 500, 2400, 500000.0, fp16=True, tied=False), 2300),
+    "mha_hs48_fp32": (Shape(192, 384, 2, 4, 4, 500, 4400, 10000.0, fp16=False, tied=True), 4300),
+    "gqa2_hs64_just_split": (Shape(256, 512, 1, 4, 2, 500, 1100, 10000.0, fp16=True, tied=True), 1040),
+}
+
+
+@pytest.mark.parametrize("name", list(LONG_CONTEXT))
+def test_long_context_attention_matches_oracle(name):
     """Config-4 style: cache pre-filled with binary16 N(0,1) up to a long position,
     then decode there; the split-context attention must agree with the CPU loop."""
-    shape = Shape(256, 512, 2, 8, 2, 1000, 4400, 500000.0, fp16=True, tied=True)
+    shape, start = LONG_CONTEXT[name]
     m, o = build(shape, 8)
     hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
-    start = 4300
     n = L * nkv * shape.seq_len * hs
     kfill = capi.synth_normal_f16(n, 501, 1.0).reshape(L, nkv, shape.seq_len, hs)
     vfill = capi.synth_normal_f16(n, 502, 1.0).reshape(L, nkv, shape.seq_len, hs)
