@@ -350,8 +350,9 @@ lpp_status lpp_profile_kernels(lpp_model *m, int pos, int reps, lpp_kernel_time 
  * o-projection, gate/up, down; then classifier and sampler.  Marks of a GEMV
  * phase: 0 phase entered, 1 own inputs received, 2 inputs staged, 3 row results
  * ready, 4 outputs published, 5 first weight step multiplied, 6 last row
- * finished.  Attention: 0 entered, 5 q/k/v received, 1 shared, 6 scores
- * computed, 2 scores exchanged, 7 values accumulated, 3 reduced, 4 published.
+ * finished.  Attention (first work item): 0 entered, 5 q/k/v received, 1 = 6 = 2
+ * shared through LDS, 7 context walked, 3 lane groups and wavefronts merged,
+ * 4 published.
  * *count = marks * phases, *marks_per_phase = marks. */
 lpp_status lpp_trace_token(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count,
                            int *marks_per_phase);

@@ -57,8 +57,7 @@ constexpr int kDepth = 4;                          // weight steps a streaming w
 constexpr int kStepLoads = 4;                      // 16-byte loads per lane and step: 4 KiB of one row
 constexpr int kPollBatch = 8;                      // tagged values one thread requests before checking any
 constexpr int kItemPositions = 1024;               // context positions per attention work item
-constexpr int kAttSubBlock = 256;                  // positions scored between two barriers of an item
-constexpr int kAttScoreFloats = 512;               // one score area (a sub-block never exceeds kIoThreads positions)
+constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS copy of the penalty window
 constexpr int kMaxHeadPad = 128;
 constexpr int kMaxAttHeads = 4;                    // query heads of one KV head a long-context work item covers
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
@@ -608,7 +607,7 @@ struct Lds {
     float* xraw;     // [dim_pad]   residual stream as last received
     float* xs;       // [xs_floats] staged GEMV input; sampler tables after the classifier
     float* results;  // [results_floats] row results of the current GEMV phase
-    float* sc;       // [2][kAttScoreFloats] attention scores of a sub-block, two areas taking turns
+    float* sc;       // [2 * kAttScoreFloats] the sampler's copy of the penalty window (as ints)
     float* qkv;      // [kMaxAttHeads + 2][kMaxHeadPad] this token's q (per head of the item), k, v
     float* red;      // [kIoWaves][kMaxAttHeads][kRedStride] attention cross-wavefront reduction
     float* gather;   // [gather_floats] attention split partials
@@ -800,187 +799,17 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
 // Attention (exchange wavefronts)
 // ---------------------------------------------------------------------------
 
-// One work item: query head h, context split `split` of `nsplits` (at most
-// kItemPositions positions), walked in sub-blocks of a few rounds of one
-// position per lane group (kGroup lanes cover one position, 8 binary16 each).
-// K and V rows of earlier positions do not depend on this token: the first
-// sub-block's rows are requested before q is polled, each later sub-block's as
-// soon as the registers are free.  The current position's k and v arrive
-// tagged and are rounded to binary16 exactly as the cache store rounds them.
-// Scores of a sub-block go to LDS once; every wavefront then forms the
-// sub-block's maximum and sum of exponentials for itself and carries the
-// running maximum (model.cpp:186-198 with the softmax of ops.cpp:56-75,
-// regrouped).
-template <int kGroup>
-__device__ __forceinline__ void att_item(Ctx& c, Io& io, const Lds& l, int layer, int h, int split, int nsplits,
-                                         int npos, bool first_item, int hs) {
-    const DecodeArgs& a = c.a;
-    constexpr int ngroups = kIoThreads / kGroup;
-    constexpr int kRounds = (ngroups >= kAttSubBlock) ? 1 : (kAttSubBlock / ngroups > 4 ? 4 : kAttSubBlock / ngroups);
-    constexpr int kSub = ngroups * kRounds;  // positions per sub-block, <= max(kAttSubBlock, kIoThreads)
-    const int kvh = h / a.gqa;
-    const int sub = io.it % kGroup, grp = io.it / kGroup;
-    const bool lane_live = sub * 8 < hs;
-    const int off = lane_live ? sub * 8 : 0;
-
-    const int chunk = (npos + nsplits - 1) / nsplits;
-    const int t_begin = split * chunk;
-    const int t_end = min(npos, t_begin + chunk);
-    const int current = npos - 1;
-    const bool has_current = current >= t_begin && current < t_end;
-    const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
-    const uint16_t* kbase = a.key_cache + head_base;
-    const uint16_t* vbase = a.value_cache + head_base;
-
-    uintx4 krow[kRounds], vrow[kRounds];
-    auto request_rows = [&](uintx4 (&rows)[kRounds], const uint16_t* base, int b0) {
-#pragma unroll
-        for (int j = 0; j < kRounds; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            rows[j] = uintx4{0u, 0u, 0u, 0u};
-            if (t < t_end && t != current && lane_live) rows[j] = load16(base + static_cast<size_t>(t) * hs + off);
-        }
-    };
-    request_rows(krow, kbase, t_begin);
-    request_rows(vrow, vbase, t_begin);
-
-    // this token's q (and, in the last split, k and v of the current position):
-    // one value per thread, shared through LDS
-    const unsigned tag_in = c.seq(layer, kQkv);
-    if (!first_item) io_sync(c.ctl, io);  // the previous item's readers have left the LDS areas
-    {
-        const int wanted = has_current ? 3 * hs : hs;  // at most 2 * kIoThreads
-        if (io.it < wanted) {
-            auto source = [&](int idx) -> const u64* {
-                const int which = div_head_size(c, idx), e = idx - which * hs;
-                return which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
-                                  : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
-            };
-            const int second = io.it + kIoThreads < wanted ? io.it + kIoThreads : io.it;
-            float in[2];
-            poll_n<2>([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
-            for (int j = 0; j < 2; ++j) {
-                const int idx = j == 0 ? io.it : second;
-                const int which = div_head_size(c, idx), e = idx - which * hs;
-                // k and v as the cache will hold them
-                l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[j] : f16_bits_to_f32(f32_to_f16_bits(in[j]));
-            }
-        }
-    }
-    if (first_item) mark(c, io, 5);
-    io_sync(c.ctl, io);
-    if (first_item) mark(c, io, 1);
-    float qv[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) qv[e] = lane_live ? l.qkv[off + e] : 0.0f;
-    // the current position's row as the cache will hold it, ready to stand in for a loaded row
-    // (a register select: a conditional LDS read per element costs a branch each)
-    uintx4 cur_k = uintx4{0u, 0u, 0u, 0u}, cur_v = uintx4{0u, 0u, 0u, 0u};
-    if (has_current && lane_live) {
-        union {
-            half8_t h;
-            uintx4 u;
-        } pk, pv;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            pk.h[e] = static_cast<half_t>(l.qkv[kMaxHeadPad + off + e]);
-            pv.h[e] = static_cast<half_t>(l.qkv[2 * kMaxHeadPad + off + e]);
-        }
-        cur_k = pk.u;
-        cur_v = pv.u;
-    }
-
-    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
-    float run_max = -INFINITY, run_sum = 0.0f;
-    float acc[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
-    int parity = 0;
-    for (int b0 = t_begin; b0 < t_end; b0 += kSub) {
-        const int n = min(kSub, t_end - b0);
-        float* sc = l.sc + parity * kAttScoreFloats;  // two score areas take turns: one barrier per sub-block is enough
-        float score[kRounds];
-#pragma unroll
-        for (int j = 0; j < kRounds; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            const half8_t kh = as_half8((t == current) ? cur_k : krow[j]);
-            float s = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf(static_cast<float>(kh[e]), qv[e], s);
-            s = group_sum<kGroup>(s) * scale;
-            score[j] = s;
-            if (t < t_end && sub == 0) sc[t - b0] = s;
-        }
-        if (b0 + kSub < t_end) request_rows(krow, kbase, b0 + kSub);
-        if (first_item && b0 == t_begin) mark(c, io, 6);
-        io_sync(c.ctl, io);
-        if (first_item && b0 == t_begin) mark(c, io, 2);
-        // every wavefront: the sub-block's maximum and sum of exponentials
-        float m = -INFINITY;
-        for (int i = lane_id(); i < n; i += kWave) m = fmaxf(m, sc[i]);
-        m = fmaxf(wave_max(m), run_max);
-        float lsum = 0.0f;
-        for (int i = lane_id(); i < n; i += kWave) lsum += expf(sc[i] - m);
-        lsum = wave_sum(lsum);
-        const float corr = (run_max == -INFINITY) ? 0.0f : expf(run_max - m);
-        run_sum = run_sum * corr + lsum;
-        run_max = m;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] *= corr;
-#pragma unroll
-        for (int j = 0; j < kRounds; ++j) {
-            const int t = b0 + grp + j * ngroups;
-            if (t < t_end) {
-                const float p = expf(score[j] - m);
-                const half8_t vh = as_half8((t == current) ? cur_v : vrow[j]);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[e] = fmaf(static_cast<float>(vh[e]), p, acc[e]);
-            }
-        }
-        if (b0 + kSub < t_end) request_rows(vrow, vbase, b0 + kSub);
-        parity ^= 1;
-    }
-    // groups of one wavefront by lane exchange, wavefronts through LDS
-    const int merge_lane = fresh_lane();
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        float v = acc[e];
-#pragma unroll
-        for (int o = kGroup; o < kWave; o <<= 1) v += lane_xor(v, o, merge_lane);
-        acc[e] = v;
-    }
-    if (lane_id() < kGroup) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) l.red[io.iw * kMaxHeadPad + sub * 8 + e] = acc[e];
-    }
-    if (first_item) mark(c, io, 7);
-    io_sync(c.ctl, io);
-    if (first_item) mark(c, io, 3);
-    const unsigned tag_out = c.seq(layer, kAtt);
-    if (io.it < hs) {
-        float o = 0.0f;
-#pragma unroll
-        for (int w = 0; w < kIoWaves; ++w) o += l.red[w * kMaxHeadPad + io.it];
-        if (nsplits == 1) {
-            publish(c.t.xb + static_cast<size_t>(h) * hs + io.it, o / run_sum, tag_out);
-        } else {
-            u64* part = c.t.part + (static_cast<size_t>(h) * c.t.splits_cap + split) * (hs + 2);
-            publish(part + io.it, o, tag_out);
-            if (io.it == 0) {
-                publish(part + hs, run_max, tag_out);
-                publish(part + hs + 1, run_sum, tag_out);
-            }
-        }
-    }
-}
-
-// exp(x) for the long-context items: one hardware exponential.  (About an ulp off expf; the
-// weights it forms are normalised by their own sum.)
+// exp(x) as one hardware exponential.  (About an ulp off expf; the weights it forms are
+// normalised by their own sum.)
 __device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
 
-// One long-context work item: kHeads query heads that share a KV head, context split `split` of
-// `nsplits`.  Every K and V row of the split is fetched ONCE and used for all kHeads heads (the
-// per-head item above reads it once per head, which at 8K positions is four times the cache
+// One attention work item: kHeads query heads that share a KV head (one head for short contexts
+// and for models without grouped queries), context split `split` of `nsplits`.  kGroup lanes cover
+// one position, 8 binary16 each.  K and V rows of earlier positions do not depend on this token:
+// the first rows are requested before q is polled, each later pass's as soon as the registers are
+// free.  The current position's k and v arrive tagged and are rounded to binary16 exactly as the
+// cache store rounds them.  Every K and V row of the split is fetched ONCE and used for all kHeads
+// heads (per-head items would read it once per head, which at 8K positions is four times the cache
 // traffic of the Llama-3 shapes).  No score ever goes to LDS and nothing synchronises inside the
 // loop: every lane group keeps its own running maximum, sum and weighted V sum per head and
 // rescales them when the maximum grows; the groups' results are merged at the end, inside a
@@ -1291,8 +1120,8 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
         const int h = item / nsplits, split = item - h * nsplits;
         io.it = exchange_thread_index(io.iw);
         // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
-        if (hs <= 64) att_item<8>(c, io, l, layer, h, split, nsplits, npos, first, hs);
-        else att_item<16>(c, io, l, layer, h, split, nsplits, npos, first, hs);
+        if (hs <= 64) att_group_item<8, 1>(c, io, l, layer, h, split, nsplits, npos, first, hs);
+        else att_group_item<16, 1>(c, io, l, layer, h, split, nsplits, npos, first, hs);
         first = false;
     }
     if (nsplits > 1) {
