@@ -56,10 +56,10 @@ constexpr int kIoThreads = kIoWaves * kWave;
 constexpr int kDepth = 4;                          // weight steps a streaming wavefront keeps in flight
 constexpr int kStepLoads = 4;                      // 16-byte loads per lane and step: 4 KiB of one row
 constexpr int kPollBatch = 8;                      // tagged values one thread requests before checking any
-constexpr int kItemPositions = 1024;               // context positions per attention work item
+constexpr int kItemPositions = 1024;               // a one-head attention work item stays within twice this many positions
 constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS copy of the penalty window
 constexpr int kMaxHeadPad = 128;
-constexpr int kMaxAttHeads = 4;                    // query heads of one KV head a long-context work item covers
+constexpr int kMaxAttHeads = 2;                    // query heads of one KV head a long-context work item covers
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
 
 typedef unsigned long long u64;
@@ -112,9 +112,9 @@ struct Blocks {
     int gather_floats;
 };
 
-// Workgroup-local coordination words.  Everything here is accessed with plain
-// (volatile) LDS operations: LDS executes one wavefront's operations in order,
-// so a flag written after data is seen after the data.
+// Workgroup-local coordination words, accessed with relaxed workgroup-scope atomics
+// (plain ds_read / ds_write): LDS executes one wavefront's operations in order, so a
+// flag written after data is seen after the data.
 struct Control {
     unsigned staged;                 // += 1 by every exchange wavefront once it has staged a GEMV phase
     unsigned io_bar;                 // arrival counter of the exchange wavefronts' barrier
