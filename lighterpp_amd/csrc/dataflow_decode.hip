@@ -619,7 +619,7 @@ struct Lds {
 __device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, int n, unsigned want) {
     const int n_pad = (n + 7) & ~7;
     for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
-    poll_values<8192 / kIoThreads>(src, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });  // 8192 values in one go
+    poll_values<kPollBatch>(src, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });
     mark(c, io, 1);
     signal_staged(c.ctl);
 }
@@ -639,7 +639,7 @@ __device__ __forceinline__ float stage_norm(Ctx& c, Io& io, const Lds& l, const 
     const int it = exchange_thread_index(io.iw);
     // The gains do not depend on anything: request this thread's first few before polling, so that
     // their memory latency is spent while the inputs are still on their way.
-    constexpr int kEarly = 8;
+    constexpr int kEarly = 4;
     float early_gain[kEarly];
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
@@ -662,8 +662,8 @@ __device__ __forceinline__ float stage_norm(Ctx& c, Io& io, const Lds& l, const 
         }
         for (int i = it + kEarly * kIoThreads; i < n; i += kIoThreads) take(i, plain_x[i], gain[i]);
     } else {
-        static_assert(kEarly == kPollBatch, "the first round of polls covers exactly the values whose gains were requested early");
-        poll_values(tagged_x, n, want, c, io,
+        // (the first round of polls covers exactly the values whose gains were requested early)
+        poll_values<kEarly>(tagged_x, n, want, c, io,
                     [&](int i, float v, int j, bool first_round) { take(i, v, first_round ? early_gain[j] : gain[i]); });
     }
     mark(c, io, 1);
