@@ -117,6 +117,7 @@ struct Blocks {
 // flag written after data is seen after the data.
 struct Control {
     unsigned staged;                 // += 1 by every exchange wavefront once it has staged a GEMV phase
+    unsigned received;               // += 1 by every exchange wavefront once the inputs of a phase (attention included) are in
     unsigned io_bar;                 // arrival counter of the exchange wavefronts' barrier
     alignas(16) unsigned progress[kGemvWaves];   // GEMV phases wavefront j has completed
     float red[2][kIoWaves];
@@ -399,9 +400,28 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
             } else {
                 more = false;
             }
-            if (kPaceSleep > 0 && ((pace >> k) & 1u)) {
-                __builtin_amdgcn_s_sleep(kPaceSleep);
+            if ((pace >> k) & 1u) {
+                // A refill after a burst that finished the wavefront's rows of phase cur_p.  A row of the
+                // very next GEMV phase goes out after a short pause, right behind the publishing stores
+                // (it must be there when that phase's inputs are).  Anything later is held until the inputs
+                // of the phase after this one have arrived: from then until that phase publishes, nothing
+                // of this workgroup's is on its way through the memory system, and a request costs no
+                // hand-over anything; sent now, it would sit in the queues in front of the values being
+                // handed over.
                 pace &= ~(1u << k);
+                const unsigned nm = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot0 + k));
+                const unsigned nq = (nm >> kStepPhaseShift) & kStepPhaseMask;
+                if ((nm & kStepValid) == 0u) {
+                    // past the wavefront's last step: nothing left to hold back
+                } else if (nq == cur_p + 1u) {
+                    __builtin_amdgcn_s_sleep(kPaceSleep);
+                } else {
+                    // phases in the exchange wavefronts' count (five per layer): qkv, attention, O, gate/up, down
+                    const unsigned io_phase = 5u * (cur_p >> 2) + ((cur_p & 3u) == 0u ? 0u : (cur_p & 3u) + 1u);
+                    const unsigned need = static_cast<unsigned>(kIoWaves) * (io_phase + 2u);
+                    lds_wait(&ctl.error, [&]() { return static_cast<int>(lds_peek(&ctl.received) - need) >= 0; });
+                    compiler_fence();
+                }
             }
             request(k, batch, slot0 + k);
         }
@@ -493,6 +513,11 @@ __device__ __forceinline__ float io_max(Control& ctl, Io& io, float v) {
 __device__ __forceinline__ void signal_staged(Control& ctl) {
     compiler_fence();
     if (lane_id() == 0) __hip_atomic_fetch_add(&ctl.staged, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+// The inputs of the current phase have arrived: for a while now nothing of this workgroup's is on
+// its way through the memory system, which is when the streaming wavefronts let held-back requests go.
+__device__ __forceinline__ void signal_received(Control& ctl) {
+    if (lane_id() == 0) __hip_atomic_fetch_add(&ctl.received, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 // Wait until every streaming wavefront has completed GEMV phase p.
@@ -621,6 +646,7 @@ __device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u6
     for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
     poll_values<kPollBatch>(src, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });
     mark(c, io, 1);
+    signal_received(c.ctl);
     signal_staged(c.ctl);
 }
 
@@ -667,6 +693,7 @@ __device__ __forceinline__ float stage_norm(Ctx& c, Io& io, const Lds& l, const 
                     [&](int i, float v, int j, bool first_round) { take(i, v, first_round ? early_gain[j] : gain[i]); });
     }
     mark(c, io, 1);
+    signal_received(c.ctl);
     signal_staged(c.ctl);
     ss = io_sum(c.ctl, io, ss);
     ss /= c.b.dim_as_float;  // n, converted on the host: here the conversion's result would be kept in (and spilled from) a vector register
@@ -871,7 +898,10 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
             }
         }
     }
-    if (first_item) mark(c, io, 5);
+    if (first_item) {
+        mark(c, io, 5);
+        signal_received(c.ctl);
+    }
     io_sync(c.ctl, io);
     if (first_item) {
         mark(c, io, 1);
@@ -1056,6 +1086,17 @@ __host__ __device__ inline int item_splits(int npos, int cap, int n_heads, int n
     return best;
 }
 
+// A workgroup without an attention item still tells its streaming wavefronts when this token's
+// q, k and v are out (one value stands for all: they are published within a microsecond of one
+// another), so that what those held back goes out while the items are computed, not before.
+__device__ __forceinline__ void idle_attention_received(Ctx& c, const Io& io, int layer) {
+    float unused[1];
+    const u64* one = c.t.q + (c.wg % c.a.dim);
+    poll_n<1>([&](int) -> const u64* { return one; }, unused, c.seq(layer, kQkv), c);
+    (void)io;
+    signal_received(c.ctl);
+}
+
 // Splits for items that cover several heads: as item_splits, with an item's length counted in
 // whole passes of `sub_positions` positions (what one trip round its loop handles).
 __host__ __device__ inline int group_item_splits(int npos, int cap, int n_chunks, int nwg, int sub_positions) {
@@ -1099,6 +1140,7 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
             else att_group_item<16, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
             first = false;
         }
+        if (first) idle_attention_received(c, io, layer);
         if (nsplits > 1) {
             // the heads of a chunk are combined by the workgroups that held its first splits
             for (int item = c.wg; item < items; item += c.nwg) {
@@ -1124,6 +1166,7 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
         else att_group_item<16, 1>(c, io, l, layer, h, split, nsplits, npos, first, hs);
         first = false;
     }
+    if (first) idle_attention_received(c, io, layer);
     if (nsplits > 1) {
         for (int item = c.wg; item < items; item += c.nwg) {
             const int h = item / nsplits, split = item - h * nsplits;
