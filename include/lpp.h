@@ -330,6 +330,34 @@ lpp_status lpp_run(lpp_model *m, const int *prompt, int n_prompt, int steps, flo
                    float topp, const float *uniforms, int *out_tokens, int out_capacity,
                    lpp_run_result *res);
 
+/* Batched prefill.  The reference has none: main.cpp:163-180 prefills by
+ * decoding the prompt token by token and dropping what the sampler returns).  Writes
+ * the key/value cache entries of tokens[0 .. n_tokens) at positions start_pos ..
+ * start_pos + n_tokens - 1, all layers, exactly what those decode steps leave behind
+ * for later steps to read (K and V rounded to binary16, model.cpp:171-176); no logits,
+ * no sampling.  The prompt goes through each layer as one batch of up to 512 tokens:
+ * GEMMs on the matrix cores, every weight read once per batch.  Needs binary16
+ * weights, dim / kv_dim / hidden_dim multiples of 128, head_size 64 or 128, at most 8
+ * query heads per KV head: lpp_prefill_supported says whether the model qualifies
+ * (LPP_ERR_UNSUPPORTED and the reason in lpp_last_error otherwise).  `tokens` is host
+ * memory.  Synchronous. */
+lpp_status lpp_prefill_supported(const lpp_model *m);
+lpp_status lpp_prefill(lpp_model *m, const int *tokens, int n_tokens, int start_pos);
+/* lpp_run with the prompt (all ids but the last) prefilled by lpp_prefill instead of
+ * by decode steps; everything else, the uniforms' indexing by position included, as
+ * lpp_run.  Falls back to lpp_run's own prefill when the model does not qualify. */
+lpp_status lpp_run_batched_prefill(lpp_model *m, const int *prompt, int n_prompt, int steps, float temperature,
+                                   float topp, const float *uniforms, int *out_tokens, int out_capacity,
+                                   lpp_run_result *res);
+/* The prefill's GEMM on its own (no counterpart in the reference, whose products are
+ * all matrix-vector): y[t][f] (+)= sum_j w[f][j] * x[t][j] for t < n_tokens, f < n;
+ * w binary16 [n][k] row-major as the weight matrices are stored, x fp32 [n_tokens][k],
+ * y fp32 [n_tokens][n]; device pointers.  x is split into a binary16 head and
+ * remainder, both multiplied into fp32 accumulators (v_mfma_f32_32x32x16_f16).
+ * n and n_tokens multiples of 128, k a multiple of 32. */
+lpp_status lpp_prefill_gemm(float *d_y, const void *d_w, const float *d_x, int n, int k, int n_tokens,
+                            int accumulate);
+
 /* Per-kernel timing of the fused path, measured with HIP events on the launch
  * stream: each kernel class is recorded n_layers times (one launch per layer,
  * so every launch streams different weights) into a graph that is replayed

@@ -107,6 +107,10 @@ SIGNATURES = {
     "lpp_checkpoint_tensor": (_i, [_vp, _i, C.POINTER(_vp), C.POINTER(_sz)]),
     "lpp_model_load_checkpoint": (_i, [C.POINTER(_vp), _vp]),
     "lpp_run": (_i, [_vp, _vp, _i, _i, _f, _f, _vp, _vp, _i, C.POINTER(LppRunResult)]),
+    "lpp_run_batched_prefill": (_i, [_vp, _vp, _i, _i, _f, _f, _vp, _vp, _i, C.POINTER(LppRunResult)]),
+    "lpp_prefill_supported": (_i, [_vp]),
+    "lpp_prefill": (_i, [_vp, _vp, _i, _i]),
+    "lpp_prefill_gemm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "lpp_gguf_open": (_i, [C.POINTER(_vp), C.c_char_p]),
     "lpp_gguf_close": (_i, [_vp]),
     "lpp_gguf_config": (_i, [_vp, C.POINTER(LppConfig)]),

@@ -147,8 +147,27 @@ lpp_status lpp_model_load_checkpoint(lpp_model** out, const lpp_checkpoint* ck) 
     return LPP_OK;
 }
 
+namespace {
+lpp_status run_loop(lpp_model* m, const int* prompt, int n_prompt, int steps, float temperature, float topp,
+                    const float* uniforms, int* out_tokens, int out_capacity, lpp_run_result* res, bool batched);
+}
+
 lpp_status lpp_run(lpp_model* m, const int* prompt, int n_prompt, int steps, float temperature, float topp,
                    const float* uniforms, int* out_tokens, int out_capacity, lpp_run_result* res) {
+    return run_loop(m, prompt, n_prompt, steps, temperature, topp, uniforms, out_tokens, out_capacity, res, false);
+}
+
+lpp_status lpp_run_batched_prefill(lpp_model* m, const int* prompt, int n_prompt, int steps, float temperature, float topp,
+                                   const float* uniforms, int* out_tokens, int out_capacity, lpp_run_result* res) {
+    return run_loop(m, prompt, n_prompt, steps, temperature, topp, uniforms, out_tokens, out_capacity, res, true);
+}
+
+}  // extern "C"
+
+namespace {
+
+lpp_status run_loop(lpp_model* m, const int* prompt, int n_prompt, int steps, float temperature, float topp,
+                    const float* uniforms, int* out_tokens, int out_capacity, lpp_run_result* res, bool batched) {
     LPP_REQUIRE(m != nullptr, "lpp_run: null model");
     LPP_REQUIRE(out_capacity >= 0 && (out_capacity == 0 || out_tokens != nullptr), "lpp_run: output capacity %d", out_capacity);
     LPP_REQUIRE(temperature == 0.0f || uniforms != nullptr, "lpp_run: uniforms required when temperature != 0");
@@ -177,8 +196,15 @@ lpp_status lpp_run(lpp_model* m, const int* prompt, int n_prompt, int steps, flo
     };
     int pos = 0;
     int n_out = 0;
-    // 1. prefill by decode, main.cpp:163-180: penalty 1.1, the sampled id is dropped
-    for (int i = 0; i < n_prompt - 1; ++i) {
+    // 1. prefill, main.cpp:163-180.  Batched: the cache entries of all but the last prompt id in one
+    //    pass per 512 ids; what the decode steps would have sampled is what the reference drops.
+    if (batched && n_prompt > 1 && lpp_prefill_supported(m) == LPP_OK) {
+        for (int i = 0; i < n_prompt - 1; ++i) push(prompt[i]);
+        LPP_TRY(lpp_prefill(m, prompt, n_prompt - 1, 0));
+        pos = n_prompt - 1;
+    }
+    //    By decode: penalty 1.1, the sampled id is dropped
+    for (int i = pos; i < n_prompt - 1; ++i) {
         push(prompt[i]);
         int ignored = 0;
         LPP_TRY(lpp_forward(m, prompt[i], pos, temperature, topp, 1.1f, history, history_len, uniforms ? uniforms[pos] : 0.0f,
@@ -217,4 +243,4 @@ lpp_status lpp_run(lpp_model* m, const int* prompt, int n_prompt, int steps, flo
     return LPP_OK;
 }
 
-}  // extern "C"
+}  // namespace

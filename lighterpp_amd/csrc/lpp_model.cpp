@@ -135,6 +135,7 @@ lpp_status lpp_model_destroy(lpp_model* m) {
     if (!m) return LPP_OK;
     (void)hipStreamSynchronize(lpp::stream());
     lpp::fused_release(m);
+    lpp::prefill_release(m);
     for (int t = 0; t < LPP_T_COUNT; ++t) lpp_free(m->w[t]);
     lpp_free(m->x); lpp_free(m->xb); lpp_free(m->xb2); lpp_free(m->hb); lpp_free(m->he);
     lpp_free(m->q); lpp_free(m->k); lpp_free(m->v); lpp_free(m->att); lpp_free(m->logits);

@@ -70,6 +70,9 @@ struct lpp_model {
     bool fused_ok = false;                   // shape supported by the fused kernels
     char fused_why[160] = "";
 
+    void* pf_buf[12] = {};                   // batched prefill: activations of a chunk of tokens (prefill.hip)
+    int pf_cap = 0;                          // tokens those buffers hold
+
     hipGraphExec_t graph_exec[2] = {nullptr, nullptr};  // [0] without, [1] with uniforms/out arrays
     hipEvent_t ev_a = nullptr, ev_b = nullptr;
 };
@@ -94,6 +97,9 @@ struct StepParams {
 };
 
 size_t tensor_bytes(const lpp_config& c, int tensor);
+
+// Implemented in prefill.hip: frees the batched prefill's buffers.
+void prefill_release(lpp_model* m);
 
 // Implemented in fused_decode.hip.
 lpp_status fused_prepare(lpp_model* m);

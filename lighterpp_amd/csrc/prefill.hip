@@ -1,0 +1,519 @@
+// prefill.hip -- batched prefill: the key/value cache entries of a run of prompt
+// tokens in one pass over the weights.
+//
+// The reference has no such path: it prefills by decoding the prompt one token at
+// a time and dropping what the sampler returns (src/main.cpp:163-180), which reads
+// every weight once per prompt token.  Here the prompt's tokens go through each
+// layer together, so the matrix products are GEMMs on the matrix cores
+// (v_mfma_f32_32x32x16_f16) and every weight is read once per chunk of up to 512
+// tokens.  What a prefill leaves behind is exactly what the decode loop reads
+// later: K and V of the prompt positions, rounded to binary16 as the cache store
+// rounds them (model.cpp:171-176, kernels.cuh:34).  The classifier and the sampler
+// are not run: the ids they would produce are the ones main.cpp drops.
+//
+// Arithmetic: weights binary16 as stored; activations fp32, split for the matrix
+// cores into a binary16 head and a binary16 remainder (x = hi + lo to about 2^-22),
+// both multiplied into the same fp32 accumulators; everything between the GEMMs
+// (RMSNorm, RoPE, softmax, SwiGLU, residual) in fp32 with the operators' own
+// operation order (ops.cpp:20-87).
+#include <cmath>
+
+#include "lpp_device.hpp"
+#include "lpp_internal.hpp"
+#include "lpp_model.hpp"
+
+namespace lpp {
+namespace pf {
+
+using namespace dev;
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kTileTokens = 128;    // token rows of a workgroup's output tile
+constexpr int kTileFeatures = 128;  // weight rows of it
+constexpr int kChunk = 512;         // prompt tokens per pass over the weights
+constexpr int kMaxGqa = 8;          // query heads per KV head the attention kernel keeps in registers
+
+// ---------------------------------------------------------------------------
+// Small per-token kernels
+// ---------------------------------------------------------------------------
+
+// x[t][:] = embedding row of tokens[t] (model.cpp:346-348).
+__global__ __launch_bounds__(256) void k_embed(const float* __restrict__ emb, const int* __restrict__ tokens,
+                                               float* __restrict__ x, int dim) {
+    const int t = blockIdx.x;
+    const float* src = emb + static_cast<size_t>(tokens[t]) * dim;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) x[static_cast<size_t>(t) * dim + i] = src[i];
+}
+
+__device__ __forceinline__ float block_sum256(float v, float* scratch) {
+    v = wave_sum(v);
+    if (lane_id() == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    const float total = (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+    __syncthreads();
+    return total;
+}
+
+__device__ __forceinline__ void split_store(half_t* hi, half_t* lo, size_t at, float v) {
+    const half_t h = static_cast<half_t>(v);
+    hi[at] = h;
+    lo[at] = static_cast<half_t>(v - static_cast<float>(h));
+}
+
+// (hi, lo)[t][:] = RMSNorm(x[t][:]) * gain (ops.cpp:20-32); rows t >= n_tokens are zero.
+__global__ __launch_bounds__(256) void k_norm_split(const float* __restrict__ x, const float* __restrict__ gain,
+                                                    half_t* __restrict__ hi, half_t* __restrict__ lo, int dim,
+                                                    int n_tokens) {
+#pragma clang fp contract(off)
+    __shared__ float scratch[4];
+    const int t = blockIdx.x;
+    const size_t row = static_cast<size_t>(t) * dim;
+    if (t >= n_tokens) {
+        for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+            hi[row + i] = static_cast<half_t>(0.0f);
+            lo[row + i] = static_cast<half_t>(0.0f);
+        }
+        return;
+    }
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        const float v = x[row + i];
+        ss += v * v;
+    }
+    ss = block_sum256(ss, scratch);
+    ss /= static_cast<float>(dim);
+    ss += 1e-5f;
+    const float scale = 1.0f / sqrtf(ss);
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) split_store(hi, lo, row + i, x[row + i] * scale * gain[i]);
+}
+
+// RoPE on q and k of token t (ops.cpp:34-54), q kept in fp32, k and v written to the
+// caches as binary16 at position pos0 + t (model.cpp:171-176).
+__global__ __launch_bounds__(256) void k_rope_scatter(float* __restrict__ q, const float* __restrict__ k,
+                                                      const float* __restrict__ v, const float2* __restrict__ rope,
+                                                      uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache,
+                                                      int layer, int pos0, int dim, int kv_dim, int hs, int seq_len) {
+#pragma clang fp contract(off)
+    const int t = blockIdx.x;
+    const int pos = pos0 + t;
+    const float2* cs_row = rope + static_cast<size_t>(pos) * (hs / 2);
+    for (int i = 2 * threadIdx.x; i < dim; i += 2 * blockDim.x) {
+        float* p = q + static_cast<size_t>(t) * dim + i;
+        const float2 cs = cs_row[(i % hs) >> 1];
+        const float q0 = p[0], q1 = p[1];
+        p[0] = q0 * cs.x - q1 * cs.y;
+        p[1] = q0 * cs.y + q1 * cs.x;
+    }
+    for (int i = 2 * threadIdx.x; i < kv_dim; i += 2 * blockDim.x) {
+        const float* pk = k + static_cast<size_t>(t) * kv_dim + i;
+        const float* pv = v + static_cast<size_t>(t) * kv_dim + i;
+        const float2 cs = cs_row[(i % hs) >> 1];
+        const float k0 = pk[0], k1 = pk[1];
+        const int head = i / hs, within = i - head * hs;
+        const size_t dst = static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(head) * seq_len * hs +
+                           static_cast<size_t>(pos) * hs + within;
+        key_cache[dst] = f32_to_f16_bits(k0 * cs.x - k1 * cs.y);
+        key_cache[dst + 1] = f32_to_f16_bits(k0 * cs.y + k1 * cs.x);
+        value_cache[dst] = f32_to_f16_bits(pv[0]);
+        value_cache[dst + 1] = f32_to_f16_bits(pv[1]);
+    }
+}
+
+// (hi, lo)[t][u] = (g * sigmoid(g)) * up (ops.cpp:78-87); rows t >= n_tokens are zero.
+__global__ __launch_bounds__(256) void k_swiglu_split(const float* __restrict__ gate, const float* __restrict__ up,
+                                                      half_t* __restrict__ hi, half_t* __restrict__ lo, int hidden,
+                                                      int n_tokens) {
+#pragma clang fp contract(off)
+    const int t = blockIdx.y;
+    const int u = blockIdx.x * blockDim.x + threadIdx.x;
+    if (u >= hidden) return;
+    const size_t at = static_cast<size_t>(t) * hidden + u;
+    float out = 0.0f;
+    if (t < n_tokens) {
+        const float g = gate[at];
+        const float sigma = 1.0f / (1.0f + expf(-g));
+        out = (g * sigma) * up[at];
+    }
+    split_store(hi, lo, at, out);
+}
+
+// ---------------------------------------------------------------------------
+// GEMM on the matrix cores: Y[t][f] (+)= sum_k W[f][k] * (Xh[t][k] + Xl[t][k])
+// ---------------------------------------------------------------------------
+//
+// W is [n][K] binary16 row-major (a weight matrix as stored), Xh/Xl are [T][K]
+// binary16 row-major, Y is [T][ldy] fp32.  n % 128 == 0, T % 128 == 0, K % 32 == 0.
+// A workgroup of four wavefronts owns a 128-feature x 128-token tile; each wavefront
+// a 64 x 64 quarter = 2 x 2 MFMA tiles of 32 x 32.  Both operands have k as their
+// contiguous dimension, so a lane reads its 8 k-values of a fragment row as one
+// 16-byte load (the two halves of the wavefront take the two halves of a 16-wide
+// k-step); the weight fragment is the A operand, the activations the B operand, and
+// a lane ends up holding, for ONE token, 4 runs of 4 consecutive features per tile.
+template <bool kAccumulate>
+__global__ __launch_bounds__(256) void k_gemm(const half_t* __restrict__ w, const half_t* __restrict__ xh,
+                                              const half_t* __restrict__ xl, float* __restrict__ y, int K, int ldy) {
+    const int lane = lane_id();
+    const int wave = wave_index();
+    const int f0 = blockIdx.x * kTileFeatures + (wave & 1) * 64;
+    const int t0 = blockIdx.y * kTileTokens + (wave >> 1) * 64;
+    const int r = lane & 31, g = lane >> 5;
+    const half_t* wrow[2];
+    const half_t* hrow[2];
+    const half_t* lrow[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        wrow[i] = w + static_cast<size_t>(f0 + 32 * i + r) * K + 8 * g;
+        hrow[i] = xh + static_cast<size_t>(t0 + 32 * i + r) * K + 8 * g;
+        lrow[i] = xl + static_cast<size_t>(t0 + 32 * i + r) * K + 8 * g;
+    }
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    // two k-steps per trip: a lane's two 16-byte pieces of a row are 32 bytes apart, and a row's
+    // 128-byte line is used up in two trips while it is still in the cache
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        half8_t a[2][2], bh[2][2], bl[2][2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                a[s][i] = *reinterpret_cast<const half8_t*>(wrow[i] + k0 + 16 * s);
+                bh[s][i] = *reinterpret_cast<const half8_t*>(hrow[i] + k0 + 16 * s);
+                bl[s][i] = *reinterpret_cast<const half8_t*>(lrow[i] + k0 + 16 * s);
+            }
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s][i], bh[s][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s][i], bl[s][j], acc[i][j], 0, 0, 0);
+                }
+    }
+    // D[m][n]: lane holds column n = lane % 32 (a token) and rows m = 8 * (e / 4) + 4 * (lane / 32) + e % 4 (features)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float* row = y + static_cast<size_t>(t0 + 32 * j + r) * ldy + f0 + 32 * i + 4 * g;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                floatx4* dst = reinterpret_cast<floatx4*>(row + 8 * e4);
+                floatx4 v = floatx4{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                if constexpr (kAccumulate) {
+                    const floatx4 old = *dst;
+                    v = floatx4{old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
+                }
+                *dst = v;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
+// Causal attention over the cache
+// ---------------------------------------------------------------------------
+//
+// One workgroup per (token t, KV head): its query heads (gqa of them) attend to
+// cache positions 0 .. pos0 + t (model.cpp:178-198; every row of the cache for these
+// positions is in place, this chunk's included).  kGroup lanes share a position,
+// 8 binary16 each; every lane group keeps a running maximum, sum and weighted V sum
+// per query head (rescaled when the maximum grows), and the groups, then the four
+// wavefronts, are merged by the same rule.  Output: the heads' outputs, split into
+// (hi, lo) for the output projection's GEMM.
+template <int kGroup>
+__global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, const uint16_t* __restrict__ key_cache,
+                                                   const uint16_t* __restrict__ value_cache, half_t* __restrict__ out_hi,
+                                                   half_t* __restrict__ out_lo, int layer, int pos0, int dim, int kv_dim,
+                                                   int hs, int gqa, int seq_len) {
+    constexpr int kGroups = kWave / kGroup;  // positions a wavefront covers per pass
+    constexpr int kWaves = 4;
+    __shared__ float red[kWaves][kMaxGqa][8 * kGroup + 2];
+    const int t = blockIdx.x, kvh = blockIdx.y;
+    const int npos = pos0 + t + 1;
+    const int lane = lane_id(), wave = wave_index();
+    const int sub = lane % kGroup, grp = lane / kGroup;
+    const bool lane_live = sub * 8 < hs;
+    const int off = lane_live ? sub * 8 : 0;
+    const size_t head_base = static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * hs;
+    const uint16_t* kbase = key_cache + head_base;
+    const uint16_t* vbase = value_cache + head_base;
+    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
+
+    float qreg[kMaxGqa][8];
+    float top[kMaxGqa], lsum[kMaxGqa], acc[kMaxGqa][8];
+#pragma unroll
+    for (int h = 0; h < kMaxGqa; ++h) {
+        top[h] = -INFINITY;
+        lsum[h] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            acc[h][e] = 0.0f;
+            qreg[h][e] = (h < gqa && lane_live) ? q[static_cast<size_t>(t) * dim + (kvh * gqa + h) * hs + off + e] : 0.0f;
+        }
+    }
+    for (int p = wave * kGroups + grp; p < npos; p += kWaves * kGroups) {
+        const half8_t kh = as_half8(load16(kbase + static_cast<size_t>(p) * hs + off));
+        const half8_t vh = as_half8(load16(vbase + static_cast<size_t>(p) * hs + off));
+#pragma unroll
+        for (int h = 0; h < kMaxGqa; ++h) {
+            if (h < gqa) {
+                float s = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s = fmaf(static_cast<float>(kh[e]), qreg[h][e], s);
+                s = lane_live ? s : 0.0f;
+#pragma unroll
+                for (int o = 1; o < kGroup; o <<= 1) s += __shfl_xor(s, o);
+                s *= scale;
+                const float grown = fmaxf(top[h], s);
+                const float corr = (top[h] == -INFINITY) ? 0.0f : expf(top[h] - grown);
+                const float pw = expf(s - grown);
+                top[h] = grown;
+                lsum[h] = lsum[h] * corr + pw;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(static_cast<float>(vh[e]), pw, acc[h][e] * corr);
+            }
+        }
+    }
+    // lane groups of a wavefront
+#pragma unroll
+    for (int h = 0; h < kMaxGqa; ++h) {
+        if (h < gqa) {
+            float all = top[h];
+#pragma unroll
+            for (int o = kGroup; o < kWave; o <<= 1) all = fmaxf(all, __shfl_xor(all, o));
+            const float f = (top[h] == -INFINITY) ? 0.0f : expf(top[h] - all);
+            float ls = lsum[h] * f;
+#pragma unroll
+            for (int o = kGroup; o < kWave; o <<= 1) ls += __shfl_xor(ls, o);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float v = acc[h][e] * f;
+#pragma unroll
+                for (int o = kGroup; o < kWave; o <<= 1) v += __shfl_xor(v, o);
+                acc[h][e] = v;
+            }
+            if (grp == 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) red[wave][h][sub * 8 + e] = acc[h][e];
+                if (sub == 0) {
+                    red[wave][h][8 * kGroup] = all;
+                    red[wave][h][8 * kGroup + 1] = ls;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // the wavefronts: thread (h, e)
+    for (int idx = threadIdx.x; idx < gqa * hs; idx += blockDim.x) {
+        const int h = idx / hs, e = idx - h * hs;
+        float all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) all = fmaxf(all, red[w][h][8 * kGroup]);
+        float o = 0.0f, ls = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float m = red[w][h][8 * kGroup];
+            const float f = (m == -INFINITY) ? 0.0f : expf(m - all);
+            o += red[w][h][e] * f;
+            ls += red[w][h][8 * kGroup + 1] * f;
+        }
+        split_store(out_hi, out_lo, static_cast<size_t>(t) * dim + (kvh * gqa + h) * hs + e, o / ls);
+    }
+}
+
+// (hi, lo) = x as it is (the GEMM entry point's own inputs).
+__global__ __launch_bounds__(256) void k_split(const float* __restrict__ x, half_t* __restrict__ hi, half_t* __restrict__ lo,
+                                               size_t count) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) split_store(hi, lo, i, x[i]);
+}
+
+}  // namespace pf
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+namespace {
+
+// Buffers of a chunk of t_pad tokens, in lpp_model::pf_buf order.
+enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufCount };
+static_assert(kBufCount <= static_cast<int>(sizeof(lpp_model::pf_buf) / sizeof(void*)), "lpp_model::pf_buf is too small");
+
+const char* unsupported_reason(const lpp_model* m) {
+    const lpp_config& c = m->cfg;
+    if (c.weight_precision != LPP_WEIGHT_FP16) return "weights are not binary16";
+    if (c.dim % pf::kTileFeatures != 0 || m->kv_dim % pf::kTileFeatures != 0 || c.hidden_dim % pf::kTileFeatures != 0)
+        return "dim, kv_dim and hidden_dim must be multiples of 128";
+    if (m->head_size != 64 && m->head_size != 128) return "head_size must be 64 or 128";
+    if (m->gqa > pf::kMaxGqa) return "more than 8 query heads per KV head";
+    return nullptr;
+}
+
+lpp_status ensure_scratch(lpp_model* m, int t_pad) {
+    if (m->pf_cap >= t_pad) return LPP_OK;
+    prefill_release(m);
+    const lpp_config& c = m->cfg;
+    const size_t t = static_cast<size_t>(t_pad);
+    const size_t widest = static_cast<size_t>(c.hidden_dim > c.dim ? c.hidden_dim : c.dim);
+    const size_t bytes[kBufCount] = {t * sizeof(int),
+                                     t * c.dim * sizeof(float),
+                                     t * c.dim * sizeof(float),
+                                     t * m->kv_dim * sizeof(float),
+                                     t * m->kv_dim * sizeof(float),
+                                     t * c.hidden_dim * sizeof(float),
+                                     t * c.hidden_dim * sizeof(float),
+                                     t * widest * sizeof(pf::half_t),
+                                     t * widest * sizeof(pf::half_t)};
+    for (int i = 0; i < kBufCount; ++i) {
+        lpp_status st = lpp_malloc(&m->pf_buf[i], bytes[i]);
+        if (st != LPP_OK) {
+            prefill_release(m);
+            return st;
+        }
+    }
+    m->pf_cap = t_pad;
+    return LPP_OK;
+}
+
+lpp_status gemm(const void* w, const pf::half_t* xh, const pf::half_t* xl, float* y, int n, int K, int t_pad, int ldy,
+                bool accumulate, hipStream_t s) {
+    LPP_REQUIRE(n % pf::kTileFeatures == 0 && t_pad % pf::kTileTokens == 0 && K % 32 == 0 && ldy % 4 == 0,
+                "prefill GEMM: shape n %d K %d T %d ldy %d", n, K, t_pad, ldy);
+    const dim3 grid(n / pf::kTileFeatures, t_pad / pf::kTileTokens);
+    if (accumulate)
+        hipLaunchKernelGGL(pf::k_gemm<true>, grid, dim3(256), 0, s, static_cast<const pf::half_t*>(w), xh, xl, y, K, ldy);
+    else
+        hipLaunchKernelGGL(pf::k_gemm<false>, grid, dim3(256), 0, s, static_cast<const pf::half_t*>(w), xh, xl, y, K, ldy);
+    LPP_CHECK_LAUNCH("k_gemm");
+    return LPP_OK;
+}
+
+// One chunk: tokens[0..n) at positions pos0 .. pos0 + n - 1; n <= kChunk.
+lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
+    const lpp_config& c = m->cfg;
+    const int dim = c.dim, kv = m->kv_dim, hidden = c.hidden_dim, hs = m->head_size;
+    const int t_pad = (n + pf::kTileTokens - 1) / pf::kTileTokens * pf::kTileTokens;
+    LPP_TRY(ensure_scratch(m, t_pad));
+    hipStream_t s = stream();
+    int* d_tokens = static_cast<int*>(m->pf_buf[kBufTokens]);
+    float* x = static_cast<float*>(m->pf_buf[kBufX]);
+    float* q = static_cast<float*>(m->pf_buf[kBufQ]);
+    float* k = static_cast<float*>(m->pf_buf[kBufK]);
+    float* v = static_cast<float*>(m->pf_buf[kBufV]);
+    float* gate = static_cast<float*>(m->pf_buf[kBufGate]);
+    float* up = static_cast<float*>(m->pf_buf[kBufUp]);
+    pf::half_t* hi = static_cast<pf::half_t*>(m->pf_buf[kBufHi]);
+    pf::half_t* lo = static_cast<pf::half_t*>(m->pf_buf[kBufLo]);
+    LPP_HIP(hipMemcpyAsync(d_tokens, tokens, static_cast<size_t>(n) * sizeof(int), hipMemcpyHostToDevice, s));
+    hipLaunchKernelGGL(pf::k_embed, dim3(n), dim3(256), 0, s, static_cast<const float*>(m->w[LPP_T_TOKEN_EMBEDDING]), d_tokens,
+                       x, dim);
+    LPP_CHECK_LAUNCH("k_embed");
+    const size_t wb = sizeof(pf::half_t);
+    auto layer_of = [&](int t, int l, size_t rows, size_t cols) {
+        return static_cast<const char*>(m->w[t]) + static_cast<size_t>(l) * rows * cols * wb;
+    };
+    for (int l = 0; l < c.n_layers; ++l) {
+        // attention block, model.cpp:216-218
+        hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
+                           static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n);
+        LPP_CHECK_LAUNCH("k_norm_split");
+        LPP_TRY(gemm(layer_of(LPP_T_WQ, l, dim, dim), hi, lo, q, dim, dim, t_pad, dim, false, s));
+        LPP_TRY(gemm(layer_of(LPP_T_WK, l, kv, dim), hi, lo, k, kv, dim, t_pad, kv, false, s));
+        LPP_TRY(gemm(layer_of(LPP_T_WV, l, kv, dim), hi, lo, v, kv, dim, t_pad, kv, false, s));
+        hipLaunchKernelGGL(pf::k_rope_scatter, dim3(n), dim3(256), 0, s, q, k, v, m->rope, m->key_cache, m->value_cache, l, pos0,
+                           dim, kv, hs, c.seq_len);
+        LPP_CHECK_LAUNCH("k_rope_scatter");
+        // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
+        if (hs == 64)
+            hipLaunchKernelGGL(pf::k_attention<8>, dim3(n, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache, m->value_cache, hi,
+                               lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len);
+        else
+            hipLaunchKernelGGL(pf::k_attention<16>, dim3(n, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache, m->value_cache, hi,
+                               lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len);
+        LPP_CHECK_LAUNCH("k_attention");
+        LPP_TRY(gemm(layer_of(LPP_T_WO, l, dim, dim), hi, lo, x, dim, dim, t_pad, dim, true, s));
+        // feed-forward block, model.cpp:221-226
+        hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
+                           static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n);
+        LPP_CHECK_LAUNCH("k_norm_split");
+        LPP_TRY(gemm(layer_of(LPP_T_W1, l, hidden, dim), hi, lo, gate, hidden, dim, t_pad, hidden, false, s));
+        LPP_TRY(gemm(layer_of(LPP_T_W3, l, hidden, dim), hi, lo, up, hidden, dim, t_pad, hidden, false, s));
+        hipLaunchKernelGGL(pf::k_swiglu_split, dim3((hidden + 255) / 256, t_pad), dim3(256), 0, s, gate, up, hi, lo, hidden, n);
+        LPP_CHECK_LAUNCH("k_swiglu_split");
+        LPP_TRY(gemm(layer_of(LPP_T_W2, l, dim, hidden), hi, lo, x, dim, hidden, t_pad, dim, true, s));
+    }
+    LPP_HIP(hipStreamSynchronize(s));
+    return LPP_OK;
+}
+
+}  // namespace
+
+void prefill_release(lpp_model* m) {
+    for (void*& p : m->pf_buf) {
+        lpp_free(p);
+        p = nullptr;
+    }
+    m->pf_cap = 0;
+}
+
+}  // namespace lpp
+
+extern "C" {
+
+lpp_status lpp_prefill_supported(const lpp_model* m) {
+    LPP_REQUIRE(m != nullptr, "lpp_prefill_supported: null model");
+    const char* why = lpp::unsupported_reason(m);
+    if (why != nullptr) return lpp::fail(LPP_ERR_UNSUPPORTED, "batched prefill unavailable: %s", why);
+    return LPP_OK;
+}
+
+lpp_status lpp_prefill(lpp_model* m, const int* tokens, int n_tokens, int start_pos) {
+    using namespace lpp;
+    LPP_REQUIRE(m != nullptr && tokens != nullptr, "lpp_prefill: null argument");
+    LPP_REQUIRE(n_tokens >= 0 && start_pos >= 0 && start_pos + n_tokens <= m->cfg.seq_len,
+                "lpp_prefill: positions [%d, %d) outside [0, %d)", start_pos, start_pos + n_tokens, m->cfg.seq_len);
+    for (int i = 0; i < n_tokens; ++i)
+        LPP_REQUIRE(tokens[i] >= 0 && tokens[i] < m->cfg.vocab_size, "lpp_prefill: token %d at %d outside [0, %d)", tokens[i], i,
+                    m->cfg.vocab_size);
+    for (int t = 0; t < LPP_T_COUNT; ++t)
+        if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
+    LPP_TRY(lpp_prefill_supported(m));
+    for (int done = 0; done < n_tokens; done += pf::kChunk) {
+        const int n = n_tokens - done < pf::kChunk ? n_tokens - done : pf::kChunk;
+        LPP_TRY(prefill_chunk(m, tokens + done, n, start_pos + done));
+    }
+    return LPP_OK;
+}
+
+lpp_status lpp_prefill_gemm(float* d_y, const void* d_w, const float* d_x, int n, int k, int n_tokens, int accumulate) {
+    using namespace lpp;
+    LPP_REQUIRE(d_y && d_w && d_x, "lpp_prefill_gemm: null argument");
+    LPP_REQUIRE(n_tokens > 0 && n_tokens % pf::kTileTokens == 0, "lpp_prefill_gemm: n_tokens %d not a positive multiple of %d",
+                n_tokens, pf::kTileTokens);
+    LPP_REQUIRE(n > 0 && n % pf::kTileFeatures == 0 && k > 0 && k % 32 == 0, "lpp_prefill_gemm: n %d k %d", n, k);
+    hipStream_t s = stream();
+    void* hi = nullptr;
+    void* lo = nullptr;
+    const size_t count = static_cast<size_t>(n_tokens) * k;
+    LPP_TRY(lpp_malloc(&hi, count * sizeof(pf::half_t)));
+    lpp_status st = lpp_malloc(&lo, count * sizeof(pf::half_t));
+    if (st == LPP_OK) {
+        hipLaunchKernelGGL(pf::k_split, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s, d_x,
+                           static_cast<pf::half_t*>(hi), static_cast<pf::half_t*>(lo), count);
+        st = gemm(d_w, static_cast<pf::half_t*>(hi), static_cast<pf::half_t*>(lo), d_y, n, k, n_tokens, n, accumulate != 0, s);
+        if (hipStreamSynchronize(s) != hipSuccess && st == LPP_OK) st = fail(LPP_ERR_HIP, "lpp_prefill_gemm: kernel failed");
+    }
+    lpp_free(hi);
+    lpp_free(lo);
+    return st;
+}
+
+}  // extern "C"

@@ -341,8 +341,19 @@ class Model:
                                          C.c_void_p(out.ctypes.data), C.byref(stats)))
         return out, hist[:hlen.value].tolist(), stats
 
-    def run(self, prompt, steps: int, temperature: float = 0.0, topp: float = 1.0, uniforms=None):
-        """lpp_run, the driver loop of src/main.cpp:139-232.  Returns (generated ids, LppRunResult)."""
+    def prefill_supported(self) -> bool:
+        """Whether lpp_prefill (batched prefill on the matrix cores) takes this model."""
+        return self.lib.lpp_prefill_supported(self.handle) == capi.LPP_OK
+
+    def prefill(self, tokens, start_pos: int = 0) -> None:
+        """lpp_prefill: the KV cache entries of `tokens` at positions start_pos.., all layers, in one batch."""
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        capi.check(self.lib.lpp_prefill(self.handle, C.c_void_p(t.ctypes.data), int(t.size), int(start_pos)))
+
+    def run(self, prompt, steps: int, temperature: float = 0.0, topp: float = 1.0, uniforms=None,
+            batched_prefill: bool = False):
+        """lpp_run, the driver loop of src/main.cpp:139-232 (lpp_run_batched_prefill: the prompt in one batch).
+        Returns (generated ids, LppRunResult)."""
         out = np.empty(max(steps, 1), dtype=np.int32)
         pp, pn = None, 0
         if prompt is not None and len(prompt) > 0:
@@ -354,8 +365,9 @@ class Model:
             assert u.size >= steps
             up = C.c_void_p(u.ctypes.data)
         res = capi.LppRunResult()
-        capi.check(self.lib.lpp_run(self.handle, pp, pn, steps, temperature, topp, up, C.c_void_p(out.ctypes.data),
-                                    int(out.size), C.byref(res)))
+        entry = self.lib.lpp_run_batched_prefill if batched_prefill else self.lib.lpp_run
+        capi.check(entry(self.handle, pp, pn, steps, temperature, topp, up, C.c_void_p(out.ctypes.data),
+                         int(out.size), C.byref(res)))
         return out[:res.n_tokens].copy(), res
 
     def profile_kernels(self, pos: int, reps: int = 20) -> list:
