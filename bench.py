@@ -123,6 +123,45 @@ def parity_check(model, shape, weights, first_token, n_steps: int):
                 checker="oracle (CPU restatement, binary16 KV store)")
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def bench_prefill(args, model, shape, name, cus) -> int:
+    """Batched prefill of N ids from position 0 (lpp_prefill): K repetitions after W warm-up ones.
+    A step is one prefill of the whole prompt; the line's value is prompt ids per second."""
+    from lighterpp_amd import capi
+    n = min(args.prefill, shape.seq_len)
+    if not model.prefill_supported():
+        print("bench.py: the batched prefill does not take this model", file=sys.stderr)
+        return 2
+    ids = capi.synth_token_ids(n, SEED + 1, shape.vocab_size)
+    reps = args.steps if args.steps is not None else 10
+    for _ in range(max(args.warmup if args.warmup != 16 else 2, 1)):
+        model.prefill(ids, 0)
+    capi.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        model.prefill(ids, 0)
+    capi.synchronize()
+    sec = (time.perf_counter() - t0) / reps
+    L, dim, kv, hidden = shape.n_layers, shape.dim, shape.kv_dim, shape.hidden_dim
+    gemm_flops = 2.0 * L * (2 * dim * dim + 2 * kv * dim + 3 * hidden * dim) * n
+    att_flops = 4.0 * L * shape.n_heads * shape.head_size * n * (n + 1) / 2
+    tflops = (gemm_flops + att_flops) / sec / 1e12
+    out = dict(metric="batched prefill, prompt ids/s, " + args.config, value=round(n / sec, 1), unit="tok/s", n_gpus=1,
+               steps=reps, warmup=2, ms_per_step=round(sec * 1e3, 3), higher_is_better=True, scaling="weak",
+               vs_baseline=None, dtype="f32 accumulate over f16 weights, activations split hi+lo", data="synthetic",
+               config=dict(workload=args.config, prompt_ids=n, chunk=512),
+               roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
+                             frac=round(tflops / MFMA_F16_PEAK_TFLOPS, 4), traffic=None,
+                             note="algorithmic flops (each product counted once; the kernel issues two MFMAs per "
+                                  "product, for the activation's head and remainder)"),
+               cpu_baseline=None,
+               device=dict(name=name.value.decode(), compute_units=cus.value))
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -133,6 +172,8 @@ def main() -> int:
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time bound of the CPU baseline sample (0 = skip)")
     ap.add_argument("--parity-steps", type=int, default=3)
     ap.add_argument("--profile-reps", type=int, default=20)
+    ap.add_argument("--prefill", type=int, default=0, metavar="N",
+                    help="time the batched prefill of N prompt ids instead of the decode loop (a second, separate line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (batch-1 decode has no multi-GPU path here); "
@@ -163,6 +204,8 @@ def main() -> int:
     log(f"{args.config}: weights resident in HBM after {time.time() - t0:.1f}s "
         f"({shape.matrix_params() / 1e6:.1f} M matrix params)")
     model.set_path(path)
+    if args.prefill > 0:
+        return bench_prefill(args, model, shape, name, cus)
     prompt = capi.synth_token_ids(max(wl["prompt"], 1), SEED + 1, shape.vocab_size)
     uniforms = capi.synth_uniform_f32(max(steps, args.warmup, 1), SEED + 2)
     temperature, penalty, cap = wl["temperature"], wl["penalty"], wl["history_cap"]

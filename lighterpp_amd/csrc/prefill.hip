@@ -144,64 +144,79 @@ __global__ __launch_bounds__(256) void k_swiglu_split(const float* __restrict__ 
 //
 // W is [n][K] binary16 row-major (a weight matrix as stored), Xh/Xl are [T][K]
 // binary16 row-major, Y is [T][ldy] fp32.  n % 128 == 0, T % 128 == 0, K % 32 == 0.
-// A workgroup of four wavefronts owns a 128-feature x 128-token tile; each wavefront
-// a 64 x 64 quarter = 2 x 2 MFMA tiles of 32 x 32.  Both operands have k as their
+// A workgroup of four wavefronts owns a square tile of 128 x 128 (kSub = 2: each wavefront
+// a 64 x 64 quarter = 2 x 2 MFMA tiles of 32 x 32) or of 64 x 64 (kSub = 1) features x tokens;
+// the smaller tile is used when the larger one would leave compute units without a workgroup.  Both operands have k as their
 // contiguous dimension, so a lane reads its 8 k-values of a fragment row as one
 // 16-byte load (the two halves of the wavefront take the two halves of a 16-wide
 // k-step); the weight fragment is the A operand, the activations the B operand, and
 // a lane ends up holding, for ONE token, 4 runs of 4 consecutive features per tile.
-template <bool kAccumulate>
+template <bool kAccumulate, int kSub>
 __global__ __launch_bounds__(256) void k_gemm(const half_t* __restrict__ w, const half_t* __restrict__ xh,
                                               const half_t* __restrict__ xl, float* __restrict__ y, int K, int ldy) {
     const int lane = lane_id();
     const int wave = wave_index();
-    const int f0 = blockIdx.x * kTileFeatures + (wave & 1) * 64;
-    const int t0 = blockIdx.y * kTileTokens + (wave >> 1) * 64;
+    constexpr int kWaveTile = 32 * kSub;  // a wavefront's square of the workgroup's (2 * kWaveTile)^2 tile
+    const int f0 = blockIdx.x * (2 * kWaveTile) + (wave & 1) * kWaveTile;
+    const int t0 = blockIdx.y * (2 * kWaveTile) + (wave >> 1) * kWaveTile;
     const int r = lane & 31, g = lane >> 5;
-    const half_t* wrow[2];
-    const half_t* hrow[2];
-    const half_t* lrow[2];
+    const half_t* wrow[kSub];
+    const half_t* hrow[kSub];
+    const half_t* lrow[kSub];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kSub; ++i) {
         wrow[i] = w + static_cast<size_t>(f0 + 32 * i + r) * K + 8 * g;
         hrow[i] = xh + static_cast<size_t>(t0 + 32 * i + r) * K + 8 * g;
         lrow[i] = xl + static_cast<size_t>(t0 + 32 * i + r) * K + 8 * g;
     }
-    floatx16 acc[2][2];
+    floatx16 acc[kSub][kSub];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kSub; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < kSub; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    // two k-steps per trip: a lane's two 16-byte pieces of a row are 32 bytes apart, and a row's
-    // 128-byte line is used up in two trips while it is still in the cache
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        half8_t a[2][2], bh[2][2], bl[2][2];
+    // Two k-steps (32 columns) per trip: a lane's two 16-byte pieces of a row are 32 bytes apart, and a
+    // row's 128-byte line is used up in two trips while it is still in the cache.  The fragments of the
+    // next trip are requested before this trip's products are issued.
+    struct Frags {
+        half8_t a[2][kSub], bh[2][kSub], bl[2][kSub];
+    };
+    auto fetch = [&](Frags& f, int k0) {
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                a[s][i] = *reinterpret_cast<const half8_t*>(wrow[i] + k0 + 16 * s);
-                bh[s][i] = *reinterpret_cast<const half8_t*>(hrow[i] + k0 + 16 * s);
-                bl[s][i] = *reinterpret_cast<const half8_t*>(lrow[i] + k0 + 16 * s);
+            for (int i = 0; i < kSub; ++i) {
+                f.a[s][i] = *reinterpret_cast<const half8_t*>(wrow[i] + k0 + 16 * s);
+                f.bh[s][i] = *reinterpret_cast<const half8_t*>(hrow[i] + k0 + 16 * s);
+                f.bl[s][i] = *reinterpret_cast<const half8_t*>(lrow[i] + k0 + 16 * s);
             }
+    };
+    auto multiply = [&](const Frags& f) {
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < kSub; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s][i], bh[s][j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s][i], bl[s][j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < kSub; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[s][i], f.bh[s][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[s][i], f.bl[s][j], acc[i][j], 0, 0, 0);
                 }
+    };
+    Frags cur, nxt;
+    fetch(cur, 0);
+    for (int k0 = 32; k0 < K; k0 += 32) {
+        fetch(nxt, k0);
+        multiply(cur);
+        cur = nxt;
     }
+    multiply(cur);
     // D[m][n]: lane holds column n = lane % 32 (a token) and rows m = 8 * (e / 4) + 4 * (lane / 32) + e % 4 (features)
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kSub; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < kSub; ++j) {
             float* row = y + static_cast<size_t>(t0 + 32 * j + r) * ldy + f0 + 32 * i + 4 * g;
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4) {
@@ -258,9 +273,18 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
             qreg[h][e] = (h < gqa && lane_live) ? q[static_cast<size_t>(t) * dim + (kvh * gqa + h) * hs + off + e] : 0.0f;
         }
     }
-    for (int p = wave * kGroups + grp; p < npos; p += kWaves * kGroups) {
-        const half8_t kh = as_half8(load16(kbase + static_cast<size_t>(p) * hs + off));
-        const half8_t vh = as_half8(load16(vbase + static_cast<size_t>(p) * hs + off));
+    // (the rows of the position after this one are requested before this one's arithmetic; past the end
+    // the last valid row is read again and dropped)
+    const int first = wave * kGroups + grp;
+    const int clamp = npos - 1;
+    uintx4 k_next = load16(kbase + static_cast<size_t>(first < npos ? first : clamp) * hs + off);
+    uintx4 v_next = load16(vbase + static_cast<size_t>(first < npos ? first : clamp) * hs + off);
+    for (int p = first; p < npos; p += kWaves * kGroups) {
+        const half8_t kh = as_half8(k_next);
+        const half8_t vh = as_half8(v_next);
+        const int pn = p + kWaves * kGroups;
+        k_next = load16(kbase + static_cast<size_t>(pn < npos ? pn : clamp) * hs + off);
+        v_next = load16(vbase + static_cast<size_t>(pn < npos ? pn : clamp) * hs + off);
 #pragma unroll
         for (int h = 0; h < kMaxGqa; ++h) {
             if (h < gqa) {
@@ -387,11 +411,17 @@ lpp_status gemm(const void* w, const pf::half_t* xh, const pf::half_t* xl, float
                 bool accumulate, hipStream_t s) {
     LPP_REQUIRE(n % pf::kTileFeatures == 0 && t_pad % pf::kTileTokens == 0 && K % 32 == 0 && ldy % 4 == 0,
                 "prefill GEMM: shape n %d K %d T %d ldy %d", n, K, t_pad, ldy);
-    const dim3 grid(n / pf::kTileFeatures, t_pad / pf::kTileTokens);
-    if (accumulate)
-        hipLaunchKernelGGL(pf::k_gemm<true>, grid, dim3(256), 0, s, static_cast<const pf::half_t*>(w), xh, xl, y, K, ldy);
-    else
-        hipLaunchKernelGGL(pf::k_gemm<false>, grid, dim3(256), 0, s, static_cast<const pf::half_t*>(w), xh, xl, y, K, ldy);
+    const pf::half_t* wh = static_cast<const pf::half_t*>(w);
+    const int big = (n / pf::kTileFeatures) * (t_pad / pf::kTileTokens);
+    if (big >= compute_units()) {
+        const dim3 grid(n / pf::kTileFeatures, t_pad / pf::kTileTokens);
+        if (accumulate) hipLaunchKernelGGL((pf::k_gemm<true, 2>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+        else hipLaunchKernelGGL((pf::k_gemm<false, 2>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+    } else {
+        const dim3 grid(n / 64, t_pad / 64);
+        if (accumulate) hipLaunchKernelGGL((pf::k_gemm<true, 1>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+        else hipLaunchKernelGGL((pf::k_gemm<false, 1>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+    }
     LPP_CHECK_LAUNCH("k_gemm");
     return LPP_OK;
 }
