@@ -35,6 +35,8 @@ def main(argv=None) -> int:
     ap.add_argument("--temperature", type=float, default=0.8)
     ap.add_argument("--seed", type=int, default=1, help="seed of the per-step uniform draws")
     ap.add_argument("--path", default="persistent", choices=list(PATHS))
+    ap.add_argument("--batched-prefill", action="store_true",
+                    help="fill the cache for the prompt in one pass per 512 ids (lpp_run_batched_prefill) instead of by decode")
     args = ap.parse_args(argv)
 
     capi.check(capi.load().lpp_init(0))
@@ -64,7 +66,7 @@ def main(argv=None) -> int:
     steps = min(args.steps, c.seq_len)
     uniforms = capi.synth_uniform_f32(steps, args.seed)
     print("\n--- Running Inference ---")
-    tokens, res = model.run(prompt, steps, args.temperature, 1.0, uniforms)
+    tokens, res = model.run(prompt, steps, args.temperature, 1.0, uniforms, batched_prefill=args.batched_prefill)
     if tok is not None:
         shown = list(prompt or [1]) + [int(t) for t in tokens]  # main.cpp:175-176, 191-192, 215-221
         sys.stdout.buffer.write(b"".join(tok.decode(t) for t in shown) + b"\n")
