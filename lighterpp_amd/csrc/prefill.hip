@@ -17,6 +17,7 @@
 // (RMSNorm, RoPE, softmax, SwiGLU, residual) in fp32 with the operators' own
 // operation order (ops.cpp:20-87).
 #include <cmath>
+#include <cstdlib>
 
 #include "lpp_device.hpp"
 #include "lpp_internal.hpp"
@@ -231,6 +232,121 @@ __global__ __launch_bounds__(256) void k_gemm(const half_t* __restrict__ w, cons
         }
 }
 
+// The same product with the operand tiles staged in LDS (K a multiple of 64).  A trip covers 64
+// columns: the workgroup copies its W, Xh and Xl tiles (rows of 128 bytes, 16 bytes per lane and
+// request, eight lanes per row) into registers while it multiplies the trip before out of LDS,
+// then stores them to LDS between two barriers.  Every byte comes from memory once per workgroup
+// (the direct kernel above fetches each fragment once per wavefront that uses it, and waits for
+// it with nothing else to do); rows are padded to 144 bytes in LDS so that the 32 rows of a
+// fragment do not all start in the same bank.
+//
+// One launch can serve up to three weight matrices that share the activations (Wq, Wk, Wv): the
+// feature tiles of the matrices are numbered one after the other along the grid's x.
+struct GemmOutputs {
+    const half_t* w[3];
+    float* y[3];
+    int ldy[3];
+    int first_tile[3];  // first feature tile of matrix i (first_tile[0] = 0); unused entries = INT_MAX
+};
+
+template <bool kAccumulate, int kSub>
+__global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* __restrict__ xh,
+                                                  const half_t* __restrict__ xl, int K) {
+    constexpr int kTile = 64 * kSub;           // rows of each operand tile (features, tokens)
+    const int which = (static_cast<int>(blockIdx.x) >= o3.first_tile[2]) ? 2 : (static_cast<int>(blockIdx.x) >= o3.first_tile[1]) ? 1 : 0;
+    const half_t* __restrict__ w = which == 2 ? o3.w[2] : (which == 1 ? o3.w[1] : o3.w[0]);
+    float* __restrict__ y = which == 2 ? o3.y[2] : (which == 1 ? o3.y[1] : o3.y[0]);
+    const int ldy = which == 2 ? o3.ldy[2] : (which == 1 ? o3.ldy[1] : o3.ldy[0]);
+    const int tile_x = static_cast<int>(blockIdx.x) - (which == 2 ? o3.first_tile[2] : (which == 1 ? o3.first_tile[1] : 0));
+    constexpr int kRowBytes = 144;             // 64 binary16 + 16 bytes of padding
+    constexpr int kChunks = kTile * 8 / 256;   // 16-byte pieces per thread and operand
+    __shared__ __align__(16) char tiles[3][kTile * kRowBytes];
+    const int tid = static_cast<int>(threadIdx.x);
+    const int lane = lane_id();
+    const int wave = wave_index();
+    const int f_base = tile_x * kTile, t_base = blockIdx.y * kTile;
+    const int r = lane & 31, g = lane >> 5;
+    const int wf = (wave & 1) * 32 * kSub, wt = (wave >> 1) * 32 * kSub;
+
+    const char* src[3][kChunks];
+    int dst[kChunks];
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+        const int id = tid + 256 * j, row = id >> 3, c = id & 7;
+        src[0][j] = reinterpret_cast<const char*>(w + static_cast<size_t>(f_base + row) * K) + 16 * c;
+        src[1][j] = reinterpret_cast<const char*>(xh + static_cast<size_t>(t_base + row) * K) + 16 * c;
+        src[2][j] = reinterpret_cast<const char*>(xl + static_cast<size_t>(t_base + row) * K) + 16 * c;
+        dst[j] = row * kRowBytes + 16 * c;
+    }
+    uintx4 stage[3][kChunks];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int o = 0; o < 3; ++o)
+#pragma unroll
+            for (int j = 0; j < kChunks; ++j) stage[o][j] = load16(src[o][j] + 2 * static_cast<size_t>(k0));
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int o = 0; o < 3; ++o)
+#pragma unroll
+            for (int j = 0; j < kChunks; ++j) *reinterpret_cast<uintx4*>(tiles[o] + dst[j]) = stage[o][j];
+    };
+
+    floatx16 acc[kSub][kSub];
+#pragma unroll
+    for (int i = 0; i < kSub; ++i)
+#pragma unroll
+        for (int j = 0; j < kSub; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    fetch(0);
+    commit();
+    __syncthreads();
+    for (int k0 = 0; k0 < K; k0 += 64) {
+        const bool more = k0 + 64 < K;
+        if (more) fetch(k0 + 64);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {  // four k-steps of 16 columns
+            half8_t a[kSub], bh[kSub], bl[kSub];
+#pragma unroll
+            for (int i = 0; i < kSub; ++i) {
+                a[i] = *reinterpret_cast<const half8_t*>(tiles[0] + (wf + 32 * i + r) * kRowBytes + 32 * s + 16 * g);
+                bh[i] = *reinterpret_cast<const half8_t*>(tiles[1] + (wt + 32 * i + r) * kRowBytes + 32 * s + 16 * g);
+                bl[i] = *reinterpret_cast<const half8_t*>(tiles[2] + (wt + 32 * i + r) * kRowBytes + 32 * s + 16 * g);
+            }
+#pragma unroll
+            for (int i = 0; i < kSub; ++i)
+#pragma unroll
+                for (int j = 0; j < kSub; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bh[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bl[j], acc[i][j], 0, 0, 0);
+                }
+        }
+        __syncthreads();  // every wavefront has read this trip's tiles
+        if (more) {
+            commit();
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kSub; ++i)
+#pragma unroll
+        for (int j = 0; j < kSub; ++j) {
+            float* row = y + static_cast<size_t>(t_base + wt + 32 * j + r) * ldy + f_base + wf + 32 * i + 4 * g;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                floatx4* out = reinterpret_cast<floatx4*>(row + 8 * e4);
+                floatx4 v = floatx4{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                if constexpr (kAccumulate) {
+                    const floatx4 old = *out;
+                    v = floatx4{old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
+                }
+                *out = v;
+            }
+        }
+}
+
 // ---------------------------------------------------------------------------
 // Causal attention over the cache
 // ---------------------------------------------------------------------------
@@ -242,6 +358,21 @@ __global__ __launch_bounds__(256) void k_gemm(const half_t* __restrict__ w, cons
 // per query head (rescaled when the maximum grows), and the groups, then the four
 // wavefronts, are merged by the same rule.  Output: the heads' outputs, split into
 // (hi, lo) for the output projection's GEMM.
+// Sum over the kGroup lanes that share a position, by DPP moves (no LDS round trip).
+template <int kGroup>
+__device__ __forceinline__ float lanes_sum(float v) {
+    static_assert(kGroup == 8 || kGroup == 16, "lane groups of 8 or 16");
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    if constexpr (kGroup == 16) v += dpp_move<kDppMirror>(v);
+    return v;
+}
+
+// exp(x) as one hardware exponential (about an ulp off expf; the weights it forms are normalised
+// by their own sum).
+__device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+
 template <int kGroup>
 __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, const uint16_t* __restrict__ key_cache,
                                                    const uint16_t* __restrict__ value_cache, half_t* __restrict__ out_hi,
@@ -292,12 +423,10 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
 #pragma unroll
                 for (int e = 0; e < 8; ++e) s = fmaf(static_cast<float>(kh[e]), qreg[h][e], s);
                 s = lane_live ? s : 0.0f;
-#pragma unroll
-                for (int o = 1; o < kGroup; o <<= 1) s += __shfl_xor(s, o);
-                s *= scale;
+                s = lanes_sum<kGroup>(s) * scale;
                 const float grown = fmaxf(top[h], s);
-                const float corr = (top[h] == -INFINITY) ? 0.0f : expf(top[h] - grown);
-                const float pw = expf(s - grown);
+                const float corr = (top[h] == -INFINITY) ? 0.0f : exp_fast(top[h] - grown);
+                const float pw = exp_fast(s - grown);
                 top[h] = grown;
                 lsum[h] = lsum[h] * corr + pw;
 #pragma unroll
@@ -312,7 +441,7 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
             float all = top[h];
 #pragma unroll
             for (int o = kGroup; o < kWave; o <<= 1) all = fmaxf(all, __shfl_xor(all, o));
-            const float f = (top[h] == -INFINITY) ? 0.0f : expf(top[h] - all);
+            const float f = (top[h] == -INFINITY) ? 0.0f : exp_fast(top[h] - all);
             float ls = lsum[h] * f;
 #pragma unroll
             for (int o = kGroup; o < kWave; o <<= 1) ls += __shfl_xor(ls, o);
@@ -344,7 +473,7 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
             const float m = red[w][h][8 * kGroup];
-            const float f = (m == -INFINITY) ? 0.0f : expf(m - all);
+            const float f = (m == -INFINITY) ? 0.0f : exp_fast(m - all);
             o += red[w][h][e] * f;
             ls += red[w][h][8 * kGroup + 1] * f;
         }
@@ -407,22 +536,62 @@ lpp_status ensure_scratch(lpp_model* m, int t_pad) {
     return LPP_OK;
 }
 
-lpp_status gemm(const void* w, const pf::half_t* xh, const pf::half_t* xl, float* y, int n, int K, int t_pad, int ldy,
-                bool accumulate, hipStream_t s) {
-    LPP_REQUIRE(n % pf::kTileFeatures == 0 && t_pad % pf::kTileTokens == 0 && K % 32 == 0 && ldy % 4 == 0,
-                "prefill GEMM: shape n %d K %d T %d ldy %d", n, K, t_pad, ldy);
-    const pf::half_t* wh = static_cast<const pf::half_t*>(w);
-    const int big = (n / pf::kTileFeatures) * (t_pad / pf::kTileTokens);
-    if (big >= compute_units()) {
-        const dim3 grid(n / pf::kTileFeatures, t_pad / pf::kTileTokens);
-        if (accumulate) hipLaunchKernelGGL((pf::k_gemm<true, 2>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
-        else hipLaunchKernelGGL((pf::k_gemm<false, 2>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
-    } else {
-        const dim3 grid(n / 64, t_pad / 64);
-        if (accumulate) hipLaunchKernelGGL((pf::k_gemm<true, 1>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
-        else hipLaunchKernelGGL((pf::k_gemm<false, 1>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+// Y_i[t][f] (+)= sum_k W_i[f][k] * x[t][k] for up to three matrices W_i of n_i rows that share x.
+struct Product {
+    const void* w;
+    float* y;
+    int n;
+};
+
+lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad, bool accumulate,
+                hipStream_t s) {
+    LPP_REQUIRE(count >= 1 && count <= 3 && t_pad % pf::kTileTokens == 0 && K % 32 == 0, "prefill GEMM: %d products, K %d, T %d",
+                count, K, t_pad);
+    int total_n = 0;
+    for (int i = 0; i < count; ++i) {
+        LPP_REQUIRE(prods[i].n > 0 && prods[i].n % pf::kTileFeatures == 0, "prefill GEMM: n %d", prods[i].n);
+        total_n += prods[i].n;
     }
-    LPP_CHECK_LAUNCH("k_gemm");
+    const bool large_tiles = (total_n / pf::kTileFeatures) * (t_pad / pf::kTileTokens) >= compute_units();
+    const int tile = large_tiles ? pf::kTileFeatures : 64;
+    const bool staged = K % 64 == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr;
+    if (staged) {
+        pf::GemmOutputs o3;
+        int at = 0;
+        for (int i = 0; i < 3; ++i) {
+            const Product& p = prods[i < count ? i : count - 1];
+            o3.w[i] = static_cast<const pf::half_t*>(p.w);
+            o3.y[i] = p.y;
+            o3.ldy[i] = p.n;
+            o3.first_tile[i] = i < count ? at : 0x7fffffff;
+            if (i < count) at += p.n / tile;
+        }
+        const dim3 grid(at, t_pad / tile);
+        if (large_tiles) {
+            if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 2>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            else hipLaunchKernelGGL((pf::k_gemm_lds<false, 2>), grid, dim3(256), 0, s, o3, xh, xl, K);
+        } else {
+            if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 1>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            else hipLaunchKernelGGL((pf::k_gemm_lds<false, 1>), grid, dim3(256), 0, s, o3, xh, xl, K);
+        }
+        LPP_CHECK_LAUNCH("k_gemm_lds");
+        return LPP_OK;
+    }
+    // fragments straight from memory: one launch per matrix
+    for (int i = 0; i < count; ++i) {
+        const pf::half_t* wh = static_cast<const pf::half_t*>(prods[i].w);
+        const dim3 grid(prods[i].n / tile, t_pad / tile);
+        float* y = prods[i].y;
+        const int ldy = prods[i].n;
+        if (large_tiles) {
+            if (accumulate) hipLaunchKernelGGL((pf::k_gemm<true, 2>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+            else hipLaunchKernelGGL((pf::k_gemm<false, 2>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+        } else {
+            if (accumulate) hipLaunchKernelGGL((pf::k_gemm<true, 1>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+            else hipLaunchKernelGGL((pf::k_gemm<false, 1>), grid, dim3(256), 0, s, wh, xh, xl, y, K, ldy);
+        }
+        LPP_CHECK_LAUNCH("k_gemm");
+    }
     return LPP_OK;
 }
 
@@ -455,9 +624,9 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
                            static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n);
         LPP_CHECK_LAUNCH("k_norm_split");
-        LPP_TRY(gemm(layer_of(LPP_T_WQ, l, dim, dim), hi, lo, q, dim, dim, t_pad, dim, false, s));
-        LPP_TRY(gemm(layer_of(LPP_T_WK, l, kv, dim), hi, lo, k, kv, dim, t_pad, kv, false, s));
-        LPP_TRY(gemm(layer_of(LPP_T_WV, l, kv, dim), hi, lo, v, kv, dim, t_pad, kv, false, s));
+        const Product qkv[3] = {{layer_of(LPP_T_WQ, l, dim, dim), q, dim}, {layer_of(LPP_T_WK, l, kv, dim), k, kv},
+                                {layer_of(LPP_T_WV, l, kv, dim), v, kv}};
+        LPP_TRY(gemm(qkv, 3, hi, lo, dim, t_pad, false, s));
         hipLaunchKernelGGL(pf::k_rope_scatter, dim3(n), dim3(256), 0, s, q, k, v, m->rope, m->key_cache, m->value_cache, l, pos0,
                            dim, kv, hs, c.seq_len);
         LPP_CHECK_LAUNCH("k_rope_scatter");
@@ -469,16 +638,18 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
             hipLaunchKernelGGL(pf::k_attention<16>, dim3(n, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache, m->value_cache, hi,
                                lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len);
         LPP_CHECK_LAUNCH("k_attention");
-        LPP_TRY(gemm(layer_of(LPP_T_WO, l, dim, dim), hi, lo, x, dim, dim, t_pad, dim, true, s));
+        const Product wo = {layer_of(LPP_T_WO, l, dim, dim), x, dim};
+        LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s));
         // feed-forward block, model.cpp:221-226
         hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
                            static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n);
         LPP_CHECK_LAUNCH("k_norm_split");
-        LPP_TRY(gemm(layer_of(LPP_T_W1, l, hidden, dim), hi, lo, gate, hidden, dim, t_pad, hidden, false, s));
-        LPP_TRY(gemm(layer_of(LPP_T_W3, l, hidden, dim), hi, lo, up, hidden, dim, t_pad, hidden, false, s));
+        const Product gate_up[2] = {{layer_of(LPP_T_W1, l, hidden, dim), gate, hidden}, {layer_of(LPP_T_W3, l, hidden, dim), up, hidden}};
+        LPP_TRY(gemm(gate_up, 2, hi, lo, dim, t_pad, false, s));
         hipLaunchKernelGGL(pf::k_swiglu_split, dim3((hidden + 255) / 256, t_pad), dim3(256), 0, s, gate, up, hi, lo, hidden, n);
         LPP_CHECK_LAUNCH("k_swiglu_split");
-        LPP_TRY(gemm(layer_of(LPP_T_W2, l, dim, hidden), hi, lo, x, dim, hidden, t_pad, dim, true, s));
+        const Product w2 = {layer_of(LPP_T_W2, l, dim, hidden), x, dim};
+        LPP_TRY(gemm(&w2, 1, hi, lo, hidden, t_pad, true, s));
     }
     LPP_HIP(hipStreamSynchronize(s));
     return LPP_OK;
@@ -538,7 +709,8 @@ lpp_status lpp_prefill_gemm(float* d_y, const void* d_w, const float* d_x, int n
     if (st == LPP_OK) {
         hipLaunchKernelGGL(pf::k_split, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s, d_x,
                            static_cast<pf::half_t*>(hi), static_cast<pf::half_t*>(lo), count);
-        st = gemm(d_w, static_cast<pf::half_t*>(hi), static_cast<pf::half_t*>(lo), d_y, n, k, n_tokens, n, accumulate != 0, s);
+        const Product one = {d_w, d_y, n};
+        st = gemm(&one, 1, static_cast<pf::half_t*>(hi), static_cast<pf::half_t*>(lo), k, n_tokens, accumulate != 0, s);
         if (hipStreamSynchronize(s) != hipSuccess && st == LPP_OK) st = fail(LPP_ERR_HIP, "lpp_prefill_gemm: kernel failed");
     }
     lpp_free(hi);
