@@ -247,6 +247,10 @@ struct GemmOutputs {
     float* y[3];
     int ldy[3];
     int first_tile[3];  // first feature tile of matrix i (first_tile[0] = 0); unused entries = INT_MAX
+    // Split K: workgroup z of the grid multiplies columns [z * k_len, (z + 1) * k_len) and writes its
+    // partial product to y + z * split_stride (rows of K_total columns in w and x; k_len of them used).
+    int k_len;
+    size_t split_stride;
 };
 
 template <bool kAccumulate, int kSub>
@@ -258,6 +262,8 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
     float* __restrict__ y = which == 2 ? o3.y[2] : (which == 1 ? o3.y[1] : o3.y[0]);
     const int ldy = which == 2 ? o3.ldy[2] : (which == 1 ? o3.ldy[1] : o3.ldy[0]);
     const int tile_x = static_cast<int>(blockIdx.x) - (which == 2 ? o3.first_tile[2] : (which == 1 ? o3.first_tile[1] : 0));
+    const int k_first = static_cast<int>(blockIdx.z) * o3.k_len;  // K below is the row length; this workgroup covers k_len columns
+    y += static_cast<size_t>(blockIdx.z) * o3.split_stride;
     constexpr int kRowBytes = 144;             // 64 binary16 + 16 bytes of padding
     constexpr int kChunks = kTile * 8 / 256;   // 16-byte pieces per thread and operand
     __shared__ __align__(16) char tiles[3][kTile * kRowBytes];
@@ -273,9 +279,9 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
         const int id = tid + 256 * j, row = id >> 3, c = id & 7;
-        src[0][j] = reinterpret_cast<const char*>(w + static_cast<size_t>(f_base + row) * K) + 16 * c;
-        src[1][j] = reinterpret_cast<const char*>(xh + static_cast<size_t>(t_base + row) * K) + 16 * c;
-        src[2][j] = reinterpret_cast<const char*>(xl + static_cast<size_t>(t_base + row) * K) + 16 * c;
+        src[0][j] = reinterpret_cast<const char*>(w + static_cast<size_t>(f_base + row) * K + k_first) + 16 * c;
+        src[1][j] = reinterpret_cast<const char*>(xh + static_cast<size_t>(t_base + row) * K + k_first) + 16 * c;
+        src[2][j] = reinterpret_cast<const char*>(xl + static_cast<size_t>(t_base + row) * K + k_first) + 16 * c;
         dst[j] = row * kRowBytes + 16 * c;
     }
     uintx4 stage[3][kChunks];
@@ -303,8 +309,8 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
     fetch(0);
     commit();
     __syncthreads();
-    for (int k0 = 0; k0 < K; k0 += 64) {
-        const bool more = k0 + 64 < K;
+    for (int k0 = 0; k0 < o3.k_len; k0 += 64) {
+        const bool more = k0 + 64 < o3.k_len;
         if (more) fetch(k0 + 64);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {  // four k-steps of 16 columns
@@ -481,6 +487,19 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
     }
 }
 
+// x[i] += p[0][i] + p[1][i] + ... in that order: the partial products of a GEMM whose K was split.
+__global__ __launch_bounds__(256) void k_add_partials(float* __restrict__ x, const float* __restrict__ p, int splits,
+                                                      size_t stride, size_t count) {
+    const size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (i >= count) return;
+    floatx4 v = *reinterpret_cast<const floatx4*>(x + i);
+    for (int s = 0; s < splits; ++s) {
+        const floatx4 a = *reinterpret_cast<const floatx4*>(p + s * stride + i);
+        v = floatx4{v[0] + a[0], v[1] + a[1], v[2] + a[2], v[3] + a[3]};
+    }
+    *reinterpret_cast<floatx4*>(x + i) = v;
+}
+
 // (hi, lo) = x as it is (the GEMM entry point's own inputs).
 __global__ __launch_bounds__(256) void k_split(const float* __restrict__ x, half_t* __restrict__ hi, half_t* __restrict__ lo,
                                                size_t count) {
@@ -543,8 +562,11 @@ struct Product {
     int n;
 };
 
+// `partials` (optional, partial_floats long): room for the partial products of a split K.  A long K
+// with few output tiles (the down projection: 8192 columns, 2048 rows) is cut into up to four
+// ranges, each multiplied by its own workgroups into `partials`, and added to y in a fixed order.
 lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad, bool accumulate,
-                hipStream_t s) {
+                hipStream_t s, float* partials = nullptr, size_t partial_floats = 0) {
     LPP_REQUIRE(count >= 1 && count <= 3 && t_pad % pf::kTileTokens == 0 && K % 32 == 0, "prefill GEMM: %d products, K %d, T %d",
                 count, K, t_pad);
     int total_n = 0;
@@ -555,8 +577,35 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
     const bool large_tiles = (total_n / pf::kTileFeatures) * (t_pad / pf::kTileTokens) >= compute_units();
     const int tile = large_tiles ? pf::kTileFeatures : 64;
     const bool staged = K % 64 == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr;
+    if (staged && accumulate && count == 1 && partials != nullptr) {
+        const int n = prods[0].n;
+        const int big_tiles = (n / pf::kTileFeatures) * (t_pad / pf::kTileTokens);
+        int splits = 1;
+        while (splits < 4 && big_tiles * splits < compute_units() && K % (128 * splits) == 0 && K / (2 * splits) >= 1024) splits *= 2;
+        const size_t stride = static_cast<size_t>(t_pad) * n;
+        if (splits > 1 && stride * splits <= partial_floats) {
+            pf::GemmOutputs o3;
+            for (int i = 0; i < 3; ++i) {
+                o3.w[i] = static_cast<const pf::half_t*>(prods[0].w);
+                o3.y[i] = partials;
+                o3.ldy[i] = n;
+                o3.first_tile[i] = i == 0 ? 0 : 0x7fffffff;
+            }
+            o3.k_len = K / splits;
+            o3.split_stride = stride;
+            hipLaunchKernelGGL((pf::k_gemm_lds<false, 2>), dim3(n / pf::kTileFeatures, t_pad / pf::kTileTokens, splits), dim3(256), 0,
+                               s, o3, xh, xl, K);
+            LPP_CHECK_LAUNCH("k_gemm_lds");
+            hipLaunchKernelGGL(pf::k_add_partials, dim3(static_cast<unsigned>((stride / 4 + 255) / 256)), dim3(256), 0, s, prods[0].y,
+                               partials, splits, stride, stride);
+            LPP_CHECK_LAUNCH("k_add_partials");
+            return LPP_OK;
+        }
+    }
     if (staged) {
         pf::GemmOutputs o3;
+        o3.k_len = K;
+        o3.split_stride = 0;
         int at = 0;
         for (int i = 0; i < 3; ++i) {
             const Product& p = prods[i < count ? i : count - 1];
@@ -649,7 +698,8 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         hipLaunchKernelGGL(pf::k_swiglu_split, dim3((hidden + 255) / 256, t_pad), dim3(256), 0, s, gate, up, hi, lo, hidden, n);
         LPP_CHECK_LAUNCH("k_swiglu_split");
         const Product w2 = {layer_of(LPP_T_W2, l, dim, hidden), x, dim};
-        LPP_TRY(gemm(&w2, 1, hi, lo, hidden, t_pad, true, s));
+        // (the gate buffer is free again: room for the partial products of a split K)
+        LPP_TRY(gemm(&w2, 1, hi, lo, hidden, t_pad, true, s, gate, static_cast<size_t>(t_pad) * hidden));
     }
     LPP_HIP(hipStreamSynchronize(s));
     return LPP_OK;
