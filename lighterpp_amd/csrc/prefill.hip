@@ -357,12 +357,12 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
 // Causal attention over the cache
 // ---------------------------------------------------------------------------
 //
-// One workgroup per (token t, KV head): its query heads (gqa of them) attend to
-// cache positions 0 .. pos0 + t (model.cpp:178-198; every row of the cache for these
+// One wavefront per (token t, KV head), four tokens to a workgroup: its query heads (gqa of
+// them) attend to cache positions 0 .. pos0 + t (model.cpp:178-198; every row of the cache for these
 // positions is in place, this chunk's included).  kGroup lanes share a position,
 // 8 binary16 each; every lane group keeps a running maximum, sum and weighted V sum
-// per query head (rescaled when the maximum grows), and the groups, then the four
-// wavefronts, are merged by the same rule.  Output: the heads' outputs, split into
+// per query head (rescaled when the maximum grows), and the groups are merged by the
+// same rule at the end.  Output: the heads' outputs, split into
 // (hi, lo) for the output projection's GEMM.
 // Sum over the kGroup lanes that share a position, by DPP moves (no LDS round trip).
 template <int kGroup>
@@ -383,13 +383,12 @@ template <int kGroup>
 __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, const uint16_t* __restrict__ key_cache,
                                                    const uint16_t* __restrict__ value_cache, half_t* __restrict__ out_hi,
                                                    half_t* __restrict__ out_lo, int layer, int pos0, int dim, int kv_dim,
-                                                   int hs, int gqa, int seq_len) {
+                                                   int hs, int gqa, int seq_len, int n_tokens) {
     constexpr int kGroups = kWave / kGroup;  // positions a wavefront covers per pass
-    constexpr int kWaves = 4;
-    __shared__ float red[kWaves][kMaxGqa][8 * kGroup + 2];
-    const int t = blockIdx.x, kvh = blockIdx.y;
-    const int npos = pos0 + t + 1;
     const int lane = lane_id(), wave = wave_index();
+    const int t = static_cast<int>(blockIdx.x) * 4 + wave, kvh = blockIdx.y;
+    if (t >= n_tokens) return;  // (wavefronts of a workgroup do not meet again)
+    const int npos = pos0 + t + 1;
     const int sub = lane % kGroup, grp = lane / kGroup;
     const bool lane_live = sub * 8 < hs;
     const int off = lane_live ? sub * 8 : 0;
@@ -412,14 +411,14 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
     }
     // (the rows of the position after this one are requested before this one's arithmetic; past the end
     // the last valid row is read again and dropped)
-    const int first = wave * kGroups + grp;
+    const int first = grp;
     const int clamp = npos - 1;
     uintx4 k_next = load16(kbase + static_cast<size_t>(first < npos ? first : clamp) * hs + off);
     uintx4 v_next = load16(vbase + static_cast<size_t>(first < npos ? first : clamp) * hs + off);
-    for (int p = first; p < npos; p += kWaves * kGroups) {
+    for (int p = first; p < npos; p += kGroups) {
         const half8_t kh = as_half8(k_next);
         const half8_t vh = as_half8(v_next);
-        const int pn = p + kWaves * kGroups;
+        const int pn = p + kGroups;
         k_next = load16(kbase + static_cast<size_t>(pn < npos ? pn : clamp) * hs + off);
         v_next = load16(vbase + static_cast<size_t>(pn < npos ? pn : clamp) * hs + off);
 #pragma unroll
@@ -458,32 +457,12 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
                 for (int o = kGroup; o < kWave; o <<= 1) v += __shfl_xor(v, o);
                 acc[h][e] = v;
             }
-            if (grp == 0) {
+            if (grp == 0 && lane_live) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) red[wave][h][sub * 8 + e] = acc[h][e];
-                if (sub == 0) {
-                    red[wave][h][8 * kGroup] = all;
-                    red[wave][h][8 * kGroup + 1] = ls;
-                }
+                for (int e = 0; e < 8; ++e)
+                    split_store(out_hi, out_lo, static_cast<size_t>(t) * dim + (kvh * gqa + h) * hs + off + e, acc[h][e] / ls);
             }
         }
-    }
-    __syncthreads();
-    // the wavefronts: thread (h, e)
-    for (int idx = threadIdx.x; idx < gqa * hs; idx += blockDim.x) {
-        const int h = idx / hs, e = idx - h * hs;
-        float all = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) all = fmaxf(all, red[w][h][8 * kGroup]);
-        float o = 0.0f, ls = 0.0f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            const float m = red[w][h][8 * kGroup];
-            const float f = (m == -INFINITY) ? 0.0f : exp_fast(m - all);
-            o += red[w][h][e] * f;
-            ls += red[w][h][8 * kGroup + 1] * f;
-        }
-        split_store(out_hi, out_lo, static_cast<size_t>(t) * dim + (kvh * gqa + h) * hs + e, o / ls);
     }
 }
 
@@ -681,11 +660,11 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         LPP_CHECK_LAUNCH("k_rope_scatter");
         // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
         if (hs == 64)
-            hipLaunchKernelGGL(pf::k_attention<8>, dim3(n, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache, m->value_cache, hi,
-                               lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len);
+            hipLaunchKernelGGL(pf::k_attention<8>, dim3((n + 3) / 4, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache,
+                               m->value_cache, hi, lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len, n);
         else
-            hipLaunchKernelGGL(pf::k_attention<16>, dim3(n, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache, m->value_cache, hi,
-                               lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len);
+            hipLaunchKernelGGL(pf::k_attention<16>, dim3((n + 3) / 4, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache,
+                               m->value_cache, hi, lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len, n);
         LPP_CHECK_LAUNCH("k_attention");
         const Product wo = {layer_of(LPP_T_WO, l, dim, dim), x, dim};
         LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s));
