@@ -466,6 +466,149 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same attention on the matrix cores
+// ---------------------------------------------------------------------------
+//
+// A wavefront owns 32 query rows = (32 / gqa) consecutive tokens x the gqa query heads of one KV
+// head, and walks the cache in blocks of 32 positions:
+//   S^T[pos][row] = sum_d K[pos][d] Q[row][d]     A = K block (a lane's 8 d-values: one 16-byte
+//                                                 load from the cache row), B = Q (head + remainder)
+//   online softmax: in the result a LANE holds one query row (its column) and 16 of the block's 32
+//                   positions, the lane 32 further on the other 16 -- maximum, sum and rescaling are
+//                   per lane, with one exchange between the two halves of the wavefront
+//   O^T[d][row] += sum_pos V^T[d][pos] P^T[pos][row]   A = V transposed (k_transpose_v keeps a copy
+//                                                      of the layer's V with positions contiguous),
+//                                                      B = P straight from the lane's own registers
+// A lane's 16 positions of a block are {8j + 4g .. 8j + 4g + 3 : j = 0..3} (g = lane / 32), so as
+// B operand of the second product it supplies, per 16-position step, positions 4g..4g+3 and
+// 8+4g..8+4g+3; the V^T fragment is loaded in the same order (two 8-byte loads).  Any such
+// permutation of k is fine as long as both operands use it.
+// Probabilities and queries are split into binary16 head + remainder like every other activation.
+
+// vt[kvh][d][p] = V[kvh][p][d] of `layer` for p < n_pos, zero for n_pos <= p < vt_stride.
+__global__ __launch_bounds__(256) void k_transpose_v(const uint16_t* __restrict__ value_cache, uint16_t* __restrict__ vt,
+                                                     int layer, int kv_dim, int hs, int seq_len, int n_pos, int vt_stride) {
+    __shared__ uint16_t tile[32][128 + 2];
+    const int p0 = blockIdx.x * 32, kvh = blockIdx.y;
+    const uint16_t* src = value_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * hs;
+    for (int idx = threadIdx.x; idx < 32 * hs; idx += blockDim.x) {
+        const int p = idx / hs, d = idx - p * hs;
+        tile[p][d] = (p0 + p < n_pos) ? src[static_cast<size_t>(p0 + p) * hs + d] : static_cast<uint16_t>(0);
+    }
+    __syncthreads();
+    uint16_t* dst = vt + static_cast<size_t>(kvh) * hs * vt_stride;
+    for (int idx = threadIdx.x; idx < 32 * hs; idx += blockDim.x) {
+        const int d = idx >> 5, p = idx & 31;
+        dst[static_cast<size_t>(d) * vt_stride + p0 + p] = tile[p][d];
+    }
+}
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+template <int kHs>
+__global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict__ q, const uint16_t* __restrict__ key_cache,
+                                                        const uint16_t* __restrict__ vt, half_t* __restrict__ out_hi,
+                                                        half_t* __restrict__ out_lo, int layer, int pos0, int dim, int kv_dim,
+                                                        int gqa, int seq_len, int n_tokens, int vt_stride) {
+    constexpr int kDTiles = kHs / 32, kKSteps = kHs / 16;
+    const int lane = lane_id(), wave = wave_index();
+    const int r = lane & 31, g = lane >> 5;
+    const int tokens_per_tile = 32 / gqa;
+    const int t0 = (static_cast<int>(blockIdx.x) * 4 + wave) * tokens_per_tile;
+    if (t0 >= n_tokens) return;  // (wavefronts of a workgroup do not meet again)
+    const int kvh = blockIdx.y;
+    const int my_tok = t0 + r / gqa, my_head = r % gqa;
+    const bool valid = my_tok < n_tokens;
+    const int tok_c = valid ? my_tok : n_tokens - 1;
+    const int last_tok = (t0 + tokens_per_tile < n_tokens ? t0 + tokens_per_tile : n_tokens) - 1;
+    const int limit = pos0 + last_tok + 1;    // positions the tile reads: [0, limit)
+    const int my_limit = pos0 + tok_c + 1;    // positions this lane's row attends to: [0, my_limit)
+    const uint16_t* kbase = key_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * kHs;
+    const uint16_t* vtb = vt + static_cast<size_t>(kvh) * kHs * vt_stride;
+    const float scale = 1.0f / sqrtf(static_cast<float>(kHs));  // model.cpp:188
+
+    half8_t qh[kKSteps], ql[kKSteps];
+    {
+        const float* qrow = q + static_cast<size_t>(tok_c) * dim + (kvh * gqa + my_head) * kHs + 8 * g;
+#pragma unroll
+        for (int s = 0; s < kKSteps; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = qrow[16 * s + e];
+                const half_t h = static_cast<half_t>(v);
+                qh[s][e] = h;
+                ql[s][e] = static_cast<half_t>(v - static_cast<float>(h));
+            }
+    }
+    floatx16 o[kDTiles];
+#pragma unroll
+    for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[dt][e] = 0.0f;
+    float top = -INFINITY, lsum = 0.0f;
+
+    for (int p0 = 0; p0 < limit; p0 += 32) {
+        floatx16 st;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) st[e] = 0.0f;
+        const int prow = (p0 + r < seq_len) ? p0 + r : seq_len - 1;  // (rows past the tile's limit are masked below)
+        const uint16_t* krow = kbase + static_cast<size_t>(prow) * kHs + 8 * g;
+#pragma unroll
+        for (int s = 0; s < kKSteps; ++s) {
+            const half8_t kf = as_half8(load16(krow + 16 * s));
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qh[s], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, ql[s], st, 0, 0, 0);
+        }
+        float sv[16];
+        float block_top = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int pos = p0 + 8 * (e >> 2) + 4 * g + (e & 3);
+            sv[e] = (pos < my_limit) ? st[e] * scale : -INFINITY;
+            block_top = fmaxf(block_top, sv[e]);
+        }
+        block_top = fmaxf(block_top, __shfl_xor(block_top, 32));
+        const float grown = fmaxf(top, block_top);  // finite from the first block on: position 0 is in every row's range
+        const float corr = (top == -INFINITY) ? 0.0f : exp_fast(top - grown);
+        half8_t ph[2], pl[2];
+        float block_sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float pw = (sv[e] == -INFINITY) ? 0.0f : exp_fast(sv[e] - grown);
+            block_sum += pw;
+            const half_t h = static_cast<half_t>(pw);
+            ph[e >> 3][e & 7] = h;
+            pl[e >> 3][e & 7] = static_cast<half_t>(pw - static_cast<float>(h));
+        }
+        block_sum += __shfl_xor(block_sum, 32);
+        lsum = lsum * corr + block_sum;
+        top = grown;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                const uint16_t* vrow = vtb + static_cast<size_t>(32 * dt + r) * vt_stride + p0 + 16 * s2 + 4 * g;
+                const half4_t a0 = *reinterpret_cast<const half4_t*>(vrow);
+                const half4_t a1 = *reinterpret_cast<const half4_t*>(vrow + 8);
+                const half8_t vf = half8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, ph[s2], o[dt], 0, 0, 0);
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pl[s2], o[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (valid) {
+        const size_t base = static_cast<size_t>(my_tok) * dim + (kvh * gqa + my_head) * kHs;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                split_store(out_hi, out_lo, base + 32 * dt + 8 * (e >> 2) + 4 * g + (e & 3), o[dt][e] / lsum);
+    }
+}
+
 // x[i] += p[0][i] + p[1][i] + ... in that order: the partial products of a GEMM whose K was split.
 __global__ __launch_bounds__(256) void k_add_partials(float* __restrict__ x, const float* __restrict__ p, int splits,
                                                       size_t stride, size_t count) {
@@ -495,7 +638,7 @@ __global__ __launch_bounds__(256) void k_split(const float* __restrict__ x, half
 namespace {
 
 // Buffers of a chunk of t_pad tokens, in lpp_model::pf_buf order.
-enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufCount };
+enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufVt, kBufCount };
 static_assert(kBufCount <= static_cast<int>(sizeof(lpp_model::pf_buf) / sizeof(void*)), "lpp_model::pf_buf is too small");
 
 const char* unsupported_reason(const lpp_model* m) {
@@ -522,7 +665,9 @@ lpp_status ensure_scratch(lpp_model* m, int t_pad) {
                                      t * c.hidden_dim * sizeof(float),
                                      t * c.hidden_dim * sizeof(float),
                                      t * widest * sizeof(pf::half_t),
-                                     t * widest * sizeof(pf::half_t)};
+                                     t * widest * sizeof(pf::half_t),
+                                     // one layer's V with positions contiguous: [kv_dim][seq_len rounded up to 32]
+                                     static_cast<size_t>(m->kv_dim) * ((c.seq_len + 31) / 32 * 32) * sizeof(uint16_t)};
     for (int i = 0; i < kBufCount; ++i) {
         lpp_status st = lpp_malloc(&m->pf_buf[i], bytes[i]);
         if (st != LPP_OK) {
@@ -659,7 +804,23 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
                            dim, kv, hs, c.seq_len);
         LPP_CHECK_LAUNCH("k_rope_scatter");
         // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
-        if (hs == 64)
+        const bool matrix_cores = 32 % m->gqa == 0 && getenv("LPP_PREFILL_VALU_ATTENTION") == nullptr;
+        if (matrix_cores) {
+            const int n_pos = pos0 + n, vt_stride = (n_pos + 31) / 32 * 32;
+            uint16_t* vt = static_cast<uint16_t*>(m->pf_buf[kBufVt]);
+            hipLaunchKernelGGL(pf::k_transpose_v, dim3(vt_stride / 32, c.n_kv_heads), dim3(256), 0, s, m->value_cache, vt, l, kv, hs,
+                               c.seq_len, n_pos, vt_stride);
+            LPP_CHECK_LAUNCH("k_transpose_v");
+            const int tiles = (n + 32 / m->gqa - 1) / (32 / m->gqa);
+            const dim3 grid((tiles + 3) / 4, c.n_kv_heads);
+            if (hs == 64)
+                hipLaunchKernelGGL(pf::k_attention_mfma<64>, grid, dim3(256), 0, s, q, m->key_cache, vt, hi, lo, l, pos0, dim, kv,
+                                   m->gqa, c.seq_len, n, vt_stride);
+            else
+                hipLaunchKernelGGL(pf::k_attention_mfma<128>, grid, dim3(256), 0, s, q, m->key_cache, vt, hi, lo, l, pos0, dim, kv,
+                                   m->gqa, c.seq_len, n, vt_stride);
+            LPP_CHECK_LAUNCH("k_attention_mfma");
+        } else if (hs == 64)
             hipLaunchKernelGGL(pf::k_attention<8>, dim3((n + 3) / 4, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache,
                                m->value_cache, hi, lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len, n);
         else

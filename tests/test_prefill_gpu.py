@@ -93,8 +93,14 @@ def assert_caches_agree(a, b, shape, upto):
     assert not kfb[:, :, upto:, :].any() and not vfb[:, :, upto:, :].any(), "slots beyond the prompt were written"
 
 
+@pytest.mark.parametrize("variant", ["matrix_cores", "fallback_kernels"])
 @pytest.mark.parametrize("name", list(SHAPES))
-def test_prefill_leaves_what_decode_leaves(name):
+def test_prefill_leaves_what_decode_leaves(name, variant, monkeypatch):
+    if variant == "fallback_kernels":
+        # the attention on the vector ALUs and the GEMM with fragments straight from memory (what
+        # shapes outside the fast kernels' conditions get)
+        monkeypatch.setenv("LPP_PREFILL_VALU_ATTENTION", "1")
+        monkeypatch.setenv("LPP_PREFILL_DIRECT", "1")
     shape = SHAPES[name]
     a, b = Model(shape), Model(shape)
     w = a.load_synthetic(7, keep=True)
@@ -226,3 +232,28 @@ def test_prefill_at_full_size_against_decode():
         assert got_tok == want_tok
         tok = want_tok
     b.close()
+
+
+def test_gguf_model_through_the_command_line_with_batched_prefill(tmp_path):
+    """An F16 GGUF file (dims that the batched prefill takes) through python -m lighterpp_amd.driver with and
+    without --batched-prefill: same ids out."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import gguf_writer as gw
+    from lighterpp_amd import synth_tensor
+    shape = Shape(256, 512, 2, 4, 2, 300, 128, 10000.0, fp16=True, tied=True)
+    w = {t: synth_tensor(shape, t, 31) for t in range(12)}
+    file = tmp_path / "model.gguf"
+    gw.write_gguf(file, gw.llama_kv(shape), gw.llama_tensors(shape, w, True, True))
+    root = Path(__file__).resolve().parent.parent
+    ids = ",".join(str(int(i)) for i in capi.synth_token_ids(50, 6, shape.vocab_size))
+    outs = []
+    for extra in ([], ["--batched-prefill"]):
+        out = subprocess.run([sys.executable, "-m", "lighterpp_amd.driver", str(file), "--prompt-ids", ids, "--steps", "100",
+                              "--temperature", "0", "--path", "persistent"] + extra,
+                             cwd=root, capture_output=True, text=True, timeout=110)
+        assert out.returncode == 0, out.stderr
+        outs.append(out.stdout.split("--- Running Inference ---\n", 1)[1].split("\n\n--- Statistics ---", 1)[0])
+    assert outs[0] == outs[1] and len(outs[0].strip()) > 0
