@@ -257,3 +257,26 @@ def test_gguf_model_through_the_command_line_with_batched_prefill(tmp_path):
         assert out.returncode == 0, out.stderr
         outs.append(out.stdout.split("--- Running Inference ---\n", 1)[1].split("\n\n--- Statistics ---", 1)[0])
     assert outs[0] == outs[1] and len(outs[0].strip()) > 0
+
+
+@pytest.mark.parametrize("n", [1, 2, 31, 33, 49])
+def test_prefill_ragged_lengths_and_a_cache_that_ends_inside_a_block(n):
+    """Prompt lengths around the 32-position blocks of the attention, on a cache of 50 positions (the last
+    block of keys and of the transposed V runs past the end of the cache)."""
+    shape = Shape(256, 512, 2, 4, 2, 1024, 50, 10000.0, fp16=True, tied=True)
+    a, b = Model(shape), Model(shape)
+    a.load_synthetic(13)
+    b.load_synthetic(13)
+    a.set_path(capi.PATH_FUSED)
+    b.set_path(capi.PATH_FUSED)
+    prompt = capi.synth_token_ids(n, 21, shape.vocab_size)
+    decode_prompt(a, prompt)
+    b.prefill(prompt, 0)
+    assert_caches_agree(a, b, shape, n)
+    if n < shape.seq_len:
+        ta = a.forward(int(prompt[-1]), n, 0.0)
+        tb = b.forward(int(prompt[-1]), n, 0.0)
+        assert rel_err(b.buffer(capi.B_LOGITS), a.buffer(capi.B_LOGITS).astype(np.float64)) <= LOGIT_TOL
+        assert ta == tb
+    a.close()
+    b.close()
