@@ -253,7 +253,7 @@ struct GemmOutputs {
     size_t split_stride;
 };
 
-template <bool kAccumulate, int kSub>
+template <bool kAccumulate, int kSub, int kTripK>
 __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* __restrict__ xh,
                                                   const half_t* __restrict__ xl, int K) {
     constexpr int kTile = 64 * kSub;           // rows of each operand tile (features, tokens)
@@ -264,8 +264,9 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
     const int tile_x = static_cast<int>(blockIdx.x) - (which == 2 ? o3.first_tile[2] : (which == 1 ? o3.first_tile[1] : 0));
     const int k_first = static_cast<int>(blockIdx.z) * o3.k_len;  // K below is the row length; this workgroup covers k_len columns
     y += static_cast<size_t>(blockIdx.z) * o3.split_stride;
-    constexpr int kRowBytes = 144;             // 64 binary16 + 16 bytes of padding
-    constexpr int kChunks = kTile * 8 / 256;   // 16-byte pieces per thread and operand
+    constexpr int kRowBytes = 2 * kTripK + 16;             // a trip's columns of a row + 16 bytes of padding
+    constexpr int kRowChunks = kTripK / 8;                 // 16-byte pieces of it
+    constexpr int kChunks = kTile * kRowChunks / 256;      // pieces per thread and operand
     __shared__ __align__(16) char tiles[3][kTile * kRowBytes];
     const int tid = static_cast<int>(threadIdx.x);
     const int lane = lane_id();
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
     int dst[kChunks];
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
-        const int id = tid + 256 * j, row = id >> 3, c = id & 7;
+        const int id = tid + 256 * j, row = id / kRowChunks, c = id % kRowChunks;
         src[0][j] = reinterpret_cast<const char*>(w + static_cast<size_t>(f_base + row) * K + k_first) + 16 * c;
         src[1][j] = reinterpret_cast<const char*>(xh + static_cast<size_t>(t_base + row) * K + k_first) + 16 * c;
         src[2][j] = reinterpret_cast<const char*>(xl + static_cast<size_t>(t_base + row) * K + k_first) + 16 * c;
@@ -309,11 +310,11 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
     fetch(0);
     commit();
     __syncthreads();
-    for (int k0 = 0; k0 < o3.k_len; k0 += 64) {
-        const bool more = k0 + 64 < o3.k_len;
-        if (more) fetch(k0 + 64);
+    for (int k0 = 0; k0 < o3.k_len; k0 += kTripK) {
+        const bool more = k0 + kTripK < o3.k_len;
+        if (more) fetch(k0 + kTripK);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {  // four k-steps of 16 columns
+        for (int s = 0; s < kTripK / 16; ++s) {  // k-steps of 16 columns
             half8_t a[kSub], bh[kSub], bl[kSub];
 #pragma unroll
             for (int i = 0; i < kSub; ++i) {
@@ -717,7 +718,7 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
             }
             o3.k_len = K / splits;
             o3.split_stride = stride;
-            hipLaunchKernelGGL((pf::k_gemm_lds<false, 2>), dim3(n / pf::kTileFeatures, t_pad / pf::kTileTokens, splits), dim3(256), 0,
+            hipLaunchKernelGGL((pf::k_gemm_lds<false, 2, 64>), dim3(n / pf::kTileFeatures, t_pad / pf::kTileTokens, splits), dim3(256), 0,
                                s, o3, xh, xl, K);
             LPP_CHECK_LAUNCH("k_gemm_lds");
             hipLaunchKernelGGL(pf::k_add_partials, dim3(static_cast<unsigned>((stride / 4 + 255) / 256)), dim3(256), 0, s, prods[0].y,
@@ -741,11 +742,17 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
         }
         const dim3 grid(at, t_pad / tile);
         if (large_tiles) {
-            if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 2>), grid, dim3(256), 0, s, o3, xh, xl, K);
-            else hipLaunchKernelGGL((pf::k_gemm_lds<false, 2>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 2, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            else hipLaunchKernelGGL((pf::k_gemm_lds<false, 2, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
         } else {
-            if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 1>), grid, dim3(256), 0, s, o3, xh, xl, K);
-            else hipLaunchKernelGGL((pf::k_gemm_lds<false, 1>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            // (small tiles: a trip of 128 columns where K allows, half the barriers and round trips per product)
+            if (K % 128 == 0 && getenv("LPP_PREFILL_TRIP64") == nullptr) {
+                if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 1, 128>), grid, dim3(256), 0, s, o3, xh, xl, K);
+                else hipLaunchKernelGGL((pf::k_gemm_lds<false, 1, 128>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            } else {
+                if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 1, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
+                else hipLaunchKernelGGL((pf::k_gemm_lds<false, 1, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
+            }
         }
         LPP_CHECK_LAUNCH("k_gemm_lds");
         return LPP_OK;
