@@ -280,3 +280,35 @@ def test_prefill_ragged_lengths_and_a_cache_that_ends_inside_a_block(n):
         assert ta == tb
     a.close()
     b.close()
+
+
+def test_prefill_of_a_long_prompt_at_full_size():
+    """Llama-3.2-1B shape with the long-context cache: 1500 prompt ids = three batches (512, 512, 476), the later
+    ones attending to the earlier ones' cache entries; caches and the next step against prefill by decode."""
+    shape = CONFIGS["c4_llama32_1b_longctx_fp16"]
+    n = 1500
+    prompt = capi.synth_token_ids(n, 14, shape.vocab_size)
+    a = Model(shape)
+    a.load_synthetic(1)
+    a.set_path(capi.PATH_PERSISTENT)
+    decode_prompt(a, prompt)
+    tok_a = a.forward(int(prompt[-1]), n, 0.0)
+    logits_a = a.buffer(capi.B_LOGITS).astype(np.float64)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    ka = a.buffer(capi.B_KEY_CACHE).view(np.float16).reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :].astype(F)
+    va = a.buffer(capi.B_VALUE_CACHE).view(np.float16).reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :].astype(F)
+    a.close()
+    b = Model(shape)
+    b.load_synthetic(1)
+    b.set_path(capi.PATH_PERSISTENT)
+    b.prefill(prompt, 0)
+    kb = b.buffer(capi.B_KEY_CACHE).view(np.float16).reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :].astype(F)
+    vb = b.buffer(capi.B_VALUE_CACHE).view(np.float16).reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :].astype(F)
+    for x, y in ((kb, ka), (vb, va)):
+        scale = np.abs(y).max()
+        assert np.all(np.abs(x - y) <= np.maximum(np.abs(y) * 2.0 ** -9, scale * 2.0 ** -11))
+        assert np.mean(x == y) > 0.6
+    tok_b = b.forward(int(prompt[-1]), n, 0.0)
+    assert rel_err(b.buffer(capi.B_LOGITS), logits_a) <= LOGIT_TOL
+    assert tok_a == tok_b
+    b.close()
