@@ -345,7 +345,8 @@ lpp_status lpp_prefill_supported(const lpp_model *m);
 lpp_status lpp_prefill(lpp_model *m, const int *tokens, int n_tokens, int start_pos);
 /* lpp_run with the prompt (all ids but the last) prefilled by lpp_prefill instead of
  * by decode steps; everything else, the uniforms' indexing by position included, as
- * lpp_run.  Falls back to lpp_run's own prefill when the model does not qualify. */
+ * lpp_run.  Falls back to lpp_run's own prefill when the model does not qualify or the
+ * prompt has fewer than 9 ids (a batch costs about five decode steps). */
 lpp_status lpp_run_batched_prefill(lpp_model *m, const int *prompt, int n_prompt, int steps, float temperature,
                                    float topp, const float *uniforms, int *out_tokens, int out_capacity,
                                    lpp_run_result *res);

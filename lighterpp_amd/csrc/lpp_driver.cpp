@@ -198,7 +198,9 @@ lpp_status run_loop(lpp_model* m, const int* prompt, int n_prompt, int steps, fl
     int n_out = 0;
     // 1. prefill, main.cpp:163-180.  Batched: the cache entries of all but the last prompt id in one
     //    pass per 512 ids; what the decode steps would have sampled is what the reference drops.
-    if (batched && n_prompt > 1 && lpp_prefill_supported(m) == LPP_OK) {
+    //    (a batch costs about as much as five decode steps at the 1B shape: short prompts stay with decode)
+    constexpr int kShortestBatchedPrompt = 8;
+    if (batched && n_prompt - 1 >= kShortestBatchedPrompt && lpp_prefill_supported(m) == LPP_OK) {
         for (int i = 0; i < n_prompt - 1; ++i) push(prompt[i]);
         LPP_TRY(lpp_prefill(m, prompt, n_prompt - 1, 0));
         pos = n_prompt - 1;
