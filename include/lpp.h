@@ -359,6 +359,18 @@ lpp_status lpp_run_batched_prefill(lpp_model *m, const int *prompt, int n_prompt
 lpp_status lpp_prefill_gemm(float *d_y, const void *d_w, const float *d_x, int n, int k, int n_tokens,
                             int accumulate);
 
+/* lpp_prefill_gemm for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, checks and result, bit for bit; the
+ * binary16 head and remainder of x go to an 8 MiB array that lives in the library's
+ * device image instead of two fresh allocations, so n_tokens * k may not exceed
+ * 2097152 (LPP_ERR_INVALID_ARG beyond that).  Nothing is allocated, freed or
+ * synchronised: the launches are queued on the library's stream and the call
+ * returns.  Every call on a device uses that device's one array: calls that overlap
+ * on one device (two streams, two threads) race. */
+lpp_status lpp_prefill_gemm_noalloc(float *d_y, const void *d_w, const float *d_x, int n, int k,
+                                    int n_tokens, int accumulate);
+
 /* Per-kernel timing of the fused path, measured with HIP events on the launch
  * stream: each kernel class is recorded n_layers times (one launch per layer,
  * so every launch streams different weights) into a graph that is replayed

@@ -111,6 +111,7 @@ SIGNATURES = {
     "lpp_prefill_supported": (_i, [_vp]),
     "lpp_prefill": (_i, [_vp, _vp, _i, _i]),
     "lpp_prefill_gemm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "lpp_prefill_gemm_noalloc": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "lpp_gguf_open": (_i, [C.POINTER(_vp), C.c_char_p]),
     "lpp_gguf_close": (_i, [_vp]),
     "lpp_gguf_config": (_i, [_vp, C.POINTER(LppConfig)]),

@@ -54,6 +54,10 @@ int compute_units();
 // stays valid until the next call that has to grow the same table.
 lpp_status rope_table(int head_size, float rope_base, int min_positions, const float2** d_table);
 
+// Resolves, for the current device, the address of the device-resident scratch that
+// lpp_prefill_gemm_noalloc works in (prefill.hip); lpp_init calls it once per device.
+lpp_status prefill_gemm_scratch_setup();
+
 // Launch helpers implemented in the .hip files and used by the model code.
 namespace k {
 

@@ -134,7 +134,7 @@ lpp_status lpp_init(int device) {
     lpp::g_rt.device = device;
     lpp::g_rt.cus = prop.multiProcessorCount;
     lpp::g_rt.ready = true;
-    return LPP_OK;
+    return lpp::prefill_gemm_scratch_setup();
 }
 
 lpp_status lpp_set_stream(void* hip_stream) {

@@ -916,3 +916,66 @@ lpp_status lpp_prefill_gemm(float* d_y, const void* d_w, const float* d_x, int n
 }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------------------
+// The same product for callers that cannot allocate
+// ---------------------------------------------------------------------------
+
+namespace lpp {
+namespace {
+
+// Room for the binary16 head and remainder of the activations: kNoAllocElements each.
+constexpr size_t kNoAllocElements = size_t{1} << 21;
+static __device__ __align__(256) unsigned char scratch[2 * kNoAllocElements * sizeof(pf::half_t)];
+
+// Device address of `scratch` per device.  In host code the array's name is only a handle
+// for hipGetSymbolAddress; every device that loads the library holds its own copy.
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+lpp_status scratch_address(void** out) {
+    int device = -1;
+    LPP_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(LPP_ERR_UNSUPPORTED, "device ordinal %d beyond %d", device, kMaxDevices - 1);
+    if (g_scratch_ptr[device] == nullptr) {
+        void* p = nullptr;
+        LPP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return fail(LPP_ERR_HIP, "hipGetSymbolAddress returned no address for the prefill scratch");
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return LPP_OK;
+}
+
+}  // namespace
+
+lpp_status prefill_gemm_scratch_setup() {
+    void* p = nullptr;
+    return scratch_address(&p);
+}
+
+}  // namespace lpp
+
+extern "C" {
+
+lpp_status lpp_prefill_gemm_noalloc(float* d_y, const void* d_w, const float* d_x, int n, int k, int n_tokens, int accumulate) {
+    using namespace lpp;
+    LPP_REQUIRE(d_y && d_w && d_x, "lpp_prefill_gemm_noalloc: null argument");
+    LPP_REQUIRE(n_tokens > 0 && n_tokens % pf::kTileTokens == 0, "lpp_prefill_gemm_noalloc: n_tokens %d not a positive multiple of %d",
+                n_tokens, pf::kTileTokens);
+    LPP_REQUIRE(n > 0 && n % pf::kTileFeatures == 0 && k > 0 && k % 32 == 0, "lpp_prefill_gemm_noalloc: n %d k %d", n, k);
+    const size_t count = static_cast<size_t>(n_tokens) * k;
+    LPP_REQUIRE(count <= kNoAllocElements, "lpp_prefill_gemm_noalloc: n_tokens * k = %zu exceeds the built-in scratch of %zu elements",
+                count, kNoAllocElements);
+    hipStream_t s = stream();
+    void* base = nullptr;
+    LPP_TRY(scratch_address(&base));
+    pf::half_t* hi = static_cast<pf::half_t*>(base);
+    pf::half_t* lo = hi + kNoAllocElements;
+    hipLaunchKernelGGL(pf::k_split, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s, d_x, hi, lo, count);
+    LPP_CHECK_LAUNCH("k_split");
+    const Product one = {d_w, d_y, n};
+    return gemm(&one, 1, hi, lo, k, n_tokens, accumulate != 0, s);
+}
+
+}  // extern "C"
