@@ -104,22 +104,29 @@ def cpu_baseline(shape, weights, wl, first_token, start, budget_s: float):
                 sample=f"{n} decode steps from position 0 of the same workload, single thread, {el:.1f}s")
 
 
-def parity_check(model, shape, weights, first_token, n_steps: int):
-    """Teacher-forced logits comparison against the oracle on the first positions."""
+def parity_check(model, shape, weights, prompt, n_steps: int, start: int):
+    """Teacher-forced logits comparison against the oracle from the workload's own first position:
+    the prompt ids, then the oracle's greedy ids.  A workload that starts on a pre-filled cache
+    (config 4) gets the same cache contents on both sides, widened exactly for the oracle."""
     import oracle_binding as ob
     from lighterpp_amd import capi
     o = ob.OracleModel(shape, weights, fp16=shape.fp16, kv_round_f16=True)
     model.reset()
-    tok, worst, agree = first_token, 0.0, 0
-    for pos in range(n_steps):
+    if start > 0:
+        prefill_cache(model, shape, start)
+        o.buf("key_cache")[:] = capi.f16_to_f32(model.buffer(capi.B_KEY_CACHE))
+        o.buf("value_cache")[:] = capi.f16_to_f32(model.buffer(capi.B_VALUE_CACHE))
+    tok, worst, agree = int(prompt[0]), 0.0, 0
+    for i in range(n_steps):
+        pos = start + i
         nxt = model.forward(tok, pos, 0.0)
         want = o.forward_logits(tok, pos)
         got = model.buffer(capi.B_LOGITS)
         worst = max(worst, float(np.max(np.abs(got - want)) / np.max(np.abs(want))))
         agree += int(nxt == int(np.argmax(want)))
-        tok = int(np.argmax(want))
+        tok = int(prompt[i + 1]) if i + 1 < len(prompt) else int(np.argmax(want))
     o.close()
-    return dict(steps=n_steps, max_rel_logit_err=worst, greedy_agreement=agree / n_steps, tolerance=2e-3,
+    return dict(steps=n_steps, first_pos=start, max_rel_logit_err=worst, greedy_agreement=agree / n_steps, tolerance=2e-3,
                 checker="oracle (CPU restatement, binary16 KV store)")
 
 
@@ -260,7 +267,7 @@ def main() -> int:
 
     parity = None
     if args.parity_steps > 0:
-        parity = parity_check(model, shape, weights, int(prompt[0]), args.parity_steps)
+        parity = parity_check(model, shape, weights, prompt, min(args.parity_steps, shape.seq_len - wl["start"]), wl["start"])
         log(f"parity: {parity}")
     cpu = None
     if args.cpu_seconds > 0:

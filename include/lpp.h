@@ -193,7 +193,20 @@ lpp_status lpp_model_tie_classifier(lpp_model *m);
 lpp_status lpp_model_tensor_ptr(lpp_model *m, int tensor, void **d_ptr);
 lpp_status lpp_model_buffer_ptr(lpp_model *m, int buffer, void **d_ptr, size_t *bytes);
 
+/* LPP_PATH_PERSISTENT takes weight rows of up to 32 KiB (8192 fp32 or 16384 binary16
+ * columns); for a wider dim or hidden_dim this returns LPP_ERR_UNSUPPORTED and the path
+ * stays as it was. */
 lpp_status lpp_model_set_path(lpp_model *m, int path);
+/* Test hooks of LPP_PATH_PERSISTENT (no counterpart in the reference).  Its kernel waits
+ * for values other workgroups publish with a bounded number of polls (default 2^20, far
+ * beyond any real wait): a wait that runs out raises a flag that ends every other wait,
+ * all workgroups leave the kernel normally, and lpp_forward / lpp_generate return
+ * LPP_ERR_HIP ("gave up waiting"); the model is usable again after lpp_model_reset or
+ * simply at the next call, because values carry sequence numbers that never repeat.
+ * set_spin_limit changes the bound; set_sequence_base moves the 32-bit sequence count
+ * (the library re-zeroes its exchange slots and restarts the count before it can wrap). */
+lpp_status lpp_model_set_spin_limit(lpp_model *m, unsigned polls);
+lpp_status lpp_model_set_sequence_base(lpp_model *m, unsigned base);
 /* Forget the KV cache contents (zero-fill, as malloc_run_state leaves it). */
 lpp_status lpp_model_reset(lpp_model *m);
 
@@ -324,7 +337,9 @@ typedef struct lpp_run_result {
  * the last prompt id (penalty 1.05) until position `steps` or an end-of-sequence
  * id; 64-entry sliding penalty window.  prompt == NULL stands for the single id 1
  * (main.cpp:147-151).  uniforms[pos] is the draw of the forward at position pos
- * (the reference draws inside every forward, prefill included).  Positions beyond
+ * (the reference draws inside every forward, prefill included): the array must hold
+ * max(steps, n_prompt - 1) entries, since a prompt longer than `steps` is still
+ * prefilled to its end; it may be NULL only when temperature is 0.  Positions beyond
  * seq_len are an error here (the reference overruns its cache). */
 lpp_status lpp_run(lpp_model *m, const int *prompt, int n_prompt, int steps, float temperature,
                    float topp, const float *uniforms, int *out_tokens, int out_capacity,
@@ -333,8 +348,9 @@ lpp_status lpp_run(lpp_model *m, const int *prompt, int n_prompt, int steps, flo
 /* Batched prefill.  The reference has none: main.cpp:163-180 prefills by
  * decoding the prompt token by token and dropping what the sampler returns).  Writes
  * the key/value cache entries of tokens[0 .. n_tokens) at positions start_pos ..
- * start_pos + n_tokens - 1, all layers, exactly what those decode steps leave behind
- * for later steps to read (K and V rounded to binary16, model.cpp:171-176); no logits,
+ * start_pos + n_tokens - 1, all layers: what those decode steps leave behind for later
+ * steps to read (K and V rounded to binary16, model.cpp:171-176), within one binary16
+ * step of it (the GEMMs sum in another order than the decode GEMVs); no logits,
  * no sampling.  The prompt goes through each layer as one batch of up to 512 tokens:
  * GEMMs on the matrix cores, every weight read once per batch.  Needs binary16
  * weights, dim / kv_dim / hidden_dim multiples of 128, head_size 64 or 128, at most 8
@@ -397,6 +413,12 @@ lpp_status lpp_profile_kernels(lpp_model *m, int pos, int reps, lpp_kernel_time 
  * *count = marks * phases, *marks_per_phase = marks. */
 lpp_status lpp_trace_token(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count,
                            int *marks_per_phase);
+/* The same with every workgroup traced: out[(w * *count) + marks * i + k], w < *workgroups,
+ * all on workgroup 0's time axis; capacity >= *count * *workgroups (one workgroup per
+ * compute unit).  The marks cost about half a microsecond each: a traced token is some
+ * 10 % slower than an untraced one. */
+lpp_status lpp_trace_token_all(lpp_model *m, int pos, unsigned long long *out, int capacity, int *count,
+                               int *marks_per_phase, int *workgroups);
 
 /* ===================================================================== */
 /* C. Runtime plumbing                                                    */

@@ -93,6 +93,8 @@ SIGNATURES = {
     "lpp_model_tensor_ptr": (_i, [_vp, _i, C.POINTER(_vp)]),
     "lpp_model_buffer_ptr": (_i, [_vp, _i, C.POINTER(_vp), C.POINTER(_sz)]),
     "lpp_model_set_path": (_i, [_vp, _i]),
+    "lpp_model_set_spin_limit": (_i, [_vp, C.c_uint]),
+    "lpp_model_set_sequence_base": (_i, [_vp, C.c_uint]),
     "lpp_model_reset": (_i, [_vp]),
     "lpp_attention": (_i, [_vp, _i, _i]),
     "lpp_transformer_block": (_i, [_vp, _i, _i]),
@@ -100,6 +102,7 @@ SIGNATURES = {
     "lpp_generate": (_i, [_vp, _i, _i, _i, _f, _f, _f, _vp, _ip, _i, _vp, _vp, C.POINTER(LppGenStats)]),
     "lpp_profile_kernels": (_i, [_vp, _i, _i, C.POINTER(LppKernelTime), _i, _ip]),
     "lpp_trace_token": (_i, [_vp, _i, C.POINTER(C.c_ulonglong), _i, _ip, _ip]),
+    "lpp_trace_token_all": (_i, [_vp, _i, _vp, _i, _ip, _ip, _ip]),
     # D. checkpoint reader and driver loop
     "lpp_checkpoint_open": (_i, [C.POINTER(_vp), C.c_char_p]),
     "lpp_checkpoint_close": (_i, [_vp]),

@@ -63,6 +63,9 @@ constexpr int kMaxAttHeads = 2;                    // query heads of one KV head
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
 
 typedef unsigned long long u64;
+// Sequence-number base beyond which the host re-zeroes the tagged slots and restarts the count
+// (a token advances the base by 5 * layers + 2; 2^32 would be reached after tens of millions of tokens).
+constexpr unsigned kTagWrapGuard = 0xf0000000u;
 
 __device__ __forceinline__ u64 pack(float v, unsigned tag) {
     return (static_cast<u64>(tag) << 32) | static_cast<u64>(__float_as_uint(v));
@@ -96,6 +99,7 @@ struct Tagged {
     unsigned base;    // sequence-number base of this launch, advanced by the host once per token
     unsigned* abort;  // raised by a wavefront whose poll ran out of patience
     unsigned spin_limit;
+    int trace_stride;  // timeline: 0 = workgroup 0 only; else every workgroup writes its own block of this many words
 };
 
 // Rows of each matrix one workgroup owns (a contiguous block), and LDS sizes.
@@ -1415,10 +1419,14 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     const int wave = wave_index();
     if (wave < kGemvWaves) {
         gemv_role<kF16>(a, ctl, row_lists + static_cast<size_t>(wg * kGemvWaves + wave) * row_list_stride, wave, l.xs,
-                        l.results, wg == 0 && wave == 0 && a.trace != nullptr);
+                        l.results, (wg == 0 || t.trace_stride > 0) && wave == 0 && a.trace != nullptr);
     } else {
-        Ctx c{a, t, b, ctl, t.base, (wg == 0) ? a.trace : nullptr, 0u,
-              __builtin_amdgcn_readfirstlane(a.step->token), t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg};
+        // (kept inside the vocabulary whatever a launch that gave up left in the record: it indexes the embedding)
+        const int token_in = min(max(__builtin_amdgcn_readfirstlane(a.step->token), 0), a.vocab - 1);
+        unsigned long long* my_trace = nullptr;
+        if (a.trace != nullptr && (wg == 0 || t.trace_stride > 0)) my_trace = a.trace + static_cast<size_t>(wg) * t.trace_stride;
+        Ctx c{a, t, b, ctl, t.base, my_trace, 0u,
+              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg};
         Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
         if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
         io_role<kF16>(c, io, l);
@@ -1516,6 +1524,7 @@ df::Tagged tagged_of(const lpp_model* m, bool generating) {
     t.base = m->df_base;
     t.abort = m->sync_words + 65;
     t.spin_limit = m->spin_limit;
+    t.trace_stride = m->df_trace_stride;
     return t;
 }
 
@@ -1626,9 +1635,32 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
 
 size_t dataflow_tagged_bytes(const lpp_model* m) { return tagged_count(m, kGridCap) * sizeof(df::u64); }
 
+// A streaming wavefront covers one column slice of at most kStepLoads 1-KiB chunks per row, and a
+// row has at most one slice per streaming wavefront: rows beyond 8 x 4 KiB (8192 fp32 or 16384
+// binary16 columns) do not fit.  nullptr when the shape fits, else the reason.
+const char* dataflow_unsupported_reason(const lpp_model* m) {
+    const lpp_config& c = m->cfg;
+    const int chunk_cols = c.weight_precision == LPP_WEIGHT_FP16 ? 512 : 256;
+    const int widest = c.hidden_dim > c.dim ? c.hidden_dim : c.dim;
+    if (df::slice_width(widest, chunk_cols) > df::kStepLoads * chunk_cols)
+        return "persistent decode: weight rows wider than 32 KiB (8192 fp32 or 16384 binary16 columns)";
+    if (m->head_size > df::kMaxHeadPad) return "persistent decode: head_size exceeds 128";
+    return nullptr;
+}
+
 template <bool kF16>
 static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
+    if (const char* why = dataflow_unsupported_reason(m)) return fail(LPP_ERR_UNSUPPORTED, "%s", why);
     const Plan p = plan_for(m);
+    // Sequence numbers are compared for equality, so they must not come round to values that slots
+    // written long ago (split partials of a longer context, say) may still hold: well before the
+    // 32-bit count wraps, drain the stream, clear every tagged slot and start again from zero.
+    if (m->df_base > df::kTagWrapGuard) {
+        LPP_HIP(hipStreamSynchronize(s));
+        LPP_TRY(lpp_memset(m->tagged, 0, dataflow_tagged_bytes(m)));
+        LPP_HIP(hipStreamSynchronize(s));
+        m->df_base = 0;
+    }
     if (m->persist_grid == 0) {
         LPP_REQUIRE(p.grid <= kGridCap, "persistent decode: %d compute units exceed the statistics table", p.grid);
         LPP_REQUIRE(m->head_size <= df::kMaxHeadPad, "persistent decode: head_size %d exceeds %d", m->head_size,

@@ -612,11 +612,12 @@ extern "C" lpp_status lpp_profile_kernels(lpp_model* m, int pos, int reps, lpp_k
                                                       : profile_impl<false>(m, pos, reps, out, capacity, count);
 }
 
-// Timeline of one token on the persistent path, workgroup 0: for phase i, mark k
-// is out[marks * i + k], in 10 ns ticks from the kernel's first instruction
-// (0 where a mark does not apply).  The last of three replays is reported.
-extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count,
-                                      int* marks_per_phase) {
+// Timeline of one token on the persistent path: for phase i, mark k is
+// out[marks * i + k], in 10 ns ticks from workgroup 0's first instruction (0 where a
+// mark does not apply).  The last of three replays is reported.  With all_workgroups
+// the same block follows for every workgroup, one after the other.
+static lpp_status trace_impl(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count, int* marks_per_phase,
+                             int* workgroups, bool all_workgroups) {
     using namespace lpp;
     LPP_REQUIRE(m && out && count && marks_per_phase, "lpp_trace_token: null argument");
     LPP_REQUIRE(pos >= 0 && pos < m->cfg.seq_len, "lpp_trace_token: pos %d outside [0, %d)", pos, m->cfg.seq_len);
@@ -625,11 +626,14 @@ extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long*
         if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
     const int marks = static_cast<int>(dataflow_trace_marks());
     const int n = marks * static_cast<int>(dataflow_phases_per_token(m->cfg.n_layers));
-    LPP_REQUIRE(capacity >= n, "lpp_trace_token: capacity %d < %d", capacity, n);
+    const int nwg = all_workgroups ? compute_units() : 1;
+    const size_t block = static_cast<size_t>(n) + 1;  // the last word of a block is the workgroup's start time
+    LPP_REQUIRE(static_cast<size_t>(capacity) >= static_cast<size_t>(n) * nwg, "lpp_trace_token: capacity %d < %zu", capacity,
+                static_cast<size_t>(n) * nwg);
     const int saved_path = m->path;
     m->path = LPP_PATH_PERSISTENT;
     void* p = nullptr;
-    LPP_TRY(lpp_malloc(&p, static_cast<size_t>(n + 1) * sizeof(unsigned long long)));
+    LPP_TRY(lpp_malloc(&p, block * nwg * sizeof(unsigned long long)));
     unsigned long long* d_trace = static_cast<unsigned long long*>(p);
     StepParams sp{};
     sp.pos = pos;
@@ -639,13 +643,15 @@ extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long*
     sp.freeze = 1;
     hipStream_t s = stream();
     lpp_status st = begin_run(m, sp, s);
-    if (st == LPP_OK) st = lpp_memset(d_trace, 0, static_cast<size_t>(n + 1) * sizeof(unsigned long long));
+    if (st == LPP_OK) st = lpp_memset(d_trace, 0, block * nwg * sizeof(unsigned long long));
+    m->df_trace_stride = all_workgroups ? static_cast<int>(block) : 0;
     for (int rep = 0; rep < 3 && st == LPP_OK; ++rep) {
         DecodeArgs a = make_args(m, false);
         a.trace = d_trace;
         st = dataflow_launch(m, a, s);
     }
-    std::vector<unsigned long long> host(static_cast<size_t>(n + 1));
+    m->df_trace_stride = 0;
+    std::vector<unsigned long long> host(block * nwg);
     if (st == LPP_OK && hipStreamSynchronize(s) != hipSuccess) st = fail(LPP_ERR_HIP, "trace run failed");
     if (st == LPP_OK && hipMemcpy(host.data(), d_trace, host.size() * sizeof(unsigned long long),
                                   hipMemcpyDeviceToHost) != hipSuccess)
@@ -654,8 +660,24 @@ extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long*
     m->path = saved_path;
     if (st != LPP_OK) return st;
     const unsigned long long t0 = host[static_cast<size_t>(n)];
-    for (int i = 0; i < n; ++i) out[i] = host[static_cast<size_t>(i)] >= t0 ? host[static_cast<size_t>(i)] - t0 : 0ull;
+    for (int w = 0; w < nwg; ++w)
+        for (int i = 0; i < n; ++i) {
+            const unsigned long long v = host[w * block + static_cast<size_t>(i)];
+            out[static_cast<size_t>(w) * n + i] = v >= t0 ? v - t0 : 0ull;
+        }
     *count = n;
     *marks_per_phase = marks;
+    if (workgroups) *workgroups = nwg;
     return LPP_OK;
+}
+
+extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count,
+                                      int* marks_per_phase) {
+    return trace_impl(m, pos, out, capacity, count, marks_per_phase, nullptr, false);
+}
+
+extern "C" lpp_status lpp_trace_token_all(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count,
+                                          int* marks_per_phase, int* workgroups) {
+    LPP_REQUIRE(workgroups != nullptr, "lpp_trace_token_all: null argument");
+    return trace_impl(m, pos, out, capacity, count, marks_per_phase, workgroups, true);
 }

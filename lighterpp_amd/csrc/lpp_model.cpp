@@ -224,7 +224,21 @@ lpp_status lpp_model_set_path(lpp_model* m, int path) {
     LPP_REQUIRE(m != nullptr, "lpp_model_set_path: null model");
     LPP_REQUIRE(path == LPP_PATH_OPS || path == LPP_PATH_FUSED || path == LPP_PATH_PERSISTENT,
                 "lpp_model_set_path: path %d", path);
+    if (path == LPP_PATH_PERSISTENT)
+        if (const char* why = lpp::dataflow_unsupported_reason(m)) return lpp::fail(LPP_ERR_UNSUPPORTED, "%s", why);
     m->path = path;
+    return LPP_OK;
+}
+
+lpp_status lpp_model_set_spin_limit(lpp_model* m, unsigned polls) {
+    LPP_REQUIRE(m != nullptr && polls > 0u, "lpp_model_set_spin_limit: null model or zero bound");
+    m->spin_limit = polls;
+    return LPP_OK;
+}
+
+lpp_status lpp_model_set_sequence_base(lpp_model* m, unsigned base) {
+    LPP_REQUIRE(m != nullptr, "lpp_model_set_sequence_base: null model");
+    m->df_base = base;
     return LPP_OK;
 }
 

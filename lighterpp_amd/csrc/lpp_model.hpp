@@ -63,6 +63,7 @@ struct lpp_model {
     float df_temperature = 0.0f, df_penalty = 1.0f, df_r = 0.0f;
     const float* df_uniforms_host = nullptr; // per-step draws of the generate call in progress (host memory)
     unsigned df_base = 0;                    // sequence-number base of the next persistent launch
+    int df_trace_stride = 0;                 // timeline words per workgroup when every workgroup is traced (0: workgroup 0 only)
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
     unsigned spin_limit = 1u << 20;          // polls a wait for tagged inputs may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
@@ -100,6 +101,9 @@ size_t tensor_bytes(const lpp_config& c, int tensor);
 
 // Implemented in prefill.hip: frees the batched prefill's buffers.
 void prefill_release(lpp_model* m);
+
+// Implemented in dataflow_decode.hip: why LPP_PATH_PERSISTENT cannot take this model's shape, or nullptr.
+const char* dataflow_unsupported_reason(const lpp_model* m);
 
 // Implemented in fused_decode.hip.
 lpp_status fused_prepare(lpp_model* m);

@@ -48,7 +48,13 @@ def main(argv=None) -> int:
     print(f"Dim: {c.dim}\nHidden Dim: {c.hidden_dim}\nLayers: {c.n_layers}\nHeads: {c.n_heads}\nKV Heads: {c.n_kv_heads}")
     print(f"Vocab: {c.vocab_size}\nSeq Len: {c.seq_len}\nRoPE Base: {c.rope_base:.0f}\nTemperature: {args.temperature:.2f}")
     model = Model.from_gguf(ck) if is_gguf else Model.from_checkpoint(ck)
-    model.set_path(PATHS[args.path])
+    try:
+        model.set_path(PATHS[args.path])
+    except capi.LppError as e:  # e.g. fp32 rows wider than the persistent kernel takes
+        if e.status != capi.LPP_ERR_UNSUPPORTED or args.path != "persistent":
+            raise
+        print(f"note: {e}; using the fused graph path")
+        model.set_path(PATHS["fused"])
     tok = None
     if args.tokenizer:
         tok = Tokenizer.load(args.tokenizer, c.vocab_size)
@@ -64,7 +70,7 @@ def main(argv=None) -> int:
         prompt = tok.encode(args.prompt, 2048)  # main.cpp:140-146
         print(f"Encoded {len(prompt)} tokens.")
     steps = min(args.steps, c.seq_len)
-    uniforms = capi.synth_uniform_f32(steps, args.seed)
+    uniforms = capi.synth_uniform_f32(max(steps, len(prompt or [1])), args.seed)  # one draw per position, prompt included
     print("\n--- Running Inference ---")
     tokens, res = model.run(prompt, steps, args.temperature, 1.0, uniforms, batched_prefill=args.batched_prefill)
     if tok is not None:

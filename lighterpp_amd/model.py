@@ -362,7 +362,9 @@ class Model:
         up = None
         if uniforms is not None:
             u = np.ascontiguousarray(uniforms, dtype=np.float32)
-            assert u.size >= steps
+            need = max(steps, pn - 1)  # one draw per position: the prompt is prefilled to its end whatever `steps` is
+            if u.size < need:
+                raise ValueError(f"run: {u.size} uniforms for {need} positions (max(steps, len(prompt) - 1))")
             up = C.c_void_p(u.ctypes.data)
         res = capi.LppRunResult()
         entry = self.lib.lpp_run_batched_prefill if batched_prefill else self.lib.lpp_run

@@ -299,3 +299,87 @@ def test_persistent_timeline_is_ordered():
     assert published[-1] < 100_000_00, "a tiny model's token takes far less than a second (10 ns ticks)"
     m.close()
     o.close()
+
+
+def test_rows_wider_than_the_persistent_kernel_takes():
+    """fp32 rows of more than 8192 columns (eight column slices of 1024) do not fit the persistent
+    kernel's step lists: it must refuse the shape, not drop columns; the other two schedules take it
+    and agree with the oracle."""
+    shape = Shape(256, 8448, 1, 4, 2, 300, 16, 10000.0, fp16=False, tied=True)
+    m, o = build(shape, 6)
+    with pytest.raises(capi.LppError) as e:
+        m.set_path(capi.PATH_PERSISTENT)
+    assert e.value.status == capi.LPP_ERR_UNSUPPORTED
+    wants, fed, tok = [], [], 5
+    for pos in range(6):
+        fed.append(tok)
+        wants.append(o.forward_logits(tok, pos))
+        tok = int(np.argmax(wants[-1]))
+    for path in (capi.PATH_OPS, capi.PATH_FUSED):
+        m.reset()
+        m.set_path(path)
+        for pos in range(6):
+            m.forward(fed[pos], pos, 0.0)
+            assert rel_err(m.buffer(capi.B_LOGITS), wants[pos]) <= LOGIT_TOL
+    m.close()
+    o.close()
+    # the widest rows it does take: 8192 fp32 columns, all eight slices full
+    shape = Shape(256, 8192, 1, 4, 2, 300, 16, 10000.0, fp16=False, tied=True)
+    m, o = build(shape, 6)
+    m.set_path(capi.PATH_PERSISTENT)
+    tok = 5
+    for pos in range(6):
+        m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL
+        tok = int(np.argmax(want))
+    m.close()
+    o.close()
+
+
+def test_persistent_bounded_wait_gives_up_and_recovers():
+    """The persistent kernel's waits for other workgroups' values are bounded.  With the bound set to
+    one poll by the host, a wait runs out, every workgroup leaves the kernel normally, the call
+    reports LPP_ERR_HIP, and the same model decodes correctly again once the bound is restored."""
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m, o = build(shape, 12)
+    m.set_path(capi.PATH_PERSISTENT)
+    tok = 9
+    want0 = o.forward_logits(tok, 0)
+    assert m.forward(tok, 0, 0.0) == int(np.argmax(want0))
+    capi.check(m.lib.lpp_model_set_spin_limit(m.handle, 1))
+    with pytest.raises(capi.LppError) as e:
+        m.forward(int(np.argmax(want0)), 1, 0.0)
+    assert e.value.status == capi.LPP_ERR_HIP and "gave up" in str(e.value)
+    with pytest.raises(capi.LppError):
+        m.generate(3, 1, 4, temperature=0.0)
+    capi.check(m.lib.lpp_model_set_spin_limit(m.handle, 1 << 20))
+    m.reset()
+    tok = 9
+    for pos in range(8):
+        nxt = m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos) if pos > 0 else want0
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL
+        assert nxt == int(np.argmax(want))
+        tok = nxt
+    m.close()
+    o.close()
+
+
+def test_persistent_sequence_numbers_restart_before_they_wrap():
+    """Hand-over tags are 32-bit sequence numbers compared for equality.  Moved close to the end of
+    their range by the host, they are re-based (slots cleared, count restarted) without a wrong step."""
+    shape = SMALL_SHAPES["gqa4_fp16"]
+    m, o = build(shape, 13)
+    m.set_path(capi.PATH_PERSISTENT)
+    tok = 4
+    for pos in range(12):
+        if pos == 4:
+            capi.check(m.lib.lpp_model_set_sequence_base(m.handle, 0xF0000000 - 20))  # two tokens short of the guard
+        nxt = m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL, pos
+        assert nxt == int(np.argmax(want))
+        tok = nxt
+    m.close()
+    o.close()
