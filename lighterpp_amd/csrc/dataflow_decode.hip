@@ -38,7 +38,10 @@
 // finished reading the phase before the previous one.  Global polls are bounded:
 // a wavefront that gives up raises a shared abort flag that ends every other
 // poll, and no LDS wait depends on a global one, so the grid always drains.
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <unordered_map>
 #include <vector>
 
 #include "decode_phases.hpp"
@@ -59,6 +62,10 @@ constexpr int kPollBatch = 8;                      // tagged values one thread r
 constexpr int kItemPositions = 1024;               // a one-head attention work item stays within twice this many positions
 constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS copy of the penalty window
 constexpr int kMaxHeadPad = 128;
+#ifndef LPP_SHORT_ROUNDS
+#define LPP_SHORT_ROUNDS 2
+#endif
+constexpr int kShortRounds = LPP_SHORT_ROUNDS;          // cache rows per lane group a one-head work item requests at once
 constexpr int kMaxAttHeads = 2;                    // query heads of one KV head a long-context work item covers
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
 
@@ -89,6 +96,11 @@ struct Tagged {
     u64* hb;     // [hidden]  SwiGLU output
     u64* part;   // [n_heads][splits_cap][head_size + 2] attention split partials
     u64* stats;  // [nwg][4]  per-workgroup sampler statistics (max, sum, argmax)
+    // Copies of hb that only the compute units of one XCD write and read (gather_values): [n_xcc][near_hidden_stride]
+    u64* near_hb;
+    int near_hidden_stride;  // tagged values per XCD
+    int n_xcc;               // XCDs the workgroups go round in turn; 1: no near copies
+    int share_hidden;        // values of hb each workgroup of an XCD fetches for the others
     int splits_cap;
     unsigned hs_magic;     // floor(2^32 / head_size) + 1: x / head_size == __umulhi(x, hs_magic) for x < 2^25
     int att_splits;        // context splits per query head at this position (worked out on the host: the search
@@ -106,7 +118,12 @@ struct Tagged {
 struct Blocks {
     int qkv;    // rows of the stacked [Wq; Wk; Wv], even
     int o;      // rows of Wo
-    int gu;     // hidden units (one gate row and one up row each)
+    int gu;     // hidden units (one gate row and one up row each) of a workgroup from gu_split on
+    int gu_a;   // hidden units of each of the first gu_split workgroups (those that hold the attention items of a short
+    int gu_split;   // context: they park nothing and own fewer units instead)
+    int park_rows;  // gate/up rows a workgroup from gu_split on keeps in LDS instead of streaming them (even; 0: none)
+    int park_floats;
+    int slice_dim;  // columns per slice of a dim-column row (slice_width)
     int down;   // rows of W2
     int cls;    // rows of the classifier
     int ns_dim, ns_hidden;  // partial sums per row of a dim-column / hidden-column matrix (slices_used)
@@ -115,6 +132,21 @@ struct Blocks {
     int results_floats;
     int gather_floats;
 };
+
+// Hidden units of a workgroup: a contiguous run, gu_a units for each of the first gu_split workgroups, gu for the rest.
+__host__ __device__ inline int gu_unit0(const Blocks& b, int wg) {
+    return wg < b.gu_split ? wg * b.gu_a : b.gu_split * b.gu_a + (wg - b.gu_split) * b.gu;
+}
+__host__ __device__ inline int gu_units(const Blocks& b, int hidden, int wg) {
+    const int block = wg < b.gu_split ? b.gu_a : b.gu;
+    const int n = hidden - gu_unit0(b, wg);
+    return n < 0 ? 0 : (n > block ? block : n);
+}
+// The last rows of the workgroup's gate/up block are the parked ones.
+__host__ __device__ inline int gu_parked_rows(const Blocks& b, int wg, int units) {
+    if (wg < b.gu_split) return 0;
+    return 2 * units < b.park_rows ? 2 * units : b.park_rows;
+}
 
 // Workgroup-local coordination words, accessed with relaxed workgroup-scope atomics
 // (plain ds_read / ds_write): LDS executes one wavefront's operations in order, so a
@@ -191,6 +223,7 @@ struct Ctx {
     int token, pos, history_len;
     float temperature, penalty, r;
     int wg, nwg;
+    int xcc, rank_in_xcc;  // the XCD this workgroup runs on and its index among that XCD's workgroups
 
     __device__ __forceinline__ unsigned seq(int layer, int phase) const {
         return base + 1u + 5u * static_cast<unsigned>(layer) + static_cast<unsigned>(phase);
@@ -628,6 +661,83 @@ __device__ __forceinline__ void poll_n(AddrFn addr, float (&out)[N], unsigned wa
     for (int j = 0; j < N; ++j) out[j] = value_of(got[j]);
 }
 
+// The XCD a wavefront runs on.
+__device__ __forceinline__ int hardware_xcc() {
+    unsigned v;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+    return static_cast<int>(v & 0xfu);
+}
+
+// A long vector every workgroup needs in full (the SwiGLU output), fetched in two hops.  Polled
+// directly, each of the 256 compute units pulls the whole vector across the fabric between the
+// XCDs, again for every attempt that comes too early: two megabytes per XCD and attempt at 8192
+// values.  Here the workgroups of an XCD share that work: workgroup r of the XCD polls slice r of the vector (device scope, as before) and stores it,
+// tags included, into a copy of the vector that belongs to its XCD; every workgroup then polls that
+// copy.  Those stores stay in the XCD's own L2 (plain stores; a device-scope store would write
+// through and drop the line), and the polls are non-temporal loads, which the compute unit's L1
+// does not keep: they are served by the L2 the stores went to.  Nothing outside the XCD ever
+// touches its copy, so the L2 needs no help to stay coherent.  A stale line anywhere can only
+// delay a poll (a value is taken when it carries the expected sequence number), not corrupt it.
+// Measured at the 1B shape: the down projection's inputs arrive 0.8 us sooner per layer; the
+// dim-sized vectors (2048 to 4096 values) gain nothing from the second hop and stay with direct polls.
+constexpr unsigned kNearPatience = 1024;  // polls of the near copy before a thread turns to the vector itself
+template <class Sink>
+__device__ __forceinline__ void gather_values(const u64* src, u64* near_all, int near_stride, int share, int n, unsigned want,
+                                              const Ctx& c, const Io& io, Sink sink) {
+    const int it = exchange_thread_index(io.iw);
+    u64* near = near_all + static_cast<size_t>(c.xcc) * near_stride;
+    for (int e = it; e < share; e += kIoThreads) {
+        const int i = c.rank_in_xcc * share + e;
+        if (i < n) {
+            u64 got;
+            unsigned spins = 0;
+            while (true) {
+                got = peek(src + i);
+                if (tag_of(got) == want) break;
+                if (poll_give_up(c, spins)) break;
+            }
+            asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(near + i), "v"(got) : "memory");
+        }
+    }
+    for (int first = it; first < n; first += 4 * kIoThreads) {
+        // (addresses past the end re-read the thread's first value; their results are dropped)
+        const u64* p0 = near + first;
+        const u64* p1 = near + (first + kIoThreads < n ? first + kIoThreads : first);
+        const u64* p2 = near + (first + 2 * kIoThreads < n ? first + 2 * kIoThreads : first);
+        const u64* p3 = near + (first + 3 * kIoThreads < n ? first + 3 * kIoThreads : first);
+        u64 g0, g1, g2, g3;
+        unsigned spins = 0;
+        while (true) {
+            if (spins <= kNearPatience) {
+                // (one statement, the wait included: the compiler sees the results only once they are in)
+                asm volatile(
+                    "global_load_dwordx2 %0, %4, off nt\n\t"
+                    "global_load_dwordx2 %1, %5, off nt\n\t"
+                    "global_load_dwordx2 %2, %6, off nt\n\t"
+                    "global_load_dwordx2 %3, %7, off nt\n\t"
+                    "s_waitcnt vmcnt(0)"
+                    : "=&v"(g0), "=&v"(g1), "=&v"(g2), "=&v"(g3)
+                    : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+                    : "memory");
+            } else {
+                // The near copy has not filled: should the workgroups ever not be spread over the XCDs the way the
+                // slices assume, the vector itself is still where it always was.
+                g0 = peek(src + (p0 - near));
+                g1 = peek(src + (p1 - near));
+                g2 = peek(src + (p2 - near));
+                g3 = peek(src + (p3 - near));
+            }
+            if (tag_of(g0) == want && tag_of(g1) == want && tag_of(g2) == want && tag_of(g3) == want) break;
+            if (poll_give_up(c, spins)) break;
+        }
+        const bool first_round = first == it;
+        sink(first, value_of(g0), 0, first_round);
+        if (first + kIoThreads < n) sink(first + kIoThreads, value_of(g1), 1, first_round);
+        if (first + 2 * kIoThreads < n) sink(first + 2 * kIoThreads, value_of(g2), 2, first_round);
+        if (first + 3 * kIoThreads < n) sink(first + 3 * kIoThreads, value_of(g3), 3, first_round);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Staging (exchange wavefronts)
 // ---------------------------------------------------------------------------
@@ -640,15 +750,21 @@ struct Lds {
     float* qkv;      // [kMaxAttHeads + 2][kMaxHeadPad] this token's q (per head of the item), k, v
     float* red;      // [kIoWaves][kMaxAttHeads][kRedStride] attention cross-wavefront reduction
     float* gather;   // [gather_floats] attention split partials
+    float* park;     // [park_floats] parked gate/up rows (binary16), row after row
 };
 
 // xs = the tagged vector itself, zero padded to a multiple of 8.  (The streaming
 // wavefronts are done with the previous contents: every exchange wavefront waited
 // for all of them before publishing.)
-__device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, int n, unsigned want) {
+// (near_all: the per-XCD copies of this vector, or nullptr for one that is polled directly)
+__device__ __forceinline__ void stage_tagged(Ctx& c, Io& io, float* xs, const u64* src, u64* near_all, int near_stride, int share,
+                                             int n, unsigned want) {
     const int n_pad = (n + 7) & ~7;
     for (int i = n + io.it; i < n_pad; i += kIoThreads) xs[i] = 0.0f;
-    poll_values<kPollBatch>(src, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });
+    if (near_all != nullptr && c.t.n_xcc > 1)
+        gather_values(src, near_all, near_stride, share, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });
+    else
+        poll_values<kPollBatch>(src, n, want, c, io, [&](int i, float v, int, bool) { xs[i] = v; });
     mark(c, io, 1);
     signal_received(c.ctl);
     signal_staged(c.ctl);
@@ -792,9 +908,10 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
 
 // x = xraw + W . src (model.cpp:160,218 and :225-226)
 __device__ __forceinline__ void io_proj(Ctx& c, Io& io, const Lds& l, int gphase, int block, int d, int nslices,
-                                        const u64* src, unsigned src_tag, unsigned out_tag) {
+                                        const u64* src, u64* near_all, int near_stride, int share, unsigned src_tag,
+                                        unsigned out_tag) {
     mark(c, io, 0);
-    stage_tagged(c, io, l.xs, src, d, src_tag);
+    stage_tagged(c, io, l.xs, src, near_all, near_stride, share, d, src_tag);
     mark(c, io, 2);
     const int row0 = c.wg * block;
     const int nrows = block_rows(c.a.dim, block, c.wg);
@@ -805,6 +922,98 @@ __device__ __forceinline__ void io_proj(Ctx& c, Io& io, const Lds& l, int gphase
     ++c.phase_index;
 }
 
+// Parked gate/up rows.  While the attention runs, most compute units have nothing to do and the memory
+// system is nearly idle, but the streaming wavefronts can only run as far ahead as their registers
+// reach.  A workgroup without an attention item therefore copies the last park_rows rows of its
+// gate/up block into LDS during that time (exchange wavefront w takes parked rows w, w + 8, ...), and
+// the same wavefront multiplies them out of LDS while the streaming wavefronts work through the rest
+// of the block: those rows are simply absent from the streaming wavefronts' lists.  The sums are formed
+// exactly as a streaming wavefront forms them (same lanes, same order), so a row gives the same bits
+// whichever way it went.  Once a context is long enough for the attention items to spread beyond the
+// first n_heads workgroups, the host launches with the other plan: no parked rows, uniform blocks.
+__device__ __forceinline__ void park_fetch(Ctx& c, Io& io, const Lds& l, int layer) {
+    const DecodeArgs& a = c.a;
+    const int units = gu_units(c.b, a.hidden, c.wg);
+    const int parked = gu_parked_rows(c.b, c.wg, units);
+    if (parked == 0) return;
+    const int first_row = 2 * units - parked;
+    const int unit0 = gu_unit0(c.b, c.wg);
+    const int lane = fresh_lane();
+    const int row_bytes = a.dim * 2;
+    const int loads_per_row = (row_bytes + 1023) >> 10;  // one wavefront load covers 1 KiB
+    const int mine = (parked - io.iw + kIoWaves - 1) / kIoWaves;
+    const int total = mine * loads_per_row;
+    constexpr int kBatch = 12;
+    char* park = reinterpret_cast<char*>(l.park);
+    for (int base = 0; base < total; base += kBatch) {
+        uintx4 v[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const int idx = base + i;
+            const int jj = idx / loads_per_row, chunk = idx - jj * loads_per_row;
+            const int j = io.iw + jj * kIoWaves;
+            const int r = first_row + j;
+            const int byte = (chunk << 10) + lane * 16;
+            v[i] = uintx4{0u, 0u, 0u, 0u};
+            if (idx < total && byte < row_bytes) {
+                const char* row = ((r & 1) ? a.w3 : a.w1) +
+                                  (static_cast<size_t>(layer) * a.hidden + unit0 + (r >> 1)) * static_cast<size_t>(row_bytes);
+                v[i] = load16_stream(row + byte);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const int idx = base + i;
+            const int jj = idx / loads_per_row, chunk = idx - jj * loads_per_row;
+            const int j = io.iw + jj * kIoWaves;
+            const int byte = (chunk << 10) + lane * 16;
+            if (idx < total && byte < row_bytes) *reinterpret_cast<uintx4*>(park + static_cast<size_t>(j) * row_bytes + byte) = v[i];
+        }
+    }
+}
+
+// results[row * ns_dim + slice] of the parked rows, from LDS: what a streaming wavefront computes for a step
+// (one chain of multiply-adds per 1-KiB chunk, added pairwise, then across the wavefront).
+__device__ __forceinline__ void park_multiply(Ctx& c, Io& io, const Lds& l) {
+    const DecodeArgs& a = c.a;
+    const int units = gu_units(c.b, a.hidden, c.wg);
+    const int parked = gu_parked_rows(c.b, c.wg, units);
+    if (parked == 0) return;
+    const int first_row = 2 * units - parked;
+    const int lane = fresh_lane();
+    const int row_bytes = a.dim * 2;
+    constexpr int kChunkCols = kWave * 8;
+    const char* park = reinterpret_cast<const char*>(l.park);
+    for (int s = 0; s < c.b.ns_dim; ++s) {
+        const int begin = s * c.b.slice_dim;
+        const int width = min(c.b.slice_dim, a.dim - begin);
+        floatx4 xr[kStepLoads][2];
+        const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int u = 0; u < kStepLoads; ++u) {
+            const int local = u * kChunkCols + lane * 8;
+            const bool live = local < width;
+            const float* src = l.xs + begin + (live ? local : 0);
+            xr[u][0] = *reinterpret_cast<const floatx4*>(src);
+            xr[u][1] = *reinterpret_cast<const floatx4*>(src + 4);
+            xr[u][0] = live ? xr[u][0] : zero;
+            xr[u][1] = live ? xr[u][1] : zero;
+        }
+        for (int j = io.iw; j < parked; j += kIoWaves) {
+            const char* row = park + static_cast<size_t>(j) * row_bytes + static_cast<size_t>(begin) * 2;
+            float part[kStepLoads];
+#pragma unroll
+            for (int u = 0; u < kStepLoads; ++u) {
+                const int local = u * kChunkCols + lane * 8;
+                const uintx4 w = *reinterpret_cast<const uintx4*>(row + static_cast<size_t>(local < width ? local : 0) * 2);
+                part[u] = dot8(w, xr[u][0], xr[u][1], 0.0f);
+            }
+            const float sum = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
+            if (lane == 0) l.results[(first_row + j) * c.b.ns_dim + s] = sum;
+        }
+    }
+}
+
 __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int layer) {
 #pragma clang fp contract(off)
     const DecodeArgs& a = c.a;
@@ -812,9 +1021,13 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
     const float scale =
         stage_norm(c, io, l, c.t.x, nullptr, a.dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * a.dim);
     mark(c, io, 2);
-    const int unit0 = c.wg * c.b.gu;
-    const int units = block_rows(a.hidden, c.b.gu, c.wg);
+    const int unit0 = gu_unit0(c.b, c.wg);
+    const int units = gu_units(c.b, a.hidden, c.wg);
     const unsigned tag = c.seq(layer, kGateUp);
+    if (c.b.park_rows > 0) {
+        park_multiply(c, io, l);
+        io_sync(c.ctl, io);  // the parked rows' sums are read by other exchange wavefronts below
+    }
     finished_rows(c, io, 4 * layer + kGGateUp, 2 * units, [&](int r) {
         if (r & 1) return;  // the gate row's thread finishes the unit
         const int u = r >> 1;
@@ -846,13 +1059,12 @@ __device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp
 // rescales them when the maximum grows; the groups' results are merged at the end, inside a
 // wavefront by lane exchange, across wavefronts through LDS (the same merge the splits undergo
 // later in att_combine).  model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped.
-template <int kGroup, int kHeads>
+template <int kGroup, int kHeads, int kRounds>
 __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int layer, int h0, int split, int nsplits,
                                                int npos, bool first_item, int hs) {
     static_assert(kHeads <= kMaxAttHeads, "LDS areas are sized for kMaxAttHeads heads");
     const DecodeArgs& a = c.a;
     constexpr int ngroups = kIoThreads / kGroup;
-    constexpr int kRounds = 2;
     constexpr int kSub = ngroups * kRounds;
     const int kvh = h0 / a.gqa;
     const int sub = io.it % kGroup, grp = io.it / kGroup;
@@ -1140,11 +1352,12 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
             const int chunk = item / nsplits, split = item - chunk * nsplits;
             const int h0 = chunk * heads_per_item;
             io.it = exchange_thread_index(io.iw);
-            if (hs <= 64) att_group_item<8, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
-            else att_group_item<16, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
+            if (hs <= 64) att_group_item<8, 2, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
+            else att_group_item<16, 2, 2>(c, io, l, layer, h0, split, nsplits, npos, first, hs);
             first = false;
         }
         if (first) idle_attention_received(c, io, layer);
+        park_fetch(c, io, l, layer);
         if (nsplits > 1) {
             // the heads of a chunk are combined by the workgroups that held its first splits
             for (int item = c.wg; item < items; item += c.nwg) {
@@ -1166,11 +1379,12 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
         const int h = item / nsplits, split = item - h * nsplits;
         io.it = exchange_thread_index(io.iw);
         // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
-        if (hs <= 64) att_group_item<8, 1>(c, io, l, layer, h, split, nsplits, npos, first, hs);
-        else att_group_item<16, 1>(c, io, l, layer, h, split, nsplits, npos, first, hs);
+        if (hs <= 64) att_group_item<8, 1, kShortRounds>(c, io, l, layer, h, split, nsplits, npos, first, hs);
+        else att_group_item<16, 1, kShortRounds>(c, io, l, layer, h, split, nsplits, npos, first, hs);
         first = false;
     }
     if (first) idle_attention_received(c, io, layer);
+    park_fetch(c, io, l, layer);
     if (nsplits > 1) {
         for (int item = c.wg; item < items; item += c.nwg) {
             const int h = item / nsplits, split = item - h * nsplits;
@@ -1382,12 +1596,13 @@ __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
         fresh();
         io_attention(c, io, l, layer);
         fresh();
-        io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.b.ns_dim, c.t.xb, c.seq(layer, kAtt), c.seq(layer, kOproj));
+        io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.b.ns_dim, c.t.xb, nullptr, 0, 0, c.seq(layer, kAtt),
+                c.seq(layer, kOproj));
         fresh();
         io_gateup(c, io, l, layer);
         fresh();
-        io_proj(c, io, l, 4 * layer + kGDown, c.b.down, a.hidden, c.b.ns_hidden, c.t.hb, c.seq(layer, kGateUp),
-                c.seq(layer, kDown));
+        io_proj(c, io, l, 4 * layer + kGDown, c.b.down, a.hidden, c.b.ns_hidden, c.t.hb, c.t.near_hb, c.t.near_hidden_stride,
+                c.t.share_hidden, c.seq(layer, kGateUp), c.seq(layer, kDown));
     }
     fresh();
     io_classify_sample(c, io, l);
@@ -1413,6 +1628,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.qkv = l.sc + 2 * kAttScoreFloats;
     l.red = l.qkv + (kMaxAttHeads + 2) * kMaxHeadPad;
     l.gather = l.red + kIoWaves * kMaxAttHeads * kRedStride;
+    l.park = l.gather + b.gather_floats;
     for (unsigned i = threadIdx.x; i < sizeof(Control) / sizeof(unsigned); i += blockDim.x)
         reinterpret_cast<unsigned*>(&ctl)[i] = 0u;
     __syncthreads();  // the only workgroup-wide barrier: the two kinds of wavefronts part ways here
@@ -1425,12 +1641,20 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
         const int token_in = min(max(__builtin_amdgcn_readfirstlane(a.step->token), 0), a.vocab - 1);
         unsigned long long* my_trace = nullptr;
         if (a.trace != nullptr && (wg == 0 || t.trace_stride > 0)) my_trace = a.trace + static_cast<size_t>(wg) * t.trace_stride;
+        // Workgroups go round the XCDs in turn (from wherever the launch before stopped): workgroups w, w + n_xcc,
+        // w + 2 n_xcc, ... share an XCD, which the hardware names, and w / n_xcc numbers them within it.
+        const int n_xcc = t.n_xcc > 1 ? t.n_xcc : 1;
         Ctx c{a, t, b, ctl, t.base, my_trace, 0u,
-              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg};
+              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg, hardware_xcc() % n_xcc, wg / n_xcc};
         Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
         if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
         io_role<kF16>(c, io, l);
     }
+}
+
+// Which XCD each workgroup of a launch of this shape lands on.
+__global__ void k_probe_xcc(int* out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = hardware_xcc();
 }
 
 }  // namespace df
@@ -1453,7 +1677,8 @@ struct Plan {
     size_t lds_bytes;
 };
 
-Plan plan_for(const lpp_model* m) {
+// parking: keep the last gate/up rows of most workgroups in LDS (short contexts); false: every row streams.
+Plan plan_for(const lpp_model* m, bool parking) {
     const lpp_config& c = m->cfg;
     Plan p;
     p.grid = compute_units();
@@ -1480,16 +1705,54 @@ Plan plan_for(const lpp_model* m) {
     if (b.cls * b.ns_dim > slots) slots = b.cls * b.ns_dim;
     b.results_floats = (slots + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
-    p.lds_bytes = static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
-                                      (df::kMaxAttHeads + 2) * df::kMaxHeadPad + df::kIoWaves * df::kMaxAttHeads * df::kRedStride +
-                                      b.gather_floats) * sizeof(float);
+    b.slice_dim = df::slice_width(c.dim, chunk_cols);
+    b.gu_a = b.gu;
+    b.gu_split = 0;
+    b.park_rows = 0;
+    b.park_floats = 0;
+    auto lds_floats = [&]() {
+        return static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
+                                   (df::kMaxAttHeads + 2) * df::kMaxHeadPad + df::kIoWaves * df::kMaxAttHeads * df::kRedStride +
+                                   b.gather_floats + b.park_floats);
+    };
+    // Parked gate/up rows: whatever LDS is left (binary16 models; the workgroups that hold the attention
+    // items of a short context, one per query head, park nothing and own that many fewer hidden units).
+    if (parking && c.weight_precision == LPP_WEIGHT_FP16 && c.n_heads < p.grid) {
+        constexpr size_t kLdsBytes = 160 * 1024, kReserve = 2048;  // the rest is for the kernel's static LDS
+        const size_t used = lds_floats() * sizeof(float);
+        const size_t row_bytes = static_cast<size_t>(c.dim) * 2;
+        int rows = used + kReserve < kLdsBytes ? static_cast<int>((kLdsBytes - kReserve - used) / row_bytes) : 0;
+        rows &= ~1;                                 // whole hidden units
+        const int cap = 4 * df::kIoWaves;           // a handful of rows per exchange wavefront is plenty
+        if (rows > cap) rows = cap;
+        // units of an ordinary workgroup if the first n_heads own rows / 2 fewer
+        const int gu = (c.hidden_dim + c.n_heads * (rows / 2) + p.grid - 1) / p.grid;
+        if (rows >= 2 && gu - rows / 2 >= 1 && 2 * gu - rows >= df::kGemvWaves) {
+            b.gu = gu;
+            b.gu_a = gu - rows / 2;
+            b.gu_split = c.n_heads;
+            b.park_rows = rows;
+            b.park_floats = static_cast<int>((static_cast<size_t>(rows) * row_bytes + 31) / 32 * 8);
+            if (2 * b.gu * b.ns_dim > slots) {
+                slots = 2 * b.gu * b.ns_dim;
+                b.results_floats = (slots + 7) & ~7;
+            }
+        }
+    }
+    p.lds_bytes = lds_floats() * sizeof(float);
     return p;
 }
+
+constexpr int kGridCap = 1024;  // workgroups the statistics table has room for
+constexpr int kMaxXcc = 8;
+// Tagged values of one XCD's copy of an n-value vector: whole 128-byte lines.
+size_t near_stride(int n) { return (static_cast<size_t>(n) + 15) / 16 * 16; }
 
 size_t tagged_count(const lpp_model* m, int grid_cap) {
     const lpp_config& c = m->cfg;
     return static_cast<size_t>(c.dim) * 3 + static_cast<size_t>(m->kv_dim) * 2 + c.hidden_dim +
-           static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2) + 4u * grid_cap;
+           static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2) + 4u * grid_cap +
+           16u + static_cast<size_t>(kMaxXcc) * near_stride(c.hidden_dim);
 }
 
 df::Tagged tagged_of(const lpp_model* m, bool generating) {
@@ -1503,7 +1766,16 @@ df::Tagged tagged_of(const lpp_model* m, bool generating) {
     t.xb = p;           p += c.dim;
     t.hb = p;           p += c.hidden_dim;
     t.part = p;         p += static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2);
-    t.stats = p;
+    t.stats = p;        p += 4u * kGridCap;
+    p = reinterpret_cast<df::u64*>((reinterpret_cast<uintptr_t>(p) + 127) & ~static_cast<uintptr_t>(127));
+    t.near_hidden_stride = static_cast<int>(near_stride(c.hidden_dim));
+    t.near_hb = p;
+    {
+        const int nwg = m->persist_grid > 0 ? m->persist_grid : compute_units();
+        t.n_xcc = (m->df_xcc > 1 && m->df_xcc <= kMaxXcc && nwg % m->df_xcc == 0) ? m->df_xcc : 1;
+        const int per_xcc = nwg / t.n_xcc;
+        t.share_hidden = (c.hidden_dim + per_xcc - 1) / per_xcc;
+    }
     t.splits_cap = splits_cap_for(m);
     t.hs_magic = static_cast<unsigned>((1ull << 32) / static_cast<unsigned long long>(m->head_size)) + 1u;
     t.pos = m->df_pos;
@@ -1528,13 +1800,11 @@ df::Tagged tagged_of(const lpp_model* m, bool generating) {
     return t;
 }
 
-constexpr int kGridCap = 1024;  // workgroups the statistics table has room for
-
 // Step lists of the streaming wavefronts: [workgroup][wavefront][stride]
 // entries.  After a wavefront's last step the list continues with entries
 // without kStepValid that point at a readable row: the wavefront requests up to
 // a ring of steps past its last one and reads whole batches of entries.
-lpp_status build_step_lists(lpp_model* m, const Plan& p) {
+lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
     const lpp_config& c = m->cfg;
     const df::Blocks& b = p.blocks;
     const int L = c.n_layers, dim = c.dim, hidden = c.hidden_dim, kv = m->kv_dim;
@@ -1553,11 +1823,16 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
         (void)j;
         return (nrows + share - 1) / share;  // an upper bound for every wavefront
     };
+    // gate/up rows of a workgroup that go through the streaming wavefronts: all but the parked ones at the block's end
+    auto gu_streamed = [&](int wg) {
+        const int units = df::gu_units(b, hidden, wg);
+        return 2 * units - df::gu_parked_rows(b, wg, units);
+    };
     int longest = 0;
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
             const int n = L * (own(block_rows(dim + 2 * kv, b.qkv, wg), dim, j) + own(block_rows(dim, b.o, wg), dim, j) +
-                               own(block_rows(2 * hidden, 2 * b.gu, wg), dim, j) +
+                               own(gu_streamed(wg), dim, j) +
                                own(block_rows(dim, b.down, wg), hidden, j)) +
                           own(block_rows(c.vocab_size, b.cls, wg), dim, j);
             if (n > longest) longest = n;
@@ -1568,6 +1843,8 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
     LPP_REQUIRE(b.results_floats <= static_cast<int>(df::kStepSlotMask) + 1 && dim < 65536 && hidden < 65536,
                 "persistent decode: shape too large for the step lists");
     std::vector<df::StepEntry> host(static_cast<size_t>(p.grid) * df::kGemvWaves * stride);
+    // columns of every matrix row the lists (and the parked rows) account for, keyed by the row's first byte
+    std::unordered_map<unsigned long long, int> covered;
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
             df::StepEntry* out = host.data() + (static_cast<size_t>(wg) * df::kGemvWaves + j) * stride;
@@ -1591,6 +1868,7 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
                     out[n].meta = static_cast<unsigned>(r * df::slices_used(d, chunk_cols) + slice) |
                                   (static_cast<unsigned>(phase) << df::kStepPhaseShift) | df::kStepValid;
                     out[n].cols = static_cast<unsigned>(begin) | (static_cast<unsigned>(exist) << 16);
+                    covered[row_address(r)] += exist;
                     ++n;
                 }
                 if (n > first) out[n - 1].meta |= df::kStepLastRow;
@@ -1605,8 +1883,9 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
                 phase_rows(4 * l + df::kGO, block_rows(dim, b.o, wg), dim,
                            [&](int r) { return base(LPP_T_WO) + (static_cast<size_t>(l) * dim + wg * b.o + r) * rb_dim; });
                 // local row 2u = gate row of hidden unit u, 2u + 1 = its up row
-                phase_rows(4 * l + df::kGGateUp, block_rows(2 * hidden, 2 * b.gu, wg), dim, [&](int r) {
-                    return base((r & 1) ? LPP_T_W3 : LPP_T_W1) + (static_cast<size_t>(l) * hidden + wg * b.gu + (r >> 1)) * rb_dim;
+                phase_rows(4 * l + df::kGGateUp, gu_streamed(wg), dim, [&](int r) {
+                    return base((r & 1) ? LPP_T_W3 : LPP_T_W1) +
+                           (static_cast<size_t>(l) * hidden + df::gu_unit0(b, wg) + (r >> 1)) * rb_dim;
                 });
                 phase_rows(4 * l + df::kGDown, block_rows(dim, b.down, wg), hidden, [&](int r) {
                     return base(LPP_T_W2) + (static_cast<size_t>(l) * dim + wg * b.down + r) * rb_hidden;
@@ -1620,14 +1899,40 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p) {
                 out[n].cols = 0;
             }
         }
-    lpp_free(m->df_rows);
-    m->df_rows = nullptr;
+    // Every column of every row must be multiplied exactly once per token: by a step, or as a parked row.
+    for (int wg = 0; wg < p.grid; ++wg) {
+        const int units = df::gu_units(b, hidden, wg), parked = df::gu_parked_rows(b, wg, units);
+        for (int l = 0; l < L; ++l)
+            for (int r = 2 * units - parked; r < 2 * units; ++r)
+                covered[base((r & 1) ? LPP_T_W3 : LPP_T_W1) + (static_cast<size_t>(l) * hidden + df::gu_unit0(b, wg) + (r >> 1)) * rb_dim] += dim;
+    }
+    {
+        const struct { int tensor; size_t rows; int cols; } all[] = {
+            {LPP_T_WQ, static_cast<size_t>(L) * dim, dim},       {LPP_T_WK, static_cast<size_t>(L) * kv, dim},
+            {LPP_T_WV, static_cast<size_t>(L) * kv, dim},        {LPP_T_WO, static_cast<size_t>(L) * dim, dim},
+            {LPP_T_W1, static_cast<size_t>(L) * hidden, dim},    {LPP_T_W3, static_cast<size_t>(L) * hidden, dim},
+            {LPP_T_W2, static_cast<size_t>(L) * dim, hidden},    {LPP_T_WCLS, static_cast<size_t>(c.vocab_size), dim}};
+        size_t expected = 0;
+        for (const auto& t : all) {
+            expected += t.rows;
+            for (size_t r = 0; r < t.rows; ++r) {
+                const auto it = covered.find(base(t.tensor) + r * static_cast<size_t>(t.cols) * wb);
+                if (it == covered.end() || it->second != t.cols)
+                    return fail(LPP_ERR_STATE, "persistent decode: step lists cover %d of %d columns of row %zu of tensor %d",
+                                it == covered.end() ? 0 : it->second, t.cols, r, t.tensor);
+            }
+        }
+        // (a tied classifier shares no rows with the other matrices: it is its own binary16 copy)
+        if (covered.size() != expected) return fail(LPP_ERR_STATE, "persistent decode: step lists name %zu rows, the model has %zu",
+                                                    covered.size(), expected);
+    }
+    lpp_free(m->df_rows[which]);
+    m->df_rows[which] = nullptr;
     void* d = nullptr;
     LPP_TRY(lpp_malloc(&d, host.size() * sizeof(df::StepEntry)));
-    m->df_rows = d;
-    m->df_row_stride = stride;
+    m->df_rows[which] = d;
+    m->df_row_stride[which] = stride;
     LPP_TRY(lpp_memcpy_h2d(d, host.data(), host.size() * sizeof(df::StepEntry)));
-    for (int t = 0; t < LPP_T_COUNT; ++t) m->df_rows_key[t] = m->w[t];
     return LPP_OK;
 }
 
@@ -1651,7 +1956,14 @@ const char* dataflow_unsupported_reason(const lpp_model* m) {
 template <bool kF16>
 static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
     if (const char* why = dataflow_unsupported_reason(m)) return fail(LPP_ERR_UNSUPPORTED, "%s", why);
-    const Plan p = plan_for(m);
+    // Two plans: with parked gate/up rows while only the first n_heads workgroups hold an attention item
+    // (one split per head), without them at longer contexts.  Each has its own step lists.
+    df::Tagged tagged = tagged_of(m, a.uniforms != nullptr);
+    static const bool parking_allowed = getenv("LPP_NO_PARKING") == nullptr;
+    const Plan parked_plan = plan_for(m, parking_allowed);
+    const bool use_parked = parked_plan.blocks.park_rows > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0;
+    const Plan p = use_parked ? parked_plan : plan_for(m, false);
+    const int which = use_parked ? 1 : 0;
     // Sequence numbers are compared for equality, so they must not come round to values that slots
     // written long ago (split partials of a longer context, say) may still hold: well before the
     // 32-bit count wraps, drain the stream, clear every tagged slot and start again from zero.
@@ -1660,31 +1972,68 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
         LPP_TRY(lpp_memset(m->tagged, 0, dataflow_tagged_bytes(m)));
         LPP_HIP(hipStreamSynchronize(s));
         m->df_base = 0;
+        tagged.base = 0;
     }
     if (m->persist_grid == 0) {
         LPP_REQUIRE(p.grid <= kGridCap, "persistent decode: %d compute units exceed the statistics table", p.grid);
         LPP_REQUIRE(m->head_size <= df::kMaxHeadPad, "persistent decode: head_size %d exceeds %d", m->head_size,
                     df::kMaxHeadPad);
+        const size_t lds_most = parked_plan.lds_bytes > p.lds_bytes ? parked_plan.lds_bytes : p.lds_bytes;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&df::k_decode_dataflow<kF16>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(p.lds_bytes)) != hipSuccess)
-            return fail(LPP_ERR_UNSUPPORTED, "persistent decode needs %zu bytes of LDS per workgroup", p.lds_bytes);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_most)) != hipSuccess)
+            return fail(LPP_ERR_UNSUPPORTED, "persistent decode needs %zu bytes of LDS per workgroup", lds_most);
         int per_cu = 0;
-        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, df::k_decode_dataflow<kF16>, df::kThreads,
-                                                              p.lds_bytes));
+        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, df::k_decode_dataflow<kF16>, df::kThreads, lds_most));
         if (per_cu < 1)
-            return fail(LPP_ERR_UNSUPPORTED, "persistent decode kernel does not fit a compute unit (LDS %zu bytes)",
-                        p.lds_bytes);
+            return fail(LPP_ERR_UNSUPPORTED, "persistent decode kernel does not fit a compute unit (LDS %zu bytes)", lds_most);
         m->persist_grid = p.grid;
     }
-    bool stale = m->df_rows == nullptr;
-    for (int t = 0; t < LPP_T_COUNT && !stale; ++t) stale = m->df_rows_key[t] != m->w[t];
-    if (stale) {
-        LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the old lists
-        LPP_TRY(build_step_lists(m, p));
+    if (m->df_xcc == 0) {
+        // Workgroups are handed to the XCDs in turn.  The near copies of gather_values rely on it, so it is
+        // measured, not assumed: anything but workgroup w on XCD (first + w) % n switches them off.
+        m->df_xcc = 1;
+        if (getenv("LPP_NO_XCD_LOCAL") == nullptr) {
+            void* d = nullptr;
+            LPP_TRY(lpp_malloc(&d, static_cast<size_t>(m->persist_grid) * sizeof(int)));
+            hipLaunchKernelGGL(df::k_probe_xcc, dim3(m->persist_grid), dim3(df::kThreads), 0, s, static_cast<int*>(d));
+            std::vector<int> where(m->persist_grid);
+            const hipError_t e = hipMemcpyAsync(where.data(), d, where.size() * sizeof(int), hipMemcpyDeviceToHost, s);
+            const hipError_t e2 = hipStreamSynchronize(s);
+            lpp_free(d);
+            LPP_HIP(e);
+            LPP_HIP(e2);
+            int n = 0;
+            for (int x : where) n = x + 1 > n ? x + 1 : n;
+            bool in_turn = n > 1 && n <= kMaxXcc && m->persist_grid % n == 0;
+            for (int w = 0; w < m->persist_grid && in_turn; ++w) in_turn = where[w] == (where[0] + w) % n;
+            if (in_turn) m->df_xcc = n;
+            if (getenv("LPP_DEBUG") != nullptr) {
+                for (int w = 0; w < 24 && w < m->persist_grid; ++w) fprintf(stderr, "%d ", where[w]);
+                fprintf(stderr, "\n");
+            }
+            if (getenv("LPP_DEBUG") != nullptr)
+                fprintf(stderr, "persistent decode: %d XCDs seen, workgroups %s; near copies %s\n", n,
+                        in_turn ? "in turn" : "not in turn", m->df_xcc > 1 ? "on" : "off");
+        }
+        tagged = tagged_of(m, a.uniforms != nullptr);
+        tagged.base = m->df_base;
     }
-    hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a,
-                       tagged_of(m, a.uniforms != nullptr), p.blocks, static_cast<const uint4*>(m->df_rows),
-                       m->df_row_stride);
+    bool moved = false;  // a weight tensor changed its address: both lists are stale
+    for (int t = 0; t < LPP_T_COUNT && !moved; ++t) moved = m->df_rows_key[t] != m->w[t];
+    if (moved) {
+        LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the old lists
+        for (int i = 0; i < 2; ++i) {
+            lpp_free(m->df_rows[i]);
+            m->df_rows[i] = nullptr;
+        }
+        for (int t = 0; t < LPP_T_COUNT; ++t) m->df_rows_key[t] = m->w[t];
+    }
+    // (both lists at once: a generation loop that grows past the short contexts must not stop to build the other one)
+    if (m->df_rows[which] == nullptr) LPP_TRY(build_step_lists(m, p, which));
+    if (parked_plan.blocks.park_rows > 0 && m->df_rows[1 - which] == nullptr)
+        LPP_TRY(build_step_lists(m, use_parked ? plan_for(m, false) : parked_plan, 1 - which));
+    hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a, tagged,
+                       p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
     LPP_CHECK_LAUNCH("k_decode_dataflow");
     m->df_base += df::phases_per_token(m->cfg.n_layers);
     if (!m->df_freeze) {  // what finish_token does to the device's record

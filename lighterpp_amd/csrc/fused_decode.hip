@@ -351,7 +351,8 @@ lpp_status fused_release(lpp_model* m) {
     lpp_free(m->sync_words);
     lpp_free(m->sample_scratch);
     lpp_free(m->tagged);
-    lpp_free(m->df_rows);
+    lpp_free(m->df_rows[0]);
+    lpp_free(m->df_rows[1]);
     lpp_free(m->gen_uniforms);
     return LPP_OK;
 }

@@ -54,8 +54,8 @@ struct lpp_model {
     float* gen_uniforms = nullptr;           // device copy of the per-step draws
     int gen_cap = 0;
     void* tagged = nullptr;                  // value+sequence-number vectors of the persistent kernel
-    void* df_rows = nullptr;                 // row lists of the persistent kernel's streaming wavefronts
-    int df_row_stride = 0;
+    void* df_rows[2] = {nullptr, nullptr};   // row lists of the persistent kernel's streaming wavefronts: [0] every row
+    int df_row_stride[2] = {0, 0};           // streamed, [1] with parked gate/up rows left out (short contexts)
     const void* df_rows_key[12] = {};        // weight addresses the lists were built from
     // Host's own count of the step record for the persistent path: everything but the token id
     // is known before a launch and travels as kernel arguments.
@@ -65,6 +65,7 @@ struct lpp_model {
     unsigned df_base = 0;                    // sequence-number base of the next persistent launch
     int df_trace_stride = 0;                 // timeline words per workgroup when every workgroup is traced (0: workgroup 0 only)
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
+    int df_xcc = 0;                          // XCDs the persistent kernel's workgroups go round (1: near copies off; 0: not probed)
     unsigned spin_limit = 1u << 20;          // polls a wait for tagged inputs may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
     int max_splits = 1;

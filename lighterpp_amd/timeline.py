@@ -75,6 +75,25 @@ def summarise(shape: Shape, t: np.ndarray, pos: int) -> dict:
         row["kind"] = KINDS[kind]
         row["floor"] = bytes_of[kind] / STREAM_CEILING * 1e6
         rows.append(row)
+    # attention work items (the workgroups that hold one): mark 0 entered, 5 q/k/v received, 2 shared through LDS,
+    # 7 context walked, 3 merged, 4 published
+    att = {k: [] for k in ("wait_inputs", "share", "walk", "merge", "publish")}
+    # GEMV phases, streaming wavefront 0 of every workgroup: mark 5 staged flag seen, 6 last row finished
+    gemv = {KINDS[k]: {"flag_after_staged": [], "last_row_after_flag": []} for k in (0, 2, 3, 4)}
+    for layer in range(1, L):
+        i = 5 * layer + 1
+        busy = ~np.isnan(t[:, i, 7])
+        if busy.any():
+            a = t[busy, i, :]
+            att["wait_inputs"].append(np.nanmedian(a[:, 5] - a[:, 0]))
+            att["share"].append(np.nanmedian(a[:, 2] - a[:, 5]))
+            att["walk"].append(np.nanmedian(a[:, 7] - a[:, 2]))
+            att["merge"].append(np.nanmedian(a[:, 3] - a[:, 7]))
+            att["publish"].append(np.nanmedian(a[:, 4] - a[:, 3]))
+        for k in (0, 2, 3, 4):
+            g = t[:, 5 * layer + k, :]
+            gemv[KINDS[k]]["flag_after_staged"].append(np.nanmedian(g[:, 5] - g[:, 2]))
+            gemv[KINDS[k]]["last_row_after_flag"].append(np.nanmedian(g[:, 6] - g[:, 5]))
     cls, smp = 5 * L, 5 * L + 1
     w = 2 if shape.fp16 else 4
     out = {
@@ -88,6 +107,9 @@ def summarise(shape: Shape, t: np.ndarray, pos: int) -> dict:
         "classifier_floor_us": w * shape.vocab_size * shape.dim / STREAM_CEILING * 1e6,
         "sampler_us": float(last_pub[smp] - last_pub[cls]),
         "token_us": float(last_pub[smp]),
+        "attention_item": {k: (float(np.mean(v)) if v else None) for k, v in att.items()},
+        "attention_workgroups": int(np.sum(~np.isnan(t[:, 6, 7]))) if L > 1 else 0,
+        "streaming_wavefront": {k: {kk: float(np.mean(vv)) for kk, vv in v.items()} for k, v in gemv.items()},
     }
     n_hand = 5 * L + 1
     total_floor = out["layer_floor_us"] * L + out["classifier_floor_us"]
@@ -104,6 +126,12 @@ def render(name: str, s: dict) -> str:
     for r in s["phases"]:
         lines.append(f"{r['kind']:10s} {fmt(r['span'])} {fmt(r['handover']):>10s} {fmt(r['stream'])} {fmt(r['epilogue']):>9s} "
                      f"{r['skew']:6.2f} {r['floor']:7.2f}")
+    a = s["attention_item"]
+    if a["walk"] is not None:
+        lines.append(f"attention item ({s['attention_workgroups']} workgroups hold one): inputs {a['wait_inputs']:.2f}, shared in LDS "
+                     f"{a['share']:.2f}, context walked {a['walk']:.2f}, merged {a['merge']:.2f}, published {a['publish']:.2f}")
+    lines.append("streaming wavefront 0 (after the exchange wavefronts' staged mark: flag seen, then last row done): " +
+                 "; ".join(f"{k} {v['flag_after_staged']:.2f} + {v['last_row_after_flag']:.2f}" for k, v in s["streaming_wavefront"].items()))
     lines.append(f"layer      {s['layer_us']:7.2f}   (weights of one layer at 7 TB/s: {s['layer_floor_us']:.2f})")
     lines.append(f"first layer {s['first_layer_us']:.2f}; classifier {s['classifier_us']:.2f} (floor {s['classifier_floor_us']:.2f}); "
                  f"sampler {s['sampler_us']:.2f}; token {s['token_us']:.2f}")
