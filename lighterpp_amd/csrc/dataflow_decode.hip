@@ -62,6 +62,12 @@ constexpr int kPollBatch = 8;                      // tagged values one thread r
 constexpr int kItemPositions = 1024;               // a one-head attention work item stays within twice this many positions
 constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS copy of the penalty window
 constexpr int kMaxHeadPad = 128;
+#ifndef LPP_IDLE_WAITS_FOR_Q
+#define LPP_IDLE_WAITS_FOR_Q 0
+#endif
+#ifndef LPP_PACED_STEPS
+#define LPP_PACED_STEPS 2
+#endif
 #ifndef LPP_SHORT_ROUNDS
 #define LPP_SHORT_ROUNDS 2
 #endif
@@ -316,22 +322,24 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     unsigned meta[kDepth];  // StepEntry::meta of the step held in w[k]
     unsigned cols[kDepth];  // StepEntry::cols
 
-    auto request = [&](int k, const uintx4& batch, int slot) {
-        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[0]), slot));
-        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[1]), slot));
-        const unsigned mt = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot));
-        const unsigned cl = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[3]), slot));
+    // The loads of the step whose first byte is lo | hi << 32 into ring slot k (cols[k] describes its slice).
+    auto request_at = [&](int k, unsigned lo, unsigned hi) {
         const GlobalBytes ptr =
             reinterpret_cast<GlobalBytes>(static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
-        const int width = static_cast<int>(cl >> 16);
+        const int width = static_cast<int>(cols[k] >> 16);
 #pragma unroll
         for (int u = 0; u < kStepLoads; ++u) {
             const int local = u * kChunkCols + lane * kPer;  // column inside the slice
             const int safe = (local < width) ? local : 0;    // lanes past the slice re-read its start; their activations are 0
             w[k][u] = __builtin_nontemporal_load(reinterpret_cast<GlobalVec>(ptr + static_cast<size_t>(safe) * kBytes));
         }
-        meta[k] = mt;
-        cols[k] = cl;
+    };
+    auto request = [&](int k, const uintx4& batch, int slot) {
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[0]), slot));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[1]), slot));
+        meta[k] = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[2]), slot));
+        cols[k] = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(batch[3]), slot));
+        request_at(k, lo, hi);
     };
 #pragma unroll
     for (int k = 0; k < kDepth; ++k) request(k, batch_a, k);
@@ -374,7 +382,9 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     // need multiplying would otherwise queue behind requests for later phases.
     unsigned ahead = 0u;  // bit k: the step in slot k has been multiplied already
     unsigned pace = 0u;
+    int paced = 0;  // next-phase rows sent out early since the last burst
     constexpr int kPaceSleep = 15;
+    constexpr int kPacedSteps = LPP_PACED_STEPS;
     auto run_round = [&](const uintx4& batch, int slot0) {
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) {
@@ -430,7 +440,10 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
                                 ended = ended || (m2 & kStepLastRow) != 0u;
                             }
                         }
-                        if (ended) pace |= burst;
+                        if (ended) {
+                            pace |= burst;
+                            paced = 0;
+                        }
                     }
                 }
                 ahead &= ~(1u << k);
@@ -440,7 +453,9 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
             if ((pace >> k) & 1u) {
                 // A refill after a burst that finished the wavefront's rows of phase cur_p.  A row of the
                 // very next GEMV phase goes out after a short pause, right behind the publishing stores
-                // (it must be there when that phase's inputs are).  Anything later is held until the inputs
+                // (it must be there when that phase's inputs are), and so does a second one; not more: where a
+                // wavefront's whole ring was one phase's rows, as at dim 4096, four refills of the next phase
+                // would put 128 KiB per compute unit in front of the polls.  Anything else is held until the inputs
                 // of the phase after this one have arrived: from then until that phase publishes, nothing
                 // of this workgroup's is on its way through the memory system, and a request costs no
                 // hand-over anything; sent now, it would sit in the queues in front of the values being
@@ -450,7 +465,8 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
                 const unsigned nq = (nm >> kStepPhaseShift) & kStepPhaseMask;
                 if ((nm & kStepValid) == 0u) {
                     // past the wavefront's last step: nothing left to hold back
-                } else if (nq == cur_p + 1u) {
+                } else if (nq == cur_p + 1u && paced < kPacedSteps) {
+                    ++paced;
                     __builtin_amdgcn_s_sleep(kPaceSleep);
                 } else {
                     // phases in the exchange wavefronts' count (five per layer): qkv, attention, O, gate/up, down
@@ -560,14 +576,11 @@ __device__ __forceinline__ void signal_received(Control& ctl) {
 // Wait until every streaming wavefront has completed GEMV phase p.
 __device__ __forceinline__ void wait_gemv(Control& ctl, int p) {
     const unsigned need = static_cast<unsigned>(p + 1);
-    static_assert(kGemvWaves == 8, "progress is read as two 16-byte vectors");
-    lds_wait(&ctl.error, [&]() {
-        compiler_fence();  // a fresh read every time round
-        const uint4 lo = *reinterpret_cast<const uint4*>(&ctl.progress[0]);
-        const uint4 hi = *reinterpret_cast<const uint4*>(&ctl.progress[4]);
-        const unsigned lowest = min(min(min(lo.x, lo.y), min(lo.z, lo.w)), min(min(hi.x, hi.y), min(hi.z, hi.w)));
-        return lowest >= need;
-    });
+    static_assert((kGemvWaves & (kGemvWaves - 1)) == 0, "lanes share the progress words by their low bits");
+    // One word per lane, one comparison per look: while the exchange wavefronts wait here the streaming
+    // wavefronts on the same SIMDs are multiplying, and every vector instruction of the wait is one they do not issue.
+    const unsigned* mine = &ctl.progress[fresh_lane() & (kGemvWaves - 1)];
+    lds_wait(&ctl.error, [&]() { return __builtin_amdgcn_ballot_w64(lds_ld(mine) < need) == 0ull; });
     compiler_fence();
 }
 
@@ -1306,10 +1319,13 @@ __host__ __device__ inline int item_splits(int npos, int cap, int n_heads, int n
 // q, k and v are out (one value stands for all: they are published within a microsecond of one
 // another), so that what those held back goes out while the items are computed, not before.
 __device__ __forceinline__ void idle_attention_received(Ctx& c, const Io& io, int layer) {
+#if LPP_IDLE_WAITS_FOR_Q
     float unused[1];
     const u64* one = c.t.q + (c.wg % c.a.dim);
     poll_n<1>([&](int) -> const u64* { return one; }, unused, c.seq(layer, kQkv), c);
+#endif
     (void)io;
+    (void)layer;
     signal_received(c.ctl);
 }
 
