@@ -38,6 +38,7 @@
 // finished reading the phase before the previous one.  Global polls are bounded:
 // a wavefront that gives up raises a shared abort flag that ends every other
 // poll, and no LDS wait depends on a global one, so the grid always drains.
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -111,6 +112,8 @@ struct Tagged {
     unsigned hs_magic;     // floor(2^32 / head_size) + 1: x / head_size == __umulhi(x, hs_magic) for x < 2^25
     int att_splits;        // context splits per query head at this position (worked out on the host: the search
     int att_group_splits;  // is a few dozen integer divisions); > 0: items cover two heads of a KV head, this many splits
+    float inv_sqrt_head;   // 1 / sqrt(head_size), formed on the host (on the device it would sit in a vector register all token long)
+    int lane_item_cap;     // contexts up to this many positions take the one-pass item of a head of size 64 (att_lane_item)
     // the step record, except the token id (which the previous launch left in device memory)
     int pos, history_len;
     float temperature, penalty, r;
@@ -1152,7 +1155,7 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
         cur_v = pv.u;
     }
 
-    const float scale = 1.0f / sqrtf(static_cast<float>(hs));  // model.cpp:188
+    const float scale = c.t.inv_sqrt_head;  // model.cpp:188
     float top[kHeads], lsum[kHeads], acc[kHeads][8];
 #pragma unroll
     for (int h = 0; h < kHeads; ++h) {
@@ -1265,6 +1268,241 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
                 publish(part + hs + 1, ls, tag_out);
             }
         }
+    }
+}
+
+// One query head of size 64 against a context of at most kIoWaves * 64 positions, no splits: the
+// whole context is on the compute unit before q arrives, and nothing is fetched after.  Exchange
+// wavefront w covers positions 64 w .. 64 w + 63.  Scores: a LANE holds one position's whole K row
+// (eight 16-byte pieces) and forms its dot product with q alone, so the softmax needs two
+// reductions across the wavefront and no other lane exchange.  Values: a lane holds two dimensions
+// of 32 positions (lanes 0..31 the wavefront's first 32 positions, lanes 32..63 the other 32: a
+// position's V row is one coalesced 128-byte load of half a wavefront), reads the weights the other
+// lanes formed back from LDS and adds up its two dimensions; the two halves meet in one lane
+// exchange.  The rows travel straight into LDS (global_load_lds: no register is held while q is
+// polled), piece i of every lane side by side, so each lane reads back exactly what it requested,
+// conflict-free; the room is the parked rows' area, which the workgroups that hold an item leave
+// empty, and the staged-activation area, idle between the QKV and the O projection.  The
+// wavefronts' partial results are merged as the lane groups' are in att_group_item.  Up to 512
+// positions this costs the same few hundred instructions whatever the position, where the item
+// above walks the context in passes of 128 positions, a memory round trip each.
+// model.cpp:186-198, ops.cpp:56-75.
+constexpr int kLaneItemPositions = kIoWaves * kWave;
+constexpr int kLaneBlockFloats = 2048;  // one wavefront's K rows, or its V rows: 64 positions x 64 binary16
+
+// Loads straight into LDS from one global address per lane: load I of a run reads SIZE bytes at address + GSTEP * I
+// and lands at lds + LSTEP * I + lane * SIZE.  (The instruction's immediate offset counts for both addresses: the LDS
+// base makes up the difference, so that one address register pair serves the whole run.  Spelled out with literal
+// offsets: the builtin takes integer constant expressions only, and not value-dependent ones.)
+#define LPP_LDS_LOAD(address, lds, SIZE, GSTEP, LSTEP, I) \
+    __builtin_amdgcn_global_load_lds(address, (__attribute__((address_space(3))) void*)((lds) + ((LSTEP) - (GSTEP)) * (I)), SIZE, (GSTEP) * (I), 0)
+#define LPP_LDS_LOAD4(address, lds, SIZE, GSTEP, LSTEP, I)   \
+    LPP_LDS_LOAD(address, lds, SIZE, GSTEP, LSTEP, (I));     \
+    LPP_LDS_LOAD(address, lds, SIZE, GSTEP, LSTEP, (I) + 1); \
+    LPP_LDS_LOAD(address, lds, SIZE, GSTEP, LSTEP, (I) + 2); \
+    LPP_LDS_LOAD(address, lds, SIZE, GSTEP, LSTEP, (I) + 3)
+
+// 8-KiB block b of the room described above.
+__device__ __forceinline__ float* lane_item_block(const Ctx& c, const Lds& l, int b) {
+    const int in_park = c.b.park_floats / kLaneBlockFloats;
+    return b < in_park ? l.park + b * kLaneBlockFloats : l.xs + (b - in_park) * kLaneBlockFloats;
+}
+
+// Does this workgroup hold a one-pass item (att_lane_item) in every layer of this token?  (One item per workgroup:
+// item h goes to workgroup h.)
+__device__ __forceinline__ bool lane_item_here(const Ctx& c) {
+    return c.a.head_size == 64 && c.t.att_splits == 1 && c.t.att_group_splits == 0 && c.pos + 1 <= c.t.lane_item_cap &&
+           c.wg < c.a.n_heads;
+}
+
+// The calling wavefront's K and V rows of head h in `layer` into its two LDS blocks.  Rows of positions the cache
+// does not hold yet (the current one, and what lies past the context) are fetched all the same where that saves a
+// branch, and never used.  (The host makes sure that every wavefront's 64 positions lie inside the cache's
+// seq_len.)  Fetching them a layer ahead, while the gate/up phase streams, was tried for the blocks in the parked
+// rows' area, which is free at any time: q then arrives 0.8 us sooner, but the compute unit finishes its gate/up
+// rows 3.5 us late, its share of the bandwidth being what it is.
+__device__ __forceinline__ void lane_item_fetch(const Ctx& c, const Io& io, const Lds& l, int layer, int h) {
+    typedef __attribute__((address_space(1))) const void* GlobalPtr;
+    const DecodeArgs& a = c.a;
+    constexpr int hs = 64;
+    const int npos = c.pos + 1;
+    const int t0 = io.iw * kWave;
+    if (t0 >= npos) return;
+    const int lane = fresh_lane();
+    const int half = lane >> 5, pair = lane & 31;
+    const int kvh = h / a.gqa;
+    const size_t head_base = (static_cast<size_t>(layer) * a.n_kv_heads + kvh) * a.seq_len * hs;
+    char* kbytes = reinterpret_cast<char*>(lane_item_block(c, l, 2 * io.iw));
+    char* vbytes = reinterpret_cast<char*>(lane_item_block(c, l, 2 * io.iw + 1));
+    const GlobalPtr krow = reinterpret_cast<GlobalPtr>(
+        reinterpret_cast<unsigned long long>(a.key_cache + head_base + static_cast<size_t>(t0 + lane) * hs));
+    LPP_LDS_LOAD4(krow, kbytes, 16, 16, 1024, 0);
+    LPP_LDS_LOAD4(krow, kbytes, 16, 16, 1024, 4);
+    const GlobalPtr vcol = reinterpret_cast<GlobalPtr>(reinterpret_cast<unsigned long long>(
+        reinterpret_cast<const char*>(a.value_cache + head_base + static_cast<size_t>(t0 + 32 * half) * hs) + 4 * pair));
+    // V rows four at a time, as far as the first half-wavefront's positions reach into the context
+    const int rows = min(32, npos - t0);
+    LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 0);
+    if (rows > 4) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 4); }
+    if (rows > 8) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 8); }
+    if (rows > 12) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 12); }
+    if (rows > 16) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 16); }
+    if (rows > 20) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 20); }
+    if (rows > 24) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 24); }
+    if (rows > 28) { LPP_LDS_LOAD4(vcol, vbytes, 4, 128, 256, 28); }
+}
+
+__device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int layer, int h, int npos) {
+    const DecodeArgs& a = c.a;
+    constexpr int hs = 64;
+    constexpr bool first_item = true;  // (one item per workgroup)
+    const int lane = fresh_lane();
+    const int kvh = h / a.gqa;
+    const int current = npos - 1;
+    const int t0 = io.iw * kWave, t = t0 + lane;
+    const bool wave_live = t0 < npos;  // (uniform)
+    const int half = lane >> 5, pair = lane & 31;
+    float* kblock = lane_item_block(c, l, 2 * io.iw);
+    float* vblock = lane_item_block(c, l, 2 * io.iw + 1);
+    lane_item_fetch(c, io, l, layer, h);
+
+    // q of the head, k and v of the current position: LDS row 0 holds q, rows 1 and 2 k and v as the cache will hold them
+    const unsigned tag_in = c.seq(layer, kQkv);
+    if (io.it < 3 * hs) {
+        const int which = io.it >> 6, e = io.it & 63;
+        const u64* src = which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
+                                    : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
+        float in[1];
+        poll_n<1>([&](int) -> const u64* { return src; }, in, tag_in, c);
+        l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[0] : f16_bits_to_f32(f32_to_f16_bits(in[0]));
+    }
+    if (first_item) {
+        mark(c, io, 5);
+        signal_received(c.ctl);
+    }
+    io_sync(c.ctl, io);
+    if (first_item) {
+        mark(c, io, 1);
+        mark(c, io, 6);
+        mark(c, io, 2);
+    }
+
+    float* red = l.red + (io.iw * kMaxAttHeads) * kRedStride;
+    float top = -INFINITY, lsum = 0.0f, o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+    if (wave_live) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows are in
+        if ((current >> 6) == io.iw) {
+            // The current position's k and v take their places among the fetched rows (what the fetch brought for
+            // that position is whatever the cache held before this token): from here on it is a position like any other.
+            const int slot = current - t0;
+            if (lane < 8) {  // lane i: piece i of the K row
+                union {
+                    half8_t h;
+                    uintx4 u;
+                } piece;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) piece.h[e] = static_cast<half_t>(l.qkv[kMaxHeadPad + 8 * lane + e]);
+                *reinterpret_cast<uintx4*>(kblock + 256 * lane + 4 * slot) = piece.u;
+            } else if (lane >= 32) {  // lane 32 + d: dimensions 2 d and 2 d + 1 of the V row
+                const int d = lane - 32;
+                const unsigned lo = f32_to_f16_bits(l.qkv[2 * kMaxHeadPad + 2 * d]), hi = f32_to_f16_bits(l.qkv[2 * kMaxHeadPad + 2 * d + 1]);
+                reinterpret_cast<unsigned*>(vblock)[64 * (slot & 31) + 32 * (slot >> 5) + d] = lo | (hi << 16);
+            }
+        }
+        // half a K row at a time: its four pieces and the matching half of q (every lane reads the same words of q)
+        // are all requested before the first multiply
+        float dot = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            __builtin_amdgcn_sched_barrier(0);
+            uintx4 kbits[4];
+            floatx4 qa[4], qb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                kbits[i] = *reinterpret_cast<const uintx4*>(kblock + 256 * (4 * r + i) + 4 * lane);
+                qa[i] = *reinterpret_cast<const floatx4*>(l.qkv + 8 * (4 * r + i));
+                qb[i] = *reinterpret_cast<const floatx4*>(l.qkv + 8 * (4 * r + i) + 4);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // (left alone, the scheduler pairs every read with its use: one LDS round trip per piece)
+            float part[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[i] = dot8(kbits[i], qa[i], qb[i], 0.0f);
+            dot += (part[0] + part[1]) + (part[2] + part[3]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const float score = t < npos ? dot * 0.125f : -INFINITY;  // 1 / sqrt(64), model.cpp:188
+        top = wave_max(score);
+        const float p = (score == -INFINITY) ? 0.0f : exp_fast(score - top);
+        lsum = wave_sum(p);
+        float* weights = l.sc + io.iw * kWave;  // this wavefront's 64 weights (LDS serves one wavefront's accesses in order)
+        weights[lane] = p;
+        const unsigned* vmine = reinterpret_cast<const unsigned*>(vblock) + lane;
+        const int rows = min(32, npos - t0);  // (what was fetched: lane_item_fetch)
+        // sixteen positions at a time: their values and weights are all requested before the first is used
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (16 * r < rows) {
+                unsigned bits[16];
+                floatx4 p4[4];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) bits[j] = vmine[64 * (16 * r + j)];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) p4[g] = *reinterpret_cast<const floatx4*>(weights + 32 * half + 16 * r + 4 * g);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int tv = t0 + 32 * half + 16 * r + j;
+                    // (what lies past the context may be anything, NaN included: its weight is zero, the value must be too)
+                    const unsigned b = tv < npos ? bits[j] : 0u;
+                    float& lo = (j & 1) ? o0 : o2;
+                    float& hi = (j & 1) ? o1 : o3;
+                    lo = fmaf(p4[j >> 2][j & 3], f16_bits_to_f32(static_cast<uint16_t>(b & 0xffffu)), lo);
+                    hi = fmaf(p4[j >> 2][j & 3], f16_bits_to_f32(static_cast<uint16_t>(b >> 16)), hi);
+                }
+            }
+        }
+        o0 += o2;
+        o1 += o3;
+        o0 += lane_xor(o0, 32, lane);
+        o1 += lane_xor(o1, 32, lane);
+    }
+    if (lane < 32) {
+        red[2 * pair] = o0;
+        red[2 * pair + 1] = o1;
+    }
+    if (lane == 0) {
+        red[kMaxHeadPad] = top;
+        red[kMaxHeadPad + 1] = lsum;
+    }
+    if (first_item) mark(c, io, 7);
+    io_sync(c.ctl, io);
+    if (first_item) mark(c, io, 3);
+    const unsigned tag_out = c.seq(layer, kAtt);
+    if (io.it < hs) {  // the wavefronts' partial results, through LDS: thread e
+        const int e = io.it;
+        // (all 24 words requested before the first is used: paired with their uses by the scheduler, they cost a
+        // round trip to LDS each)
+        float wtop[kIoWaves], wsum[kIoWaves], wout[kIoWaves];
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) {
+            const float* r = l.red + (w * kMaxAttHeads) * kRedStride;
+            wtop[w] = r[kMaxHeadPad];
+            wsum[w] = r[kMaxHeadPad + 1];
+            wout[w] = r[e];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) all = fmaxf(all, wtop[w]);
+        float o = 0.0f, ls = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) {
+            const float f = (wtop[w] == -INFINITY) ? 0.0f : exp_fast(wtop[w] - all);
+            o += wout[w] * f;
+            ls += wsum[w] * f;
+        }
+        publish(c.t.xb + static_cast<size_t>(h) * hs + e, o / ls, tag_out);
     }
 }
 
@@ -1395,7 +1633,8 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
         const int h = item / nsplits, split = item - h * nsplits;
         io.it = exchange_thread_index(io.iw);
         // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
-        if (hs <= 64) att_group_item<8, 1, kShortRounds>(c, io, l, layer, h, split, nsplits, npos, first, hs);
+        if (lane_item_here(c)) att_lane_item(c, io, l, layer, h, npos);
+        else if (hs <= 64) att_group_item<8, 1, kShortRounds>(c, io, l, layer, h, split, nsplits, npos, first, hs);
         else att_group_item<16, 1, kShortRounds>(c, io, l, layer, h, split, nsplits, npos, first, hs);
         first = false;
     }
@@ -1771,7 +2010,20 @@ size_t tagged_count(const lpp_model* m, int grid_cap) {
            16u + static_cast<size_t>(kMaxXcc) * near_stride(c.hidden_dim);
 }
 
-df::Tagged tagged_of(const lpp_model* m, bool generating) {
+// Positions a one-head attention item of a head of size 64 can keep on the compute unit (att_lane_item): two 8-KiB
+// blocks per 64 positions in the parked rows' area and the staged-activation area of plan p, whole blocks of 64
+// positions inside the cache; 0 where that item does not apply.
+int lane_item_positions(const lpp_model* m, const Plan& p) {
+    static const bool off = getenv("LPP_NO_LANE_ITEM") != nullptr;
+    if (off || m->head_size != 64 || m->cfg.n_heads > p.grid) return 0;
+    const int blocks = p.blocks.park_floats / df::kLaneBlockFloats + p.blocks.xs_floats / df::kLaneBlockFloats;
+    int cap = blocks / 2 * df::kWave;
+    if (cap > df::kLaneItemPositions) cap = df::kLaneItemPositions;
+    const int in_cache = m->cfg.seq_len / df::kWave * df::kWave;
+    return cap < in_cache ? cap : in_cache;
+}
+
+df::Tagged tagged_of(const lpp_model* m, bool generating, int lane_item_cap) {
     const lpp_config& c = m->cfg;
     df::Tagged t;
     df::u64* p = static_cast<df::u64*>(m->tagged);
@@ -1798,6 +2050,10 @@ df::Tagged tagged_of(const lpp_model* m, bool generating) {
     {
         const int npos = m->df_pos + 1, nwg = m->persist_grid > 0 ? m->persist_grid : compute_units();
         t.att_splits = df::item_splits(npos, t.splits_cap, c.n_heads, nwg);
+        // (a head of size 64 takes up to 512 positions in one item whose cost does not grow with the context)
+        t.inv_sqrt_head = 1.0f / sqrtf(static_cast<float>(m->head_size));
+        t.lane_item_cap = lane_item_cap;
+        if (npos <= t.lane_item_cap) t.att_splits = 1;
         t.att_group_splits = 0;
         if (m->gqa % 2 == 0 && t.att_splits > 1) {
             const int sub_positions = (m->head_size <= 64 ? df::kIoThreads / 8 : df::kIoThreads / 16) * 2;
@@ -1974,9 +2230,10 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     if (const char* why = dataflow_unsupported_reason(m)) return fail(LPP_ERR_UNSUPPORTED, "%s", why);
     // Two plans: with parked gate/up rows while only the first n_heads workgroups hold an attention item
     // (one split per head), without them at longer contexts.  Each has its own step lists.
-    df::Tagged tagged = tagged_of(m, a.uniforms != nullptr);
     static const bool parking_allowed = getenv("LPP_NO_PARKING") == nullptr;
     const Plan parked_plan = plan_for(m, parking_allowed);
+    const int lane_cap = lane_item_positions(m, parked_plan);
+    df::Tagged tagged = tagged_of(m, a.uniforms != nullptr, lane_cap);
     const bool use_parked = parked_plan.blocks.park_rows > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0;
     const Plan p = use_parked ? parked_plan : plan_for(m, false);
     const int which = use_parked ? 1 : 0;
@@ -2031,7 +2288,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
                 fprintf(stderr, "persistent decode: %d XCDs seen, workgroups %s; near copies %s\n", n,
                         in_turn ? "in turn" : "not in turn", m->df_xcc > 1 ? "on" : "off");
         }
-        tagged = tagged_of(m, a.uniforms != nullptr);
+        tagged = tagged_of(m, a.uniforms != nullptr, lane_cap);
         tagged.base = m->df_base;
     }
     bool moved = false;  // a weight tensor changed its address: both lists are stale
