@@ -93,6 +93,20 @@ __device__ __forceinline__ u64 peek(const u64* slot) {
     return __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The same inside one XCD: a plain store stays in the XCD's L2 (a device-scope one writes through and drops the line),
+// and a non-temporal load is not kept by the compute unit's L1, so it is served by that L2.  Only for slots that no
+// other XCD touches.
+__device__ __forceinline__ void publish_near(u64* slot, float v, unsigned tag) {
+    const u64 both = pack(v, tag);
+    asm volatile("global_store_dwordx2 %0, %1, off sc0" ::"v"(slot), "v"(both) : "memory");
+}
+__device__ __forceinline__ u64 peek_near(const u64* slot) {
+    u64 got;
+    // (one statement, the wait included: the compiler sees the result only once it is in)
+    asm volatile("global_load_dwordx2 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(got) : "v"(slot) : "memory");
+    return got;
+}
+
 // Tagged vectors of one model, all in one device allocation.
 struct Tagged {
     u64* x;      // [dim]     residual stream, written by the O and down projections
@@ -108,6 +122,13 @@ struct Tagged {
     int near_hidden_stride;  // tagged values per XCD
     int n_xcc;               // XCDs the workgroups go round in turn; 1: no near copies
     int share_hidden;        // values of hb each workgroup of an XCD fetches for the others
+    // Workgroup numbering by XCD: workgroup index = (ticket drawn from tickets[XCD] - ticket_base) * n_xcc + XCD.
+    unsigned* tickets;       // [n_xcc] counters, drawn once per workgroup and launch
+    unsigned ticket_base;    // what a counter read before this launch
+    // q, k and v handed to the attention items inside the XCD that formed them (near_qkv: [n_xcc][dim + 2 kv_dim])
+    u64* near_qkv;
+    int near_qkv_stride;
+    int local_qkv;           // nonzero: this token's q, k and v are published to near_qkv only
     int splits_cap;
     unsigned hs_magic;     // floor(2^32 / head_size) + 1: x / head_size == __umulhi(x, hs_magic) for x < 2^25
     int att_splits;        // context splits per query head at this position (worked out on the host: the search
@@ -132,6 +153,7 @@ struct Blocks {
     int gu_split;   // context: they park nothing and own fewer units instead)
     int park_rows;  // gate/up rows a workgroup from gu_split on keeps in LDS instead of streaming them (even; 0: none)
     int park_floats;
+    int qkv_by_xcc; // > 0: the stacked [Wq; Wk; Wv] rows are dealt out per XCD, this many KV heads (with their query heads) to each
     int slice_dim;  // columns per slice of a dim-column row (slice_width)
     int down;   // rows of W2
     int cls;    // rows of the classifier
@@ -155,6 +177,34 @@ __host__ __device__ inline int gu_units(const Blocks& b, int hidden, int wg) {
 __host__ __device__ inline int gu_parked_rows(const Blocks& b, int wg, int units) {
     if (wg < b.gu_split) return 0;
     return 2 * units < b.park_rows ? 2 * units : b.park_rows;
+}
+
+// Rows of the stacked [Wq; Wk; Wv] (dim + 2 kv_dim rows: q, then k, then v) a workgroup owns.  Plain: workgroup w
+// owns rows w * qkv .. w * qkv + qkv - 1.  By XCD (qkv_by_xcc > 0): XCD x owns the rows of KV heads x * qkv_by_xcc ..
+// and of the query heads that read them, listed per KV head as [its gqa query heads | its k rows | its v rows], and
+// the workgroups of the XCD share that list in blocks of qkv rows: everything an attention item needs of this token
+// is then formed on the XCD the item runs on.  qkv_rows() = how many of its block exist; qkv_row() = local row r as
+// an index into the stacked matrix.
+// (x = the workgroup's XCD, rank = its number within the XCD: wg % n_xcc and wg / n_xcc.)
+__host__ __device__ inline int qkv_rows(const Blocks& b, int dim, int kv_dim, int hs, int gqa, int wg, int rank) {
+    const int total = b.qkv_by_xcc > 0 ? b.qkv_by_xcc * (gqa + 2) * hs : dim + 2 * kv_dim;
+    const int first = (b.qkv_by_xcc > 0 ? rank : wg) * b.qkv;
+    const int n = total - first;
+    return n < 0 ? 0 : (n > b.qkv ? b.qkv : n);
+}
+__host__ __device__ inline int qkv_row(const Blocks& b, int dim, int kv_dim, int hs, int gqa, int wg, int x, int rank, int r) {
+    if (b.qkv_by_xcc <= 0) return wg * b.qkv + r;
+    const int listed = rank * b.qkv + r;
+    const int per_kv = (gqa + 2) * hs;
+    int j = 0, o = listed;
+    if (b.qkv_by_xcc > 1) {  // (the usual case, one KV head per XCD, needs no division)
+        j = listed / per_kv;
+        o = listed - j * per_kv;
+    }
+    const int kvh = x * b.qkv_by_xcc + j;
+    if (o < gqa * hs) return kvh * gqa * hs + o;
+    if (o < (gqa + 1) * hs) return dim + kvh * hs + (o - gqa * hs);
+    return dim + kv_dim + kvh * hs + (o - (gqa + 1) * hs);
 }
 
 // Workgroup-local coordination words, accessed with relaxed workgroup-scope atomics
@@ -677,6 +727,25 @@ __device__ __forceinline__ void poll_n(AddrFn addr, float (&out)[N], unsigned wa
     for (int j = 0; j < N; ++j) out[j] = value_of(got[j]);
 }
 
+// Two values per thread from slots inside this XCD's own copy (peek_near), both requested at once.
+template <class AddrFn>
+__device__ __forceinline__ void poll_near_2(AddrFn addr, float (&out)[2], unsigned want, const Ctx& c) {
+    const u64* p0 = addr(0);
+    const u64* p1 = addr(1);
+    u64 g0, g1;
+    unsigned spins = 0;
+    while (true) {
+        asm volatile("global_load_dwordx2 %0, %2, off nt\n\tglobal_load_dwordx2 %1, %3, off nt\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(g0), "=&v"(g1)
+                     : "v"(p0), "v"(p1)
+                     : "memory");
+        if (tag_of(g0) == want && tag_of(g1) == want) break;
+        if (poll_give_up(c, spins)) break;
+    }
+    out[0] = value_of(g0);
+    out[1] = value_of(g1);
+}
+
 // The XCD a wavefront runs on.
 __device__ __forceinline__ int hardware_xcc() {
     unsigned v;
@@ -874,14 +943,14 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     const float scale = stage_norm(c, io, l, c.t.x, emb_row, dim, layer == 0 ? 0u : c.seq(layer - 1, kDown),
                                    a.rms_att + static_cast<size_t>(layer) * dim);
     mark(c, io, 2);
-    const int row0 = c.wg * c.b.qkv;
-    const int nrows = block_rows(dim + 2 * kv_dim, c.b.qkv, c.wg);
+    const int nrows = qkv_rows(c.b, dim, kv_dim, hs, a.gqa, c.wg, c.rank_in_xcc);
     const float2* cs_row = a.rope + static_cast<size_t>(c.pos) * (hs / 2);
     const unsigned tag = c.seq(layer, kQkv);
     // (cos, sin) of this thread's first row: requested while the streaming wavefronts still multiply
     const int first_row = io.it;
-    const int first_g = row0 + first_row;
+    const int first_g = first_row < nrows ? qkv_row(c.b, dim, kv_dim, hs, a.gqa, c.wg, c.xcc, c.rank_in_xcc, first_row) : 0;
     const bool first_rotates = first_row < nrows && first_g < dim + kv_dim;
+    u64* near = c.t.local_qkv ? c.t.near_qkv + static_cast<size_t>(c.xcc) * c.t.near_qkv_stride : nullptr;
     // (a valid address either way, so that the request does not sit behind a branch)
     float first_cos, first_sin;
     pinned_load(cs_row + (first_rotates ? mod_hs(((first_g < dim) ? first_g : first_g - dim) & ~1) >> 1 : 0), first_cos, first_sin);
@@ -890,7 +959,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     wait_gemv(c.ctl, 4 * layer + kGQkv);
     mark(c, io, 3);
     for (int r = exchange_thread_index(io.iw); r < nrows; r += kIoThreads) {
-        const int g = row0 + r;
+        const int g = qkv_row(c.b, dim, kv_dim, hs, a.gqa, c.wg, c.xcc, c.rank_in_xcc, r);
         const float mine = row_result(l.results, r, c.b.ns_dim) * scale,
                     neighbour = row_result(l.results, r ^ 1, c.b.ns_dim) * scale;
         float out = mine;
@@ -904,8 +973,10 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
             }
             out = (gi & 1) ? neighbour * sin_t + mine * cos_t : mine * cos_t - neighbour * sin_t;
         }
+        // (to the attention items: across the chip, or inside this XCD when its items read nothing else)
+        if (near != nullptr) publish_near(near + g, out, tag);
         if (g < dim) {
-            publish(c.t.q + g, out, tag);
+            if (near == nullptr) publish(c.t.q + g, out, tag);
             a.q[g] = out;
         } else {  // model.cpp:171-176 / scatter_kv.cu:15-18
             const bool is_k = g < dim + kv_dim;
@@ -913,7 +984,7 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
             const int head = div_head_size(c, i), within = i - head * hs;
             const size_t dst = static_cast<size_t>(layer) * kv_dim * a.seq_len +
                                static_cast<size_t>(head) * a.seq_len * hs + static_cast<size_t>(c.pos) * hs + within;
-            publish((is_k ? c.t.k : c.t.v) + i, out, tag);
+            if (near == nullptr) publish((is_k ? c.t.k : c.t.v) + i, out, tag);
             (is_k ? a.k : a.v)[i] = out;
             (is_k ? a.key_cache : a.value_cache)[dst] = f32_to_f16_bits(out);
         }
@@ -1122,7 +1193,18 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
             };
             const int second = io.it + kIoThreads < wanted ? io.it + kIoThreads : io.it;
             float in[2];
-            poll_n<2>([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
+            if (c.t.local_qkv) {
+                // (the same slots in this XCD's copy: q, k and v stacked as their matrices are)
+                const u64* near = c.t.near_qkv + static_cast<size_t>(c.xcc) * c.t.near_qkv_stride;
+                auto near_source = [&](int idx) -> const u64* {
+                    const int which = div_head_size(c, idx), e = idx - which * hs;
+                    return near + (which < kHeads ? static_cast<size_t>(h0 + which) * hs + e
+                                                  : a.dim + (which == kHeads ? 0 : a.kv_dim) + static_cast<size_t>(kvh) * hs + e);
+                };
+                poll_near_2([&](int j) -> const u64* { return near_source(j == 0 ? io.it : second); }, in, tag_in, c);
+            } else {
+                poll_n<2>([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
+            }
             for (int j = 0; j < 2; ++j) {
                 const int idx = j == 0 ? io.it : second;
                 const int which = div_head_size(c, idx), e = idx - which * hs;
@@ -1368,19 +1450,71 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
 
     // q of the head, k and v of the current position: LDS row 0 holds q, rows 1 and 2 k and v as the cache will hold them
     const unsigned tag_in = c.seq(layer, kQkv);
-    if (io.it < 3 * hs) {
+    // Up to 64 positions the first wavefront does everything, fetching the three vectors itself: nothing is
+    // exchanged between wavefronts, so the two barriers and the merge below fall away.
+    const bool solo = npos <= kWave;  // (uniform)
+    if (solo) {
+        if (io.iw == 0) {
+            float in[3];
+            if (c.t.local_qkv) {
+                const u64* near = c.t.near_qkv + static_cast<size_t>(c.xcc) * c.t.near_qkv_stride;
+                const u64* p0 = near + static_cast<size_t>(h) * hs + lane;
+                const u64* p1 = near + a.dim + static_cast<size_t>(kvh) * hs + lane;
+                const u64* p2 = p1 + a.kv_dim;
+                u64 g0, g1, g2;
+                unsigned spins = 0;
+                while (true) {
+                    asm volatile(
+                        "global_load_dwordx2 %0, %3, off nt\n\tglobal_load_dwordx2 %1, %4, off nt\n\t"
+                        "global_load_dwordx2 %2, %5, off nt\n\ts_waitcnt vmcnt(0)"
+                        : "=&v"(g0), "=&v"(g1), "=&v"(g2)
+                        : "v"(p0), "v"(p1), "v"(p2)
+                        : "memory");
+                    if (tag_of(g0) == tag_in && tag_of(g1) == tag_in && tag_of(g2) == tag_in) break;
+                    if (poll_give_up(c, spins)) break;
+                }
+                in[0] = value_of(g0);
+                in[1] = value_of(g1);
+                in[2] = value_of(g2);
+            } else {
+                poll_n<3>(
+                    [&](int j) -> const u64* {
+                        return j == 0 ? c.t.q + static_cast<size_t>(h) * hs + lane
+                                      : (j == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + lane;
+                    },
+                    in, tag_in, c);
+            }
+            l.qkv[lane] = in[0];
+            l.qkv[kMaxHeadPad + lane] = f16_bits_to_f32(f32_to_f16_bits(in[1]));
+            l.qkv[2 * kMaxHeadPad + lane] = f16_bits_to_f32(f32_to_f16_bits(in[2]));
+        }
+    } else if (io.it < 3 * hs) {
         const int which = io.it >> 6, e = io.it & 63;
-        const u64* src = which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
-                                    : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
         float in[1];
-        poll_n<1>([&](int) -> const u64* { return src; }, in, tag_in, c);
+        if (c.t.local_qkv) {
+            const u64* src = c.t.near_qkv + static_cast<size_t>(c.xcc) * c.t.near_qkv_stride +
+                             (which == 0 ? static_cast<size_t>(h) * hs + e
+                                         : a.dim + (which == 1 ? 0 : a.kv_dim) + static_cast<size_t>(kvh) * hs + e);
+            u64 got;
+            unsigned spins = 0;
+            while (true) {
+                got = peek_near(src);
+                if (tag_of(got) == tag_in) break;
+                if (poll_give_up(c, spins)) break;
+            }
+            in[0] = value_of(got);
+        } else {
+            const u64* src = which == 0 ? c.t.q + static_cast<size_t>(h) * hs + e
+                                        : (which == 1 ? c.t.k : c.t.v) + static_cast<size_t>(kvh) * hs + e;
+            poll_n<1>([&](int) -> const u64* { return src; }, in, tag_in, c);
+        }
         l.qkv[which * kMaxHeadPad + e] = which == 0 ? in[0] : f16_bits_to_f32(f32_to_f16_bits(in[0]));
     }
     if (first_item) {
         mark(c, io, 5);
         signal_received(c.ctl);
     }
-    io_sync(c.ctl, io);
+    if (!solo) io_sync(c.ctl, io);
     if (first_item) {
         mark(c, io, 1);
         mark(c, io, 6);
@@ -1467,6 +1601,19 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
         o0 += lane_xor(o0, 32, lane);
         o1 += lane_xor(o1, 32, lane);
     }
+    const unsigned tag_out = c.seq(layer, kAtt);
+    if (solo) {
+        if (first_item) {
+            mark(c, io, 7);
+            mark(c, io, 3);
+        }
+        if (io.iw == 0 && lane < 32) {
+            u64* out = c.t.xb + static_cast<size_t>(h) * hs + 2 * pair;
+            publish(out, o0 / lsum, tag_out);
+            publish(out + 1, o1 / lsum, tag_out);
+        }
+        return;
+    }
     if (lane < 32) {
         red[2 * pair] = o0;
         red[2 * pair + 1] = o1;
@@ -1478,7 +1625,6 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
     if (first_item) mark(c, io, 7);
     io_sync(c.ctl, io);
     if (first_item) mark(c, io, 3);
-    const unsigned tag_out = c.seq(layer, kAtt);
     if (io.it < hs) {  // the wavefronts' partial results, through LDS: thread e
         const int e = io.it;
         // (all 24 words requested before the first is used: paired with their uses by the scheduler, they cost a
@@ -1628,9 +1774,13 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
     }
     int nsplits = c.t.att_splits;
     asm volatile("" : "+s"(nsplits));
-    const int items = a.n_heads * nsplits;
+    // One item per head and no splits, q, k and v handed over inside the XCD: the heads of the KV heads whose rows
+    // XCD x formed go to its first workgroups, in order.
+    const int heads_per_xcc = a.n_heads / (c.t.n_xcc > 1 ? c.t.n_xcc : 1);
+    const int items = c.t.local_qkv ? (c.rank_in_xcc < heads_per_xcc ? c.wg + 1 : 0) : a.n_heads * nsplits;
     for (int item = c.wg; item < items; item += c.nwg) {
-        const int h = item / nsplits, split = item - h * nsplits;
+        const int h = c.t.local_qkv ? c.xcc * heads_per_xcc + c.rank_in_xcc : item / nsplits;
+        const int split = c.t.local_qkv ? 0 : item - h * nsplits;
         io.it = exchange_thread_index(io.iw);
         // lane groups of 8 cover head sizes up to 64 (lanes past the head idle), groups of 16 up to 128
         if (lane_item_here(c)) att_lane_item(c, io, l, layer, h, npos);
@@ -1873,7 +2023,26 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
                                                               const uint4* __restrict__ row_lists, int row_list_stride) {
     extern __shared__ __align__(16) float lds[];
     __shared__ Control ctl;
-    const int wg = blockIdx.x, nwg = gridDim.x;
+    __shared__ int numbered;
+    const int nwg = gridDim.x;
+    // Workgroups are numbered by where they run: XCD + n_xcc * (the order in which the XCD's workgroups got here).
+    // Which rows, attention items and slices a workgroup owns then says which XCD's L2 they pass through, whatever
+    // the order in which the hardware handed the workgroups out.  An XCD that does not get its share of the
+    // workgroups (they are handed out in turn: it always has) ends the launch with an error.
+    if (threadIdx.x == 0) {
+        int number = blockIdx.x;
+        if (t.n_xcc > 1) {
+            const int x = hardware_xcc() % t.n_xcc;
+            const unsigned order = __hip_atomic_fetch_add(t.tickets + x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - t.ticket_base;
+            if (order < static_cast<unsigned>(nwg / t.n_xcc)) {
+                number = static_cast<int>(order) * t.n_xcc + x;
+            } else {
+                __hip_atomic_store(t.abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                a.step->error = 3;
+            }
+        }
+        numbered = number;
+    }
     const int dim_pad = (a.dim + 7) & ~7;
     Lds l;
     l.xraw = lds;
@@ -1887,6 +2056,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     for (unsigned i = threadIdx.x; i < sizeof(Control) / sizeof(unsigned); i += blockDim.x)
         reinterpret_cast<unsigned*>(&ctl)[i] = 0u;
     __syncthreads();  // the only workgroup-wide barrier: the two kinds of wavefronts part ways here
+    const int wg = __builtin_amdgcn_readfirstlane(numbered);
     const int wave = wave_index();
     if (wave < kGemvWaves) {
         gemv_role<kF16>(a, ctl, row_lists + static_cast<size_t>(wg * kGemvWaves + wave) * row_list_stride, wave, l.xs,
@@ -1896,11 +2066,9 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
         const int token_in = min(max(__builtin_amdgcn_readfirstlane(a.step->token), 0), a.vocab - 1);
         unsigned long long* my_trace = nullptr;
         if (a.trace != nullptr && (wg == 0 || t.trace_stride > 0)) my_trace = a.trace + static_cast<size_t>(wg) * t.trace_stride;
-        // Workgroups go round the XCDs in turn (from wherever the launch before stopped): workgroups w, w + n_xcc,
-        // w + 2 n_xcc, ... share an XCD, which the hardware names, and w / n_xcc numbers them within it.
         const int n_xcc = t.n_xcc > 1 ? t.n_xcc : 1;
         Ctx c{a, t, b, ctl, t.base, my_trace, 0u,
-              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg, hardware_xcc() % n_xcc, wg / n_xcc};
+              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg, wg % n_xcc, wg / n_xcc};
         Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
         if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
         io_role<kF16>(c, io, l);
@@ -1940,6 +2108,17 @@ Plan plan_for(const lpp_model* m, bool parking) {
     auto per = [&](int total) { return (total + p.grid - 1) / p.grid; };
     df::Blocks& b = p.blocks;
     b.qkv = (per(c.dim + 2 * m->kv_dim) + 1) & ~1;  // RoPE pairs stay inside one workgroup
+    b.qkv_by_xcc = 0;
+    {
+        // Per XCD where the KV heads divide among the XCDs (qkv_row): whole KV heads with their query heads.
+        static const bool allowed = getenv("LPP_NO_XCD_QKV") == nullptr;
+        const int n = m->df_xcc;
+        if (allowed && n > 1 && c.n_kv_heads % n == 0 && p.grid % n == 0 && c.n_heads / n <= p.grid / n) {
+            const int rows = (c.dim + 2 * m->kv_dim) / n, wgs = p.grid / n;
+            b.qkv_by_xcc = c.n_kv_heads / n;
+            b.qkv = ((rows + wgs - 1) / wgs + 1) & ~1;
+        }
+    }
     b.o = per(c.dim);
     b.gu = per(c.hidden_dim);
     b.down = per(c.dim);
@@ -1978,7 +2157,8 @@ Plan plan_for(const lpp_model* m, bool parking) {
         const size_t row_bytes = static_cast<size_t>(c.dim) * 2;
         int rows = used + kReserve < kLdsBytes ? static_cast<int>((kLdsBytes - kReserve - used) / row_bytes) : 0;
         rows &= ~1;                                 // whole hidden units
-        const int cap = 4 * df::kIoWaves;           // a handful of rows per exchange wavefront is plenty
+        static const int env_cap = getenv("LPP_PARK_ROWS") ? atoi(getenv("LPP_PARK_ROWS")) : 0;
+        const int cap = env_cap > 0 ? env_cap : 4 * df::kIoWaves;  // a handful of rows per exchange wavefront is plenty
         if (rows > cap) rows = cap;
         // units of an ordinary workgroup if the first n_heads own rows / 2 fewer
         const int gu = (c.hidden_dim + c.n_heads * (rows / 2) + p.grid - 1) / p.grid;
@@ -2007,7 +2187,7 @@ size_t tagged_count(const lpp_model* m, int grid_cap) {
     const lpp_config& c = m->cfg;
     return static_cast<size_t>(c.dim) * 3 + static_cast<size_t>(m->kv_dim) * 2 + c.hidden_dim +
            static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2) + 4u * grid_cap +
-           16u + static_cast<size_t>(kMaxXcc) * near_stride(c.hidden_dim);
+           32u + static_cast<size_t>(kMaxXcc) * (near_stride(c.hidden_dim) + near_stride(c.dim + 2 * m->kv_dim));
 }
 
 // Positions a one-head attention item of a head of size 64 can keep on the compute unit (att_lane_item): two 8-KiB
@@ -2037,7 +2217,11 @@ df::Tagged tagged_of(const lpp_model* m, bool generating, int lane_item_cap) {
     t.stats = p;        p += 4u * kGridCap;
     p = reinterpret_cast<df::u64*>((reinterpret_cast<uintptr_t>(p) + 127) & ~static_cast<uintptr_t>(127));
     t.near_hidden_stride = static_cast<int>(near_stride(c.hidden_dim));
-    t.near_hb = p;
+    t.near_hb = p;      p += static_cast<size_t>(kMaxXcc) * t.near_hidden_stride;
+    t.near_qkv_stride = static_cast<int>(near_stride(c.dim + 2 * m->kv_dim));
+    t.near_qkv = p;
+    t.tickets = m->sync_words + 96;
+    t.ticket_base = m->df_ticket_base;
     {
         const int nwg = m->persist_grid > 0 ? m->persist_grid : compute_units();
         t.n_xcc = (m->df_xcc > 1 && m->df_xcc <= kMaxXcc && nwg % m->df_xcc == 0) ? m->df_xcc : 1;
@@ -2054,6 +2238,7 @@ df::Tagged tagged_of(const lpp_model* m, bool generating, int lane_item_cap) {
         t.inv_sqrt_head = 1.0f / sqrtf(static_cast<float>(m->head_size));
         t.lane_item_cap = lane_item_cap;
         if (npos <= t.lane_item_cap) t.att_splits = 1;
+        t.local_qkv = 0;  // (set by the launch once the plan is chosen)
         t.att_group_splits = 0;
         if (m->gqa % 2 == 0 && t.att_splits > 1) {
             const int sub_positions = (m->head_size <= 64 ? df::kIoThreads / 8 : df::kIoThreads / 16) * 2;
@@ -2083,6 +2268,7 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
     const size_t wb = c.weight_precision == LPP_WEIGHT_FP16 ? 2 : 4;
     const int chunk_cols = static_cast<int>(1024 / wb);
     const size_t rb_dim = static_cast<size_t>(dim) * wb, rb_hidden = static_cast<size_t>(hidden) * wb;
+    const int n_xcc = m->df_xcc > 1 ? m->df_xcc : 1;
     auto base = [&](int t) { return reinterpret_cast<unsigned long long>(m->w[t]); };
     auto block_rows = [](int total, int block, int wg) {
         const int n = total - wg * block;
@@ -2103,7 +2289,7 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
     int longest = 0;
     for (int wg = 0; wg < p.grid; ++wg)
         for (int j = 0; j < df::kGemvWaves; ++j) {
-            const int n = L * (own(block_rows(dim + 2 * kv, b.qkv, wg), dim, j) + own(block_rows(dim, b.o, wg), dim, j) +
+            const int n = L * (own(df::qkv_rows(b, dim, kv, m->head_size, m->gqa, wg, wg / n_xcc), dim, j) + own(block_rows(dim, b.o, wg), dim, j) +
                                own(gu_streamed(wg), dim, j) +
                                own(block_rows(dim, b.down, wg), hidden, j)) +
                           own(block_rows(c.vocab_size, b.cls, wg), dim, j);
@@ -2146,8 +2332,8 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
                 if (n > first) out[n - 1].meta |= df::kStepLastRow;
             };
             for (int l = 0; l < L; ++l) {
-                phase_rows(4 * l + df::kGQkv, block_rows(dim + 2 * kv, b.qkv, wg), dim, [&](int r) {
-                    const int g = wg * b.qkv + r;
+                phase_rows(4 * l + df::kGQkv, df::qkv_rows(b, dim, kv, m->head_size, m->gqa, wg, wg / n_xcc), dim, [&](int r) {
+                    const int g = df::qkv_row(b, dim, kv, m->head_size, m->gqa, wg, wg % n_xcc, wg / n_xcc, r);
                     if (g < dim) return base(LPP_T_WQ) + (static_cast<size_t>(l) * dim + g) * rb_dim;
                     if (g < dim + kv) return base(LPP_T_WK) + (static_cast<size_t>(l) * kv + (g - dim)) * rb_dim;
                     return base(LPP_T_WV) + (static_cast<size_t>(l) * kv + (g - dim - kv)) * rb_dim;
@@ -2228,6 +2414,31 @@ const char* dataflow_unsupported_reason(const lpp_model* m) {
 template <bool kF16>
 static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
     if (const char* why = dataflow_unsupported_reason(m)) return fail(LPP_ERR_UNSUPPORTED, "%s", why);
+    if (m->df_xcc == 0) {
+        // Workgroups are handed to the XCDs in turn.  The per-XCD hand-overs rely on every XCD getting an equal share
+        // of them, so it is measured, not assumed: anything but workgroup w on XCD (first + w) % n switches them off.
+        m->df_xcc = 1;
+        if (getenv("LPP_NO_XCD_LOCAL") == nullptr) {
+            const int grid = compute_units();
+            void* d = nullptr;
+            LPP_TRY(lpp_malloc(&d, static_cast<size_t>(grid) * sizeof(int)));
+            hipLaunchKernelGGL(df::k_probe_xcc, dim3(grid), dim3(df::kThreads), 0, s, static_cast<int*>(d));
+            std::vector<int> where(grid);
+            const hipError_t e = hipMemcpyAsync(where.data(), d, where.size() * sizeof(int), hipMemcpyDeviceToHost, s);
+            const hipError_t e2 = hipStreamSynchronize(s);
+            lpp_free(d);
+            LPP_HIP(e);
+            LPP_HIP(e2);
+            int n = 0;
+            for (int x : where) n = x + 1 > n ? x + 1 : n;
+            bool in_turn = n > 1 && n <= kMaxXcc && grid % n == 0;
+            for (int w = 0; w < grid && in_turn; ++w) in_turn = where[w] == (where[0] + w) % n;
+            if (in_turn) m->df_xcc = n;
+            if (getenv("LPP_DEBUG") != nullptr)
+                fprintf(stderr, "persistent decode: %d XCDs seen, workgroups %s; per-XCD hand-overs %s\n", n,
+                        in_turn ? "in turn" : "not in turn", m->df_xcc > 1 ? "on" : "off");
+        }
+    }
     // Two plans: with parked gate/up rows while only the first n_heads workgroups hold an attention item
     // (one split per head), without them at longer contexts.  Each has its own step lists.
     static const bool parking_allowed = getenv("LPP_NO_PARKING") == nullptr;
@@ -2237,6 +2448,8 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     const bool use_parked = parked_plan.blocks.park_rows > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0;
     const Plan p = use_parked ? parked_plan : plan_for(m, false);
     const int which = use_parked ? 1 : 0;
+    // q, k and v stay inside the XCD that formed them while every head's item sits on that XCD: one item per head
+    tagged.local_qkv = (p.blocks.qkv_by_xcc > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0) ? 1 : 0;
     // Sequence numbers are compared for equality, so they must not come round to values that slots
     // written long ago (split partials of a longer context, say) may still hold: well before the
     // 32-bit count wraps, drain the stream, clear every tagged slot and start again from zero.
@@ -2261,36 +2474,6 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
             return fail(LPP_ERR_UNSUPPORTED, "persistent decode kernel does not fit a compute unit (LDS %zu bytes)", lds_most);
         m->persist_grid = p.grid;
     }
-    if (m->df_xcc == 0) {
-        // Workgroups are handed to the XCDs in turn.  The near copies of gather_values rely on it, so it is
-        // measured, not assumed: anything but workgroup w on XCD (first + w) % n switches them off.
-        m->df_xcc = 1;
-        if (getenv("LPP_NO_XCD_LOCAL") == nullptr) {
-            void* d = nullptr;
-            LPP_TRY(lpp_malloc(&d, static_cast<size_t>(m->persist_grid) * sizeof(int)));
-            hipLaunchKernelGGL(df::k_probe_xcc, dim3(m->persist_grid), dim3(df::kThreads), 0, s, static_cast<int*>(d));
-            std::vector<int> where(m->persist_grid);
-            const hipError_t e = hipMemcpyAsync(where.data(), d, where.size() * sizeof(int), hipMemcpyDeviceToHost, s);
-            const hipError_t e2 = hipStreamSynchronize(s);
-            lpp_free(d);
-            LPP_HIP(e);
-            LPP_HIP(e2);
-            int n = 0;
-            for (int x : where) n = x + 1 > n ? x + 1 : n;
-            bool in_turn = n > 1 && n <= kMaxXcc && m->persist_grid % n == 0;
-            for (int w = 0; w < m->persist_grid && in_turn; ++w) in_turn = where[w] == (where[0] + w) % n;
-            if (in_turn) m->df_xcc = n;
-            if (getenv("LPP_DEBUG") != nullptr) {
-                for (int w = 0; w < 24 && w < m->persist_grid; ++w) fprintf(stderr, "%d ", where[w]);
-                fprintf(stderr, "\n");
-            }
-            if (getenv("LPP_DEBUG") != nullptr)
-                fprintf(stderr, "persistent decode: %d XCDs seen, workgroups %s; near copies %s\n", n,
-                        in_turn ? "in turn" : "not in turn", m->df_xcc > 1 ? "on" : "off");
-        }
-        tagged = tagged_of(m, a.uniforms != nullptr, lane_cap);
-        tagged.base = m->df_base;
-    }
     bool moved = false;  // a weight tensor changed its address: both lists are stale
     for (int t = 0; t < LPP_T_COUNT && !moved; ++t) moved = m->df_rows_key[t] != m->w[t];
     if (moved) {
@@ -2309,6 +2492,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
                        p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
     LPP_CHECK_LAUNCH("k_decode_dataflow");
     m->df_base += df::phases_per_token(m->cfg.n_layers);
+    if (tagged.n_xcc > 1) m->df_ticket_base += static_cast<unsigned>(m->persist_grid / tagged.n_xcc);  // one ticket per workgroup
     if (!m->df_freeze) {  // what finish_token does to the device's record
         if (m->df_history_cap > 0 && m->df_history_len < m->df_history_cap) m->df_history_len += 1;
         m->df_pos += 1;
@@ -2319,6 +2503,21 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
 
 lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
     return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? launch_impl<true>(m, a, s) : launch_impl<false>(m, a, s);
+}
+
+// What a launch left in StepParams::error, as a status.  Code 3 (an XCD did not get its share of the workgroups)
+// also switches the per-XCD hand-overs off for this model: the next launch runs without them.
+lpp_status dataflow_report_error(lpp_model* m, int code) {
+    if (code == 0) return LPP_OK;
+    if (code == 3) {
+        m->df_xcc = 1;
+        for (int i = 0; i < 2; ++i) {  // the step lists were dealt out per XCD
+            lpp_free(m->df_rows[i]);
+            m->df_rows[i] = nullptr;
+        }
+        return fail(LPP_ERR_HIP, "decode kernel: workgroups unevenly spread over the XCDs; per-XCD hand-overs switched off");
+    }
+    return fail(LPP_ERR_HIP, "decode kernel gave up waiting for its inputs");
 }
 
 unsigned dataflow_phases_per_token(int n_layers) { return df::phases_per_token(n_layers); }

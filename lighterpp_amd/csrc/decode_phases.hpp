@@ -868,5 +868,6 @@ size_t dataflow_tagged_bytes(const lpp_model* m);
 lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s);
 unsigned dataflow_phases_per_token(int n_layers);
 unsigned dataflow_trace_marks();
+lpp_status dataflow_report_error(lpp_model* m, int code);
 
 }  // namespace lpp

@@ -403,7 +403,7 @@ lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, fl
     LPP_HIP(hipStreamSynchronize(s));
     if (m->path == LPP_PATH_PERSISTENT) {
         LPP_HIP(hipMemcpy(m->step_host, m->step, sizeof(StepParams), hipMemcpyDeviceToHost));
-        if (m->step_host->error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up waiting for its inputs");
+        if (m->step_host->error != 0) return dataflow_report_error(m, m->step_host->error);
     }
     return LPP_OK;
 }
@@ -463,7 +463,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     // Hand the penalty window back in the reference's order (oldest first).
     StepParams done{};
     LPP_HIP(hipMemcpy(&done, m->step, sizeof done, hipMemcpyDeviceToHost));
-    if (done.error != 0) return fail(LPP_ERR_HIP, "decode kernel gave up waiting for its inputs");
+    if (done.error != 0) return dataflow_report_error(m, done.error);
     if (history_cap > 0) {
         std::vector<int> ring(static_cast<size_t>(history_cap));
         LPP_HIP(hipMemcpy(ring.data(), m->history, ring.size() * sizeof(int), hipMemcpyDeviceToHost));

@@ -65,6 +65,7 @@ struct lpp_model {
     unsigned df_base = 0;                    // sequence-number base of the next persistent launch
     int df_trace_stride = 0;                 // timeline words per workgroup when every workgroup is traced (0: workgroup 0 only)
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
+    unsigned df_ticket_base = 0;             // what the per-XCD workgroup counters read before the next persistent launch
     int df_xcc = 0;                          // XCDs the persistent kernel's workgroups go round (1: near copies off; 0: not probed)
     unsigned spin_limit = 1u << 20;          // polls a wait for tagged inputs may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
