@@ -436,6 +436,10 @@ lpp_status lpp_get_stream(void **hip_stream);
 lpp_status lpp_synchronize(void);
 lpp_status lpp_malloc(void **d_ptr, size_t bytes);
 lpp_status lpp_free(void *d_ptr);
+/* Page-locked host memory, for buffers the device copies into every token (the reference allocates its
+ * host logits this way, model.cpp:42 and :94).  Memory that already exists cannot be registered: allocate it here. */
+lpp_status lpp_malloc_host(void **h_ptr, size_t bytes);
+lpp_status lpp_free_host(void *h_ptr);
 lpp_status lpp_memset(void *d_ptr, int value, size_t bytes);
 lpp_status lpp_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes);
 lpp_status lpp_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes);

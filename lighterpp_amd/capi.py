@@ -140,6 +140,8 @@ SIGNATURES = {
     "lpp_memcpy_h2d": (_i, [_vp, _vp, _sz]),
     "lpp_memcpy_d2h": (_i, [_vp, _vp, _sz]),
     "lpp_memcpy_d2d": (_i, [_vp, _vp, _sz]),
+    "lpp_malloc_host": (_i, [C.POINTER(_vp), _sz]),
+    "lpp_free_host": (_i, [_vp]),
     "lpp_device_info": (_i, [C.c_char_p, _sz, _ip, C.POINTER(_sz)]),
     "lpp_synth_normal_f32": (_i, [_vp, _sz, _u64, _u64, _f]),
     "lpp_synth_normal_f16": (_i, [_vp, _sz, _u64, _u64, _f]),

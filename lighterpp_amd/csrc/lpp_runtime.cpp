@@ -176,6 +176,26 @@ lpp_status lpp_free(void* d_ptr) {
     return LPP_OK;
 }
 
+lpp_status lpp_malloc_host(void** h_ptr, size_t bytes) {
+    LPP_REQUIRE(h_ptr != nullptr, "lpp_malloc_host: null output");
+    if (!lpp::g_rt.ready) LPP_TRY(lpp_init(0));
+    *h_ptr = nullptr;
+    if (bytes == 0) return LPP_OK;
+    hipError_t e = hipHostMalloc(h_ptr, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *h_ptr = nullptr;
+        return fail(LPP_ERR_OOM, "lpp_malloc_host: hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    }
+    return LPP_OK;
+}
+
+lpp_status lpp_free_host(void* h_ptr) {
+    if (h_ptr == nullptr) return LPP_OK;
+    LPP_HIP(hipHostFree(h_ptr));
+    return LPP_OK;
+}
+
 // The three copies are stream-ordered with the kernels and return when done.
 lpp_status lpp_memcpy_h2d(void* d_dst, const void* h_src, size_t bytes) {
     if (bytes == 0) return LPP_OK;

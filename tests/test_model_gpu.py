@@ -242,6 +242,51 @@ def test_long_context_attention_matches_oracle(name):
     o.close()
 
 
+ONE_PASS = {
+    # Heads of size 64: up to 512 positions the persistent kernel keeps a head's whole context on the compute unit
+    # (one wavefront alone up to 64 positions).  Eight KV heads: q, k and v are also handed over inside each XCD.
+    "gqa4_8kv": Shape(2048, 512, 1, 32, 8, 500, 640, 500000.0, fp16=True, tied=True),
+    "gqa2_4kv": Shape(512, 768, 2, 8, 4, 500, 640, 10000.0, fp16=True, tied=False),
+}
+
+
+@pytest.mark.parametrize("name", list(ONE_PASS))
+def test_one_pass_attention_item_matches_oracle(name):
+    """Decode across every boundary of the one-pass item: 64 positions (one wavefront / eight), 128, 384 (the
+    wavefronts' LDS blocks change areas), 512 (its last position) and beyond (back to the walking item).  The
+    cache past the context holds NaN bit patterns on the GPU: the item fetches whole blocks of 64 positions and
+    must use nothing of what lies past the current one."""
+    shape = ONE_PASS[name]
+    m, o = build(shape, 9)
+    m.set_path(capi.PATH_PERSISTENT)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    n = L * nkv * shape.seq_len * hs
+    kfill = capi.synth_normal_f16(n, 601, 1.0).reshape(L, nkv, shape.seq_len, hs)
+    vfill = capi.synth_normal_f16(n, 602, 1.0).reshape(L, nkv, shape.seq_len, hs)
+    for start in (0, 61, 126, 381, 509):
+        k_gpu, v_gpu = kfill.copy(), vfill.copy()
+        k_gpu[:, :, start:, :] = 0x7e00  # binary16 NaN
+        v_gpu[:, :, start:, :] = 0x7e00
+        m.reset()
+        m.write_buffer(capi.B_KEY_CACHE, k_gpu)
+        m.write_buffer(capi.B_VALUE_CACHE, v_gpu)
+        k_cpu, v_cpu = kfill.copy(), vfill.copy()
+        k_cpu[:, :, start:, :] = 0
+        v_cpu[:, :, start:, :] = 0
+        o.buf("key_cache")[:] = capi.f16_to_f32(k_cpu.reshape(-1))
+        o.buf("value_cache")[:] = capi.f16_to_f32(v_cpu.reshape(-1))
+        tok = 5
+        for pos in range(start, start + 6):
+            m.forward(tok, pos, 0.0)
+            want = o.forward_logits(tok, pos)
+            got = m.buffer(capi.B_LOGITS)
+            assert np.all(np.isfinite(got)), (start, pos)
+            assert rel_err(got, want) <= LOGIT_TOL, (start, pos)
+            tok = int(np.argmax(want))
+    m.close()
+    o.close()
+
+
 def test_model_argument_errors():
     shape = SMALL_SHAPES["gqa4_fp16"]
     m = Model(shape)
