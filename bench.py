@@ -17,6 +17,9 @@ Besides the throughput the line carries
                ops.cpp + model.cpp compiled for the host; falls back to the
                restated oracle) timed on a bounded sample of the same workload
                on the host cores of this machine,
+  timeline     per-phase microseconds of one traced token of the persistent
+               kernel (span, hand-over, streaming, skew, streaming floor) and the
+               restatement  token = bytes / 7 TB/s + sampler + hand-overs x mean cost,
   parity       logits of the first decoded positions against the CPU oracle.
 """
 from __future__ import annotations
@@ -36,9 +39,29 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
 HBM_PEAK_GBS = 8000.0
-# (config, kernel) -> HBM bytes fetched + written per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (2.5073 GB + 0.0029 GB at positions 0..35, where the algorithmic figure is 2.4719 GB: ratio 1.016)
-MEASURED_HBM_BYTES_PER_LAUNCH = {("c3_llama32_1b_fp16", "k_decode_dataflow"): 2.5101e9}
+# (config, kernel) -> (HBM bytes fetched + written per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, SHA-256 of
+# the kernel's source file when the two counter runs were made).  Hardware counters cannot be read in-process, so
+# the figure is a constant; it is quoted only while the kernel's source is the one that was measured, and is null
+# (with a note) from the moment the file changes until the two runs are repeated
+# (profiles/persistent_decode_c3_llama32_1b_pmc_hbm_traffic.txt gives the commands).
+KERNEL_SOURCES = {"k_decode_dataflow": ROOT / "lighterpp_amd" / "csrc" / "dataflow_decode.hip"}
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    ("c3_llama32_1b_fp16", "k_decode_dataflow"): (2.5132e9, "41546cc7fdb11b399048d99761b05c1972f0491d54f14515337f71cce6592be8"),
+}
+
+
+def measured_traffic(config: str, kernel: str):
+    """(bytes per launch or None, note or None) for the dominant kernel."""
+    import hashlib
+    entry = MEASURED_HBM_BYTES_PER_LAUNCH.get((config, kernel))
+    if entry is None:
+        return None, "no counter run for this configuration"
+    src = KERNEL_SOURCES.get(kernel)
+    if src is None or not src.exists():
+        return None, "kernel source not found: counter figure not quoted"
+    if hashlib.sha256(src.read_bytes()).hexdigest() != entry[1]:
+        return None, "kernel source changed since the counter runs: repeat them"
+    return entry[0], None
 
 METRIC = "decode tok/s at batch 1 + % of 8 TB/s HBM roofline, Llama-3.2-1B-shape fp16"
 
@@ -179,6 +202,7 @@ def main() -> int:
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time bound of the CPU baseline sample (0 = skip)")
     ap.add_argument("--parity-steps", type=int, default=3)
     ap.add_argument("--profile-reps", type=int, default=20)
+    ap.add_argument("--no-timeline", action="store_true", help="skip the traced token behind the `timeline` object")
     ap.add_argument("--prefill", type=int, default=0, metavar="N",
                     help="time the batched prefill of N prompt ids instead of the decode loop (a second, separate line)")
     args = ap.parse_args()
@@ -259,11 +283,32 @@ def main() -> int:
         # HBM bytes per launch from hardware counters cannot be read in-process: they come from two
         # rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE, each scaled by what the counter
         # reads for a kernel of known size); the figure is quoted only for the kernel it was measured on.
-        traffic = MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, dom[0]))
+        traffic, traffic_note = measured_traffic(args.config, dom[0])
         roofline = dict(bound="hbm", kernel=dom[0], achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                         frac=round(achieved / HBM_PEAK_GBS, 4), traffic=traffic,
                         bytes_per_launch=dom[3], avg_launch_us=round(dom[2] * 1e3, 3),
                         sum_of_kernel_times_ms_per_token=round(per_token_ms, 4))
+        if traffic_note:
+            roofline["traffic_note"] = traffic_note
+
+    # where the token's time goes: per-phase microseconds of one traced token at the window's middle position
+    timeline = None
+    if path == capi.PATH_PERSISTENT and not args.no_timeline:
+        from lighterpp_amd import timeline as tl
+        mid = min(start + steps // 2, shape.seq_len - 1)
+        summary = tl.summarise(shape, tl.trace(model, mid), mid)
+        timeline = dict(position=mid, traced_token_us=round(summary["token_us"], 1),
+                        layer_us=round(summary["layer_us"], 2), layer_floor_us=round(summary["layer_floor_us"], 2),
+                        phases={r["kind"]: dict(span_us=round(r["span"], 2),
+                                                handover_us=round(r["handover"], 2),
+                                                stream_us=None if r["stream"] is None else round(r["stream"], 2),
+                                                skew_us=round(r["skew"], 2), floor_us=round(r["floor"], 2))
+                                for r in summary["phases"]},
+                        classifier_us=round(summary["classifier_us"], 1), sampler_us=round(summary["sampler_us"], 1),
+                        stream_floor_us=round(summary["stream_floor_us"], 1), handovers=summary["handovers"],
+                        mean_handover_cost_us=round(summary["mean_handover_cost_us"], 2),
+                        note="every workgroup writes eight time marks per phase: the traced token is slower than "
+                             "an untraced one (avg_launch_us), the proportions are what this is for")
 
     parity = None
     if args.parity_steps > 0:
@@ -296,6 +341,7 @@ def main() -> int:
                 "peak_gbs": HBM_PEAK_GBS, "frac_of_peak": round(avg_bytes * tok_s / 1e9 / HBM_PEAK_GBS, 4),
                 "device_ms_per_token": round(stats.device_ms / steps, 5)},
         "roofline": roofline,
+        "timeline": timeline,
         "cpu_baseline": cpu,
         "parity": parity,
         "kernels": kernels,
