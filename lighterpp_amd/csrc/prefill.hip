@@ -63,9 +63,13 @@ __device__ __forceinline__ void split_store(half_t* hi, half_t* lo, size_t at, f
 }
 
 // (hi, lo)[t][:] = RMSNorm(x[t][:]) * gain (ops.cpp:20-32); rows t >= n_tokens are zero.
-__global__ __launch_bounds__(256) void k_norm_split(const float* __restrict__ x, const float* __restrict__ gain,
+// With `splits` > 0 the residual update that precedes the norm is done here: x[t][:] += p[0][t][:] +
+// p[1][t][:] + ... in that order, the partial products of a GEMM whose K was split (p[z] starts at
+// partials + z * split_stride), written back to x.
+__global__ __launch_bounds__(256) void k_norm_split(float* __restrict__ x, const float* __restrict__ gain,
                                                     half_t* __restrict__ hi, half_t* __restrict__ lo, int dim,
-                                                    int n_tokens) {
+                                                    int n_tokens, const float* __restrict__ partials, int splits,
+                                                    size_t split_stride) {
 #pragma clang fp contract(off)
     __shared__ float scratch[4];
     const int t = blockIdx.x;
@@ -78,46 +82,72 @@ __global__ __launch_bounds__(256) void k_norm_split(const float* __restrict__ x,
         return;
     }
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
-        const float v = x[row + i];
-        ss += v * v;
+    for (int i = 4 * threadIdx.x; i < dim; i += 4 * blockDim.x) {
+        floatx4 v = *reinterpret_cast<const floatx4*>(x + row + i);
+        if (splits > 0) {
+            for (int z = 0; z < splits; ++z) {
+                const floatx4 a = *reinterpret_cast<const floatx4*>(partials + z * split_stride + row + i);
+                v = floatx4{v[0] + a[0], v[1] + a[1], v[2] + a[2], v[3] + a[3]};
+            }
+            *reinterpret_cast<floatx4*>(x + row + i) = v;
+        }
+        ss += v[0] * v[0];
+        ss += v[1] * v[1];
+        ss += v[2] * v[2];
+        ss += v[3] * v[3];
     }
     ss = block_sum256(ss, scratch);
     ss /= static_cast<float>(dim);
     ss += 1e-5f;
     const float scale = 1.0f / sqrtf(ss);
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) split_store(hi, lo, row + i, x[row + i] * scale * gain[i]);
+    for (int i = 4 * threadIdx.x; i < dim; i += 4 * blockDim.x) {
+        const floatx4 v = *reinterpret_cast<const floatx4*>(x + row + i);
+        const floatx4 gn = *reinterpret_cast<const floatx4*>(gain + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) split_store(hi, lo, row + i + e, v[e] * scale * gn[e]);
+    }
 }
 
 // RoPE on q and k of token t (ops.cpp:34-54), q kept in fp32, k and v written to the
-// caches as binary16 at position pos0 + t (model.cpp:171-176).
-__global__ __launch_bounds__(256) void k_rope_scatter(float* __restrict__ q, const float* __restrict__ k,
-                                                      const float* __restrict__ v, const float2* __restrict__ rope,
-                                                      uint16_t* __restrict__ key_cache, uint16_t* __restrict__ value_cache,
-                                                      int layer, int pos0, int dim, int kv_dim, int hs, int seq_len) {
+// caches as binary16 at position pos0 + t (model.cpp:171-176).  With `splits` > 1, qs/ks/vs are the
+// first of that many partial products, split_stride floats apart, and are summed in order here;
+// q receives the rotated sum either way.
+__global__ __launch_bounds__(256) void k_rope_scatter(float* __restrict__ q, const float* __restrict__ qs,
+                                                      const float* __restrict__ ks, const float* __restrict__ vs,
+                                                      const float2* __restrict__ rope, uint16_t* __restrict__ key_cache,
+                                                      uint16_t* __restrict__ value_cache, int layer, int pos0, int dim,
+                                                      int kv_dim, int hs, int seq_len, int splits, size_t split_stride) {
 #pragma clang fp contract(off)
     const int t = blockIdx.x;
     const int pos = pos0 + t;
     const float2* cs_row = rope + static_cast<size_t>(pos) * (hs / 2);
+    auto summed = [&](const float* first, size_t at) {
+        float2 v = *reinterpret_cast<const float2*>(first + at);
+        for (int z = 1; z < splits; ++z) {
+            const float2 a = *reinterpret_cast<const float2*>(first + z * split_stride + at);
+            v.x += a.x;
+            v.y += a.y;
+        }
+        return v;
+    };
     for (int i = 2 * threadIdx.x; i < dim; i += 2 * blockDim.x) {
-        float* p = q + static_cast<size_t>(t) * dim + i;
+        const size_t at = static_cast<size_t>(t) * dim + i;
         const float2 cs = cs_row[(i % hs) >> 1];
-        const float q0 = p[0], q1 = p[1];
-        p[0] = q0 * cs.x - q1 * cs.y;
-        p[1] = q0 * cs.y + q1 * cs.x;
+        const float2 v = summed(qs, at);
+        q[at] = v.x * cs.x - v.y * cs.y;
+        q[at + 1] = v.x * cs.y + v.y * cs.x;
     }
     for (int i = 2 * threadIdx.x; i < kv_dim; i += 2 * blockDim.x) {
-        const float* pk = k + static_cast<size_t>(t) * kv_dim + i;
-        const float* pv = v + static_cast<size_t>(t) * kv_dim + i;
+        const size_t at = static_cast<size_t>(t) * kv_dim + i;
+        const float2 kk = summed(ks, at), vv = summed(vs, at);
         const float2 cs = cs_row[(i % hs) >> 1];
-        const float k0 = pk[0], k1 = pk[1];
         const int head = i / hs, within = i - head * hs;
         const size_t dst = static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(head) * seq_len * hs +
                            static_cast<size_t>(pos) * hs + within;
-        key_cache[dst] = f32_to_f16_bits(k0 * cs.x - k1 * cs.y);
-        key_cache[dst + 1] = f32_to_f16_bits(k0 * cs.y + k1 * cs.x);
-        value_cache[dst] = f32_to_f16_bits(pv[0]);
-        value_cache[dst + 1] = f32_to_f16_bits(pv[1]);
+        key_cache[dst] = f32_to_f16_bits(kk.x * cs.x - kk.y * cs.y);
+        key_cache[dst + 1] = f32_to_f16_bits(kk.x * cs.y + kk.y * cs.x);
+        value_cache[dst] = f32_to_f16_bits(vv.x);
+        value_cache[dst + 1] = f32_to_f16_bits(vv.y);
     }
 }
 
@@ -352,6 +382,269 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
                 *out = v;
             }
         }
+}
+
+// The same product as a pipeline of LDS stages filled by the memory system itself.
+//
+// A workgroup is eight wavefronts: four that multiply and four that only request data.  A request
+// instruction holds its wavefront until the compute unit's memory pipeline has taken it (64 bytes
+// a cycle: a trip's 64 KiB are 1000 cycles of that), and a wavefront that issues MFMAs cannot
+// issue them while it is held, so the requests go out from wavefronts with nothing else to do;
+// a SIMD runs one of each kind.
+//
+// The four multiplying wavefronts (2 x 2) own a tile of 64 kFi features x 64 kTj tokens; a wavefront
+// owns 32 kFi x 32 kTj of it (kFi x kTj MFMA tiles: the weight side is the longer one, because the
+// activations come twice, as head and remainder, and every fragment is read from LDS once per
+// wavefront that uses it).  A trip covers 64 columns = four k-steps of 16: the rows of the three
+// operand tiles, 128 bytes each (a whole cache line per row and trip), lie one after the other
+// in a stage of LDS, and a wavefront fills 8 rows with one global_load_lds_dwordx4 (lane i -> 16
+// bytes at M0 + 16 i): no registers are staged and nothing waits for the data but the s_waitcnt
+// of the trip that multiplies it.
+//
+// LDS banks: a fragment read takes 16 bytes per lane from 32 consecutive rows; with rows of 128
+// bytes every second row starts in the same bank, so the eight 16-byte pieces of row r are stored
+// in the order piece ^ ((r >> 1) & 7): 16 consecutive lanes then cover all 64 banks once.  The
+// permutation is applied on the way in, by the address each lane requests.
+//
+// The requests are inline assembly: written with the builtin, every LDS read of the loop would
+// wait for all outstanding requests (they may alias), which is the pipeline's whole depth.
+//
+// kMode 0 stores the tile, 1 adds it to y, 2 is the feed-forward pair: the tile's weight rows are
+// 32 kFi features of W1 (the wavefront's first kFi / 2 MFMA tiles) and the same features of W3
+// (its last kFi / 2), and what is stored is (g * sigmoid(g)) * up (ops.cpp:78-87), split into
+// binary16 head and remainder as the next product wants it.
+struct PipeJob {
+    const half_t* w[3];
+    float* y[3];
+    int ldy[3];
+    int first_tile[3];  // first feature tile of matrix i (first_tile[0] = 0); unused entries = INT_MAX
+    const half_t* xh;
+    const half_t* xl;
+    int K;      // row length of w and x
+    int k_len;  // columns a workgroup multiplies: split z covers [z * k_len, (z + 1) * k_len) and writes y + z * split_stride
+    size_t split_stride;
+    int feature_tiles, token_tiles, groups;  // groups = feature_tiles * splits
+    half_t* out_hi;                          // kMode 2: [tokens][out_ld]
+    half_t* out_lo;
+    int out_ld;
+};
+
+constexpr int kPipeTripK = 64;  // columns per trip
+
+template <int kFi, int kTj>
+struct PipeShape {
+    static constexpr int kRowBytes = 2 * kPipeTripK;
+    static constexpr int kRowsA = 64 * kFi, kRowsB = 64 * kTj, kRows = kRowsA + 2 * kRowsB;
+    static constexpr int kStageBytes = kRows * kRowBytes;
+    static constexpr int kStages = 3 * kStageBytes <= 144 * 1024 ? 3 : 2;
+    static constexpr int kLoads = kStageBytes / 4096;  // requests of 1 KiB per wavefront and stage
+    static constexpr int kLdsBytes = kStages * kStageBytes;
+};
+
+template <int kCount>
+__device__ __forceinline__ void wait_requests() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCount) : "memory");
+}
+
+__device__ __forceinline__ void swiglu_split4(half_t* hi, half_t* lo, const float* g, const float* u) {
+#pragma clang fp contract(off)
+    half_t h[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float sigma = 1.0f / (1.0f + expf(-g[e]));
+        const float v = (g[e] * sigma) * u[e];
+        h[e] = static_cast<half_t>(v);
+        l[e] = static_cast<half_t>(v - static_cast<float>(h[e]));
+    }
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    *reinterpret_cast<half4_t*>(hi) = half4_t{h[0], h[1], h[2], h[3]};
+    *reinterpret_cast<half4_t*>(lo) = half4_t{l[0], l[1], l[2], l[3]};
+}
+
+template <int kFi, int kTj, int kMode>
+__global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
+    typedef PipeShape<kFi, kTj> Shape;
+    constexpr int kRowsA = Shape::kRowsA, kRowsB = Shape::kRowsB, kStages = Shape::kStages, kLoads = Shape::kLoads;
+    constexpr int kStageBytes = Shape::kStageBytes, kRowBytes = Shape::kRowBytes;
+    constexpr int kSteps = kPipeTripK / 16;  // k-steps per trip
+    extern __shared__ __align__(1024) char pipe_lds[];
+    const int lane = lane_id();
+    const int wave_of_8 = __builtin_amdgcn_readfirstlane(wave_index());
+    const bool requester = wave_of_8 >= 4;
+    const int wave = wave_of_8 & 3;  // which quarter of the tile (multiplying) or of the requests (requesting)
+    // Workgroups are handed to the eight dies in turn: those that share a weight tile (same features
+    // and columns, other tokens) get numbers that are equal modulo 8, so the tile crosses one die's L2.
+    const int id = static_cast<int>(blockIdx.x), die = id & 7, within = id >> 3;
+    const int group = (within / job.token_tiles) * 8 + die;
+    if (group >= job.groups) return;
+    const int token_tile = within % job.token_tiles;
+    const int tile_all = group % job.feature_tiles, split = group / job.feature_tiles;
+    const int which = tile_all >= job.first_tile[2] ? 2 : (tile_all >= job.first_tile[1] ? 1 : 0);
+    const int tile_x = tile_all - (which == 2 ? job.first_tile[2] : (which == 1 ? job.first_tile[1] : 0));
+    const half_t* __restrict__ w = which == 2 ? job.w[2] : (which == 1 ? job.w[1] : job.w[0]);
+    const int K = job.K, k_first = split * job.k_len;
+    const int r = lane & 31, g = lane >> 5;
+    const int wf = wave & 1, wt = wave >> 1;
+    constexpr int kFeaturesPerTile = kMode == 2 ? 32 * kFi : 64 * kFi;
+    const int f_base = tile_x * kFeaturesPerTile, t_base = token_tile * kRowsB;
+
+    // what each lane requests: request q of this wavefront fills rows 8 (wave + 4 q) .. + 7 of a stage
+    const char* src[kLoads];
+#pragma unroll
+    for (int q = 0; q < kLoads; ++q) {
+        const int row = 8 * (wave + 4 * q) + (lane >> 3);
+        const int piece = (lane & 7) ^ ((row >> 1) & 7);
+        const half_t* from;
+        if (row < kRowsA) {
+            if constexpr (kMode == 2) {
+                const int wave_rows = 32 * kFi, half_rows = 16 * kFi;
+                const int owner = row / wave_rows, rem = row % wave_rows;
+                const half_t* matrix = rem >= half_rows ? job.w[1] : job.w[0];
+                from = matrix + static_cast<size_t>(f_base + owner * half_rows + rem % half_rows) * K;
+            } else {
+                from = w + static_cast<size_t>(f_base + row) * K;
+            }
+        } else if (row < kRowsA + kRowsB) {
+            from = job.xh + static_cast<size_t>(t_base + row - kRowsA) * K;
+        } else {
+            from = job.xl + static_cast<size_t>(t_base + row - kRowsA - kRowsB) * K;
+        }
+        src[q] = reinterpret_cast<const char*>(from + k_first) + 16 * piece;
+    }
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) char*)pipe_lds));
+    const int trips = job.k_len / kPipeTripK;
+    auto request = [&](int trip) {
+        const unsigned at = __builtin_amdgcn_readfirstlane(lds_base + (trip % kStages) * kStageBytes + wave * 1024);
+        const int column = __builtin_amdgcn_readfirstlane(trip * kRowBytes);
+#pragma unroll
+        for (int q = 0; q < kLoads; ++q)
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n" ::"v"(src[q] + column), "s"(at + q * 4096)
+                         : "memory");
+    };
+    // where each lane reads its fragments: row r of an MFMA tile, pieces 2 s + g of k-step s
+    int a_off[kSteps], b_off[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+        const int piece = (2 * s + g) ^ ((r >> 1) & 7);
+        a_off[s] = (wf * 32 * kFi + r) * kRowBytes + 16 * piece;
+        b_off[s] = (kRowsA + wt * 32 * kTj + r) * kRowBytes + 16 * piece;
+    }
+
+    floatx16 acc[kFi][kTj];
+#pragma unroll
+    for (int i = 0; i < kFi; ++i)
+#pragma unroll
+        for (int j = 0; j < kTj; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    struct Frags {
+        half8_t a[kFi], bh[kTj], bl[kTj];
+    };
+    auto read = [&](Frags& f, int trip, int s) {
+        const char* stage = pipe_lds + (trip % kStages) * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < kFi; ++i) f.a[i] = *reinterpret_cast<const half8_t*>(stage + a_off[s] + i * 32 * kRowBytes);
+#pragma unroll
+        for (int j = 0; j < kTj; ++j) {
+            f.bh[j] = *reinterpret_cast<const half8_t*>(stage + b_off[s] + j * 32 * kRowBytes);
+            f.bl[j] = *reinterpret_cast<const half8_t*>(stage + b_off[s] + (kRowsB + j * 32) * kRowBytes);
+        }
+    };
+    // (one half of a k-step's MFMAs: the weight tiles [kFi / 2 * half, kFi / 2 * (half + 1)))
+    auto multiply_half = [&](const Frags& f, int half) {
+#pragma unroll
+        for (int i = kFi / 2 * half; i < kFi / 2 * (half + 1); ++i)
+#pragma unroll
+            for (int j = 0; j < kTj; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[i], f.bh[j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[i], f.bl[j], acc[i][j], 0, 0, 0);
+            }
+    };
+    // (requesting wavefronts) wait until the requests of `trip` have landed: those of later trips, at
+    // most kStages - 2 of them, may be in flight
+    auto landed = [&](int trip, int trips) {
+        const int later = trips - 1 - trip;
+        if (kStages > 2 && later >= kStages - 2) wait_requests<(kStages - 2) * kLoads>();
+        else wait_requests<0>();
+    };
+    // One barrier per trip, inside the last k-step of the trip before: the requesting wavefronts
+    // arrive when the trip's data has landed, the multiplying ones when they hold the last
+    // fragments of the trip before in registers, which frees that trip's stage for the requests of
+    // trip t + kStages.
+    if (requester) {
+#pragma unroll
+        for (int t = 0; t < kStages - 1; ++t)
+            if (t < trips) request(t);
+        landed(0, trips);
+        __syncthreads();
+        if (kStages - 1 < trips) request(kStages - 1);
+        for (int t = 0; t < trips; ++t) {
+            landed(t + 1, trips);
+            __syncthreads();
+            if (t + kStages < trips) request(t + kStages);
+        }
+        return;
+    }
+    Frags frags[2];
+    __syncthreads();
+    read(frags[0], 0, 0);
+    // The fragments of a k-step are read from LDS behind the first half of the MFMAs of the k-step
+    // before and are waited for by the k-step after: the wait the compiler places is for every
+    // read in flight, so none may be in flight that has not had half a k-step to arrive.
+    for (int t = 0; t < trips; ++t) {
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const Frags& cur = frags[s & 1];
+            Frags& next = frags[(s + 1) & 1];
+            const bool last = s == kSteps - 1;
+            multiply_half(cur, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // (after the last trip this reads a stage nobody uses: one path through the loop)
+            if (last) __syncthreads();
+            read(next, last ? t + 1 : t, last ? 0 : s + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply_half(cur, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // D[m][n]: a lane holds column n = lane % 32 (a token) and rows m = 8 (e / 4) + 4 (lane / 32) + e % 4 (features)
+    if constexpr (kMode == 2) {
+#pragma unroll
+        for (int i = 0; i < kFi / 2; ++i)
+#pragma unroll
+            for (int j = 0; j < kTj; ++j) {
+                const size_t at = static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j + r) * job.out_ld + f_base + wf * 16 * kFi +
+                                  32 * i + 4 * g;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const float gate[4] = {acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                    const float up[4] = {acc[i + kFi / 2][j][4 * e4], acc[i + kFi / 2][j][4 * e4 + 1],
+                                         acc[i + kFi / 2][j][4 * e4 + 2], acc[i + kFi / 2][j][4 * e4 + 3]};
+                    swiglu_split4(job.out_hi + at + 8 * e4, job.out_lo + at + 8 * e4, gate, up);
+                }
+            }
+    } else {
+        float* __restrict__ y = (which == 2 ? job.y[2] : (which == 1 ? job.y[1] : job.y[0])) + static_cast<size_t>(split) * job.split_stride;
+        const int ldy = which == 2 ? job.ldy[2] : (which == 1 ? job.ldy[1] : job.ldy[0]);
+#pragma unroll
+        for (int i = 0; i < kFi; ++i)
+#pragma unroll
+            for (int j = 0; j < kTj; ++j) {
+                float* row = y + static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j + r) * ldy + f_base + wf * 32 * kFi + 32 * i + 4 * g;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    floatx4* out = reinterpret_cast<floatx4*>(row + 8 * e4);
+                    floatx4 v = floatx4{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                    if constexpr (kMode == 1) {
+                        const floatx4 old = *out;
+                        v = floatx4{old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
+                    }
+                    *out = v;
+                }
+            }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -610,12 +903,13 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     }
 }
 
-// x[i] += p[0][i] + p[1][i] + ... in that order: the partial products of a GEMM whose K was split.
+// x[i] (+)= p[0][i] + p[1][i] + ... in that order: the partial products of a GEMM whose K was split.
+template <bool kAccumulate>
 __global__ __launch_bounds__(256) void k_add_partials(float* __restrict__ x, const float* __restrict__ p, int splits,
                                                       size_t stride, size_t count) {
     const size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
     if (i >= count) return;
-    floatx4 v = *reinterpret_cast<const floatx4*>(x + i);
+    floatx4 v = kAccumulate ? *reinterpret_cast<const floatx4*>(x + i) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     for (int s = 0; s < splits; ++s) {
         const floatx4 a = *reinterpret_cast<const floatx4*>(p + s * stride + i);
         v = floatx4{v[0] + a[0], v[1] + a[1], v[2] + a[2], v[3] + a[3]};
@@ -639,7 +933,7 @@ __global__ __launch_bounds__(256) void k_split(const float* __restrict__ x, half
 namespace {
 
 // Buffers of a chunk of t_pad tokens, in lpp_model::pf_buf order.
-enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufVt, kBufCount };
+enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufVt, kBufHi2, kBufLo2, kBufCount };
 static_assert(kBufCount <= static_cast<int>(sizeof(lpp_model::pf_buf) / sizeof(void*)), "lpp_model::pf_buf is too small");
 
 const char* unsupported_reason(const lpp_model* m) {
@@ -668,7 +962,10 @@ lpp_status ensure_scratch(lpp_model* m, int t_pad) {
                                      t * widest * sizeof(pf::half_t),
                                      t * widest * sizeof(pf::half_t),
                                      // one layer's V with positions contiguous: [kv_dim][seq_len rounded up to 32]
-                                     static_cast<size_t>(m->kv_dim) * ((c.seq_len + 31) / 32 * 32) * sizeof(uint16_t)};
+                                     static_cast<size_t>(m->kv_dim) * ((c.seq_len + 31) / 32 * 32) * sizeof(uint16_t),
+                                     // the feed-forward activations, written while hi/lo are still being read
+                                     t * c.hidden_dim * sizeof(pf::half_t),
+                                     t * c.hidden_dim * sizeof(pf::half_t)};
     for (int i = 0; i < kBufCount; ++i) {
         lpp_status st = lpp_malloc(&m->pf_buf[i], bytes[i]);
         if (st != LPP_OK) {
@@ -687,76 +984,97 @@ struct Product {
     int n;
 };
 
-// `partials` (optional, partial_floats long): room for the partial products of a split K.  A long K
-// with few output tiles (the down projection: 8192 columns, 2048 rows) is cut into up to four
-// ranges, each multiplied by its own workgroups into `partials`, and added to y in a fixed order.
+template <int kFi, int kTj, int kMode>
+lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
+    typedef pf::PipeShape<kFi, kTj> Shape;
+    static bool sized = false;
+    if (!sized) {
+        LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLdsBytes));
+        sized = true;
+    }
+    const int per_die = (job.groups + 7) / 8;
+    hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
+    LPP_CHECK_LAUNCH("k_gemm_pipe");
+    return LPP_OK;
+}
+
+// `partials` (optional, partial_floats long): room for the partial products of a split K.  A product
+// with too few output tiles for the compute units is cut along K into ranges, each multiplied by
+// its own workgroups into `partials`: range z of matrix i lies at partials + z * t_pad * (n_0 + n_1 +
+// ..) + t_pad * (n_0 + .. + n_(i-1)), rows of n_i floats.  With `left_split` the caller adds the
+// ranges itself (in order, in the kernel that reads the product next) and gets their number there;
+// without it they are added to y here, in order.
 lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad, bool accumulate,
-                hipStream_t s, float* partials = nullptr, size_t partial_floats = 0) {
+                hipStream_t s, float* partials = nullptr, size_t partial_floats = 0, int* left_split = nullptr) {
     LPP_REQUIRE(count >= 1 && count <= 3 && t_pad % pf::kTileTokens == 0 && K % 32 == 0, "prefill GEMM: %d products, K %d, T %d",
                 count, K, t_pad);
+    if (left_split != nullptr) *left_split = 1;
     int total_n = 0;
+    bool wide = true;  // every matrix a whole number of 256-row tiles
     for (int i = 0; i < count; ++i) {
         LPP_REQUIRE(prods[i].n > 0 && prods[i].n % pf::kTileFeatures == 0, "prefill GEMM: n %d", prods[i].n);
         total_n += prods[i].n;
+        wide = wide && prods[i].n % 256 == 0;
+    }
+    const bool staged = K % pf::kPipeTripK == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr;
+    if (staged) {
+        const int token_tiles = t_pad / pf::kTileTokens;
+        wide = wide && (total_n / 256) * token_tiles >= compute_units() && getenv("LPP_PREFILL_NO_WIDE") == nullptr;
+        const int tile = wide ? 256 : 128;
+        const int feature_tiles = total_n / tile;
+        const size_t stride = static_cast<size_t>(t_pad) * total_n;
+        int splits = 1;
+        if (partials != nullptr && (count == 1 || left_split != nullptr)) {
+            while (splits < 8 && feature_tiles * token_tiles * splits * 2 <= compute_units() &&
+                   K % (2 * pf::kPipeTripK * splits) == 0 && K / (2 * splits) >= 512 && stride * 2 * splits <= partial_floats)
+                splits *= 2;
+        }
+        pf::PipeJob job = {};
+        int at = 0;
+        size_t before = 0;
+        for (int i = 0; i < 3; ++i) {
+            const Product& p = prods[i < count ? i : count - 1];
+            job.w[i] = static_cast<const pf::half_t*>(p.w);
+            job.y[i] = splits > 1 ? partials + before : p.y;
+            job.ldy[i] = p.n;
+            job.first_tile[i] = i < count ? at : 0x7fffffff;
+            if (i < count) {
+                at += p.n / tile;
+                before += static_cast<size_t>(t_pad) * p.n;
+            }
+        }
+        job.xh = xh;
+        job.xl = xl;
+        job.K = K;
+        job.k_len = K / splits;
+        job.split_stride = stride;
+        job.feature_tiles = feature_tiles;
+        job.token_tiles = token_tiles;
+        job.groups = feature_tiles * splits;
+        const bool add_in_kernel = accumulate && splits == 1;
+        if (wide) {
+            if (add_in_kernel) LPP_TRY((launch_pipe<4, 2, 1>(job, s)));
+            else LPP_TRY((launch_pipe<4, 2, 0>(job, s)));
+        } else {
+            if (add_in_kernel) LPP_TRY((launch_pipe<2, 2, 1>(job, s)));
+            else LPP_TRY((launch_pipe<2, 2, 0>(job, s)));
+        }
+        if (splits > 1 && left_split != nullptr) {
+            *left_split = splits;
+        } else if (splits > 1) {
+            if (accumulate)
+                hipLaunchKernelGGL(pf::k_add_partials<true>, dim3(static_cast<unsigned>((stride / 4 + 255) / 256)), dim3(256), 0, s,
+                                   prods[0].y, partials, splits, stride, stride);
+            else
+                hipLaunchKernelGGL(pf::k_add_partials<false>, dim3(static_cast<unsigned>((stride / 4 + 255) / 256)), dim3(256), 0, s,
+                                   prods[0].y, partials, splits, stride, stride);
+            LPP_CHECK_LAUNCH("k_add_partials");
+        }
+        return LPP_OK;
     }
     const bool large_tiles = (total_n / pf::kTileFeatures) * (t_pad / pf::kTileTokens) >= compute_units();
     const int tile = large_tiles ? pf::kTileFeatures : 64;
-    const bool staged = K % 64 == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr;
-    if (staged && accumulate && count == 1 && partials != nullptr) {
-        const int n = prods[0].n;
-        const int big_tiles = (n / pf::kTileFeatures) * (t_pad / pf::kTileTokens);
-        int splits = 1;
-        while (splits < 4 && big_tiles * splits < compute_units() && K % (128 * splits) == 0 && K / (2 * splits) >= 1024) splits *= 2;
-        const size_t stride = static_cast<size_t>(t_pad) * n;
-        if (splits > 1 && stride * splits <= partial_floats) {
-            pf::GemmOutputs o3;
-            for (int i = 0; i < 3; ++i) {
-                o3.w[i] = static_cast<const pf::half_t*>(prods[0].w);
-                o3.y[i] = partials;
-                o3.ldy[i] = n;
-                o3.first_tile[i] = i == 0 ? 0 : 0x7fffffff;
-            }
-            o3.k_len = K / splits;
-            o3.split_stride = stride;
-            hipLaunchKernelGGL((pf::k_gemm_lds<false, 2, 64>), dim3(n / pf::kTileFeatures, t_pad / pf::kTileTokens, splits), dim3(256), 0,
-                               s, o3, xh, xl, K);
-            LPP_CHECK_LAUNCH("k_gemm_lds");
-            hipLaunchKernelGGL(pf::k_add_partials, dim3(static_cast<unsigned>((stride / 4 + 255) / 256)), dim3(256), 0, s, prods[0].y,
-                               partials, splits, stride, stride);
-            LPP_CHECK_LAUNCH("k_add_partials");
-            return LPP_OK;
-        }
-    }
-    if (staged) {
-        pf::GemmOutputs o3;
-        o3.k_len = K;
-        o3.split_stride = 0;
-        int at = 0;
-        for (int i = 0; i < 3; ++i) {
-            const Product& p = prods[i < count ? i : count - 1];
-            o3.w[i] = static_cast<const pf::half_t*>(p.w);
-            o3.y[i] = p.y;
-            o3.ldy[i] = p.n;
-            o3.first_tile[i] = i < count ? at : 0x7fffffff;
-            if (i < count) at += p.n / tile;
-        }
-        const dim3 grid(at, t_pad / tile);
-        if (large_tiles) {
-            if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 2, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
-            else hipLaunchKernelGGL((pf::k_gemm_lds<false, 2, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
-        } else {
-            // (small tiles: a trip of 128 columns where K allows, half the barriers and round trips per product)
-            if (K % 128 == 0 && getenv("LPP_PREFILL_TRIP64") == nullptr) {
-                if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 1, 128>), grid, dim3(256), 0, s, o3, xh, xl, K);
-                else hipLaunchKernelGGL((pf::k_gemm_lds<false, 1, 128>), grid, dim3(256), 0, s, o3, xh, xl, K);
-            } else {
-                if (accumulate) hipLaunchKernelGGL((pf::k_gemm_lds<true, 1, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
-                else hipLaunchKernelGGL((pf::k_gemm_lds<false, 1, 64>), grid, dim3(256), 0, s, o3, xh, xl, K);
-            }
-        }
-        LPP_CHECK_LAUNCH("k_gemm_lds");
-        return LPP_OK;
-    }
     // fragments straight from memory: one launch per matrix
     for (int i = 0; i < count; ++i) {
         const pf::half_t* wh = static_cast<const pf::half_t*>(prods[i].w);
@@ -773,6 +1091,29 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
         LPP_CHECK_LAUNCH("k_gemm");
     }
     return LPP_OK;
+}
+
+// (hi, lo)[t][u] = SwiGLU(W1 x[t], W3 x[t])[u] in one launch: the gate and the up projection of a
+// feature share a workgroup, and the activation is applied to the accumulators.
+lpp_status gate_up_swiglu(const void* w1, const void* w3, int hidden, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad,
+                          pf::half_t* out_hi, pf::half_t* out_lo, hipStream_t s) {
+    pf::PipeJob job = {};
+    job.w[0] = static_cast<const pf::half_t*>(w1);
+    job.w[1] = static_cast<const pf::half_t*>(w3);
+    job.w[2] = job.w[1];
+    job.first_tile[0] = 0;
+    job.first_tile[1] = job.first_tile[2] = 0x7fffffff;
+    job.xh = xh;
+    job.xl = xl;
+    job.K = K;
+    job.k_len = K;
+    job.feature_tiles = hidden / 128;  // 128 features a tile: 128 rows of W1 and the same 128 of W3
+    job.token_tiles = t_pad / pf::kTileTokens;
+    job.groups = job.feature_tiles;
+    job.out_hi = out_hi;
+    job.out_lo = out_lo;
+    job.out_ld = hidden;
+    return launch_pipe<4, 2, 2>(job, s);
 }
 
 // One chunk: tokens[0..n) at positions pos0 .. pos0 + n - 1; n <= kChunk.
@@ -799,17 +1140,34 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
     auto layer_of = [&](int t, int l, size_t rows, size_t cols) {
         return static_cast<const char*>(m->w[t]) + static_cast<size_t>(l) * rows * cols * wb;
     };
+    pf::half_t* hi2 = static_cast<pf::half_t*>(m->pf_buf[kBufHi2]);
+    pf::half_t* lo2 = static_cast<pf::half_t*>(m->pf_buf[kBufLo2]);
+    // The fp32 gate and up buffers double as room for the partial products of the GEMMs whose K is
+    // split (each is t_pad * hidden floats): up for Wq/Wk/Wv, gate for Wo and then for W2.
+    const size_t room = static_cast<size_t>(t_pad) * hidden;
+    const bool fused_ffn = dim % pf::kPipeTripK == 0 && hidden % 128 == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr &&
+                           getenv("LPP_PREFILL_NO_FUSED_FFN") == nullptr;
+    int pending = 0;  // ranges of the product before (W2's, then Wo's) still to be added to x
     for (int l = 0; l < c.n_layers; ++l) {
         // attention block, model.cpp:216-218
         hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
-                           static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n);
+                           static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, gate,
+                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim);
         LPP_CHECK_LAUNCH("k_norm_split");
         const Product qkv[3] = {{layer_of(LPP_T_WQ, l, dim, dim), q, dim}, {layer_of(LPP_T_WK, l, kv, dim), k, kv},
                                 {layer_of(LPP_T_WV, l, kv, dim), v, kv}};
-        LPP_TRY(gemm(qkv, 3, hi, lo, dim, t_pad, false, s));
-        hipLaunchKernelGGL(pf::k_rope_scatter, dim3(n), dim3(256), 0, s, q, k, v, m->rope, m->key_cache, m->value_cache, l, pos0,
-                           dim, kv, hs, c.seq_len);
+        int qkv_split = 1;
+        LPP_TRY(gemm(qkv, 3, hi, lo, dim, t_pad, false, s, up, room, &qkv_split));
+        const size_t qkv_stride = static_cast<size_t>(t_pad) * (dim + 2 * kv);
+        const float* qs = qkv_split > 1 ? up : q;
+        const float* ks = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * dim : k;
+        const float* vs = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * (dim + kv) : v;
+        hipLaunchKernelGGL(pf::k_rope_scatter, dim3(n), dim3(256), 0, s, q, qs, ks, vs, m->rope, m->key_cache, m->value_cache, l,
+                           pos0, dim, kv, hs, c.seq_len, qkv_split, qkv_stride);
         LPP_CHECK_LAUNCH("k_rope_scatter");
+        // What a prefill leaves behind is the cache: the last layer's rows are in place here, and nothing
+        // reads what the rest of that layer would compute.
+        if (l == c.n_layers - 1) break;
         // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
         const bool matrix_cores = 32 % m->gqa == 0 && getenv("LPP_PREFILL_VALU_ATTENTION") == nullptr;
         if (matrix_cores) {
@@ -835,18 +1193,23 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
                                m->value_cache, hi, lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len, n);
         LPP_CHECK_LAUNCH("k_attention");
         const Product wo = {layer_of(LPP_T_WO, l, dim, dim), x, dim};
-        LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s));
+        LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s, gate, room, &pending));
         // feed-forward block, model.cpp:221-226
         hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
-                           static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n);
+                           static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, gate,
+                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim);
         LPP_CHECK_LAUNCH("k_norm_split");
-        const Product gate_up[2] = {{layer_of(LPP_T_W1, l, hidden, dim), gate, hidden}, {layer_of(LPP_T_W3, l, hidden, dim), up, hidden}};
-        LPP_TRY(gemm(gate_up, 2, hi, lo, dim, t_pad, false, s));
-        hipLaunchKernelGGL(pf::k_swiglu_split, dim3((hidden + 255) / 256, t_pad), dim3(256), 0, s, gate, up, hi, lo, hidden, n);
-        LPP_CHECK_LAUNCH("k_swiglu_split");
+        if (fused_ffn) {
+            LPP_TRY(gate_up_swiglu(layer_of(LPP_T_W1, l, hidden, dim), layer_of(LPP_T_W3, l, hidden, dim), hidden, hi, lo, dim, t_pad,
+                                   hi2, lo2, s));
+        } else {
+            const Product gate_up[2] = {{layer_of(LPP_T_W1, l, hidden, dim), gate, hidden}, {layer_of(LPP_T_W3, l, hidden, dim), up, hidden}};
+            LPP_TRY(gemm(gate_up, 2, hi, lo, dim, t_pad, false, s));
+            hipLaunchKernelGGL(pf::k_swiglu_split, dim3((hidden + 255) / 256, t_pad), dim3(256), 0, s, gate, up, hi2, lo2, hidden, n);
+            LPP_CHECK_LAUNCH("k_swiglu_split");
+        }
         const Product w2 = {layer_of(LPP_T_W2, l, dim, hidden), x, dim};
-        // (the gate buffer is free again: room for the partial products of a split K)
-        LPP_TRY(gemm(&w2, 1, hi, lo, hidden, t_pad, true, s, gate, static_cast<size_t>(t_pad) * hidden));
+        LPP_TRY(gemm(&w2, 1, hi2, lo2, hidden, t_pad, true, s, gate, room, &pending));
     }
     LPP_HIP(hipStreamSynchronize(s));
     return LPP_OK;
