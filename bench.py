@@ -175,8 +175,10 @@ def bench_prefill(args, model, shape, name, cus) -> int:
     capi.synchronize()
     sec = (time.perf_counter() - t0) / reps
     L, dim, kv, hidden = shape.n_layers, shape.dim, shape.kv_dim, shape.hidden_dim
-    gemm_flops = 2.0 * L * (2 * dim * dim + 2 * kv * dim + 3 * hidden * dim) * n
-    att_flops = 4.0 * L * shape.n_heads * shape.head_size * n * (n + 1) / 2
+    # What a prefill owes is the cache: every layer's Wk and Wv products, and Wq, attention, Wo and
+    # the feed-forward block of all layers but the last, whose output nothing reads.
+    gemm_flops = 2.0 * (L * 2 * kv * dim + (L - 1) * (2 * dim * dim + 3 * hidden * dim)) * n
+    att_flops = 4.0 * (L - 1) * shape.n_heads * shape.head_size * n * (n + 1) / 2
     tflops = (gemm_flops + att_flops) / sec / 1e12
     out = dict(metric="batched prefill, prompt ids/s, " + args.config, value=round(n / sec, 1), unit="tok/s", n_gpus=1,
                steps=reps, warmup=2, ms_per_step=round(sec * 1e3, 3), higher_is_better=True, scaling="weak",
@@ -184,8 +186,9 @@ def bench_prefill(args, model, shape, name, cus) -> int:
                config=dict(workload=args.config, prompt_ids=n, chunk=512),
                roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
                              frac=round(tflops / MFMA_F16_PEAK_TFLOPS, 4), traffic=None,
-                             note="algorithmic flops (each product counted once; the kernel issues two MFMAs per "
-                                  "product, for the activation's head and remainder)"),
+                             note="algorithmic flops of what the cache depends on (the last layer stops at its K/V "
+                                  "rows); each product counted once: the kernel issues two MFMAs per product, for "
+                                  "the activation's head and remainder"),
                cpu_baseline=None,
                device=dict(name=name.value.decode(), compute_units=cus.value))
     print(json.dumps(out))

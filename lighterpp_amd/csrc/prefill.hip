@@ -108,6 +108,71 @@ __global__ __launch_bounds__(256) void k_norm_split(float* __restrict__ x, const
     }
 }
 
+// The same with a wavefront per row and the row in registers (dim = 256 kChunks): one pass over
+// the memory, no barrier.  The sum of squares runs over the lane's elements in order, then across
+// the lanes.
+template <int kChunks>
+__global__ __launch_bounds__(256) void k_norm_split_rows(float* __restrict__ x, const float* __restrict__ gain,
+                                                         half_t* __restrict__ hi, half_t* __restrict__ lo, int n_tokens,
+                                                         int rows, const float* __restrict__ partials, int splits,
+                                                         size_t split_stride) {
+#pragma clang fp contract(off)
+    constexpr int kDim = 256 * kChunks;
+    const int lane = lane_id();
+    const int t = static_cast<int>(blockIdx.x) * 4 + wave_index();
+    if (t >= rows) return;
+    const size_t row = static_cast<size_t>(t) * kDim;
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    if (t >= n_tokens) {
+        const half4_t zero = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c) {
+            *reinterpret_cast<half4_t*>(hi + row + 256 * c + 4 * lane) = zero;
+            *reinterpret_cast<half4_t*>(lo + row + 256 * c + 4 * lane) = zero;
+        }
+        return;
+    }
+    floatx4 v[kChunks];
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) v[c] = *reinterpret_cast<const floatx4*>(x + row + 256 * c + 4 * lane);
+    if (splits > 0) {
+        for (int z = 0; z < splits; ++z) {
+#pragma unroll
+            for (int c = 0; c < kChunks; ++c) {
+                const floatx4 a = *reinterpret_cast<const floatx4*>(partials + z * split_stride + row + 256 * c + 4 * lane);
+                v[c] = floatx4{v[c][0] + a[0], v[c][1] + a[1], v[c][2] + a[2], v[c][3] + a[3]};
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c) *reinterpret_cast<floatx4*>(x + row + 256 * c + 4 * lane) = v[c];
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+        ss += v[c][0] * v[c][0];
+        ss += v[c][1] * v[c][1];
+        ss += v[c][2] * v[c][2];
+        ss += v[c][3] * v[c][3];
+    }
+    ss = wave_sum(ss);
+    ss /= static_cast<float>(kDim);
+    ss += 1e-5f;
+    const float scale = 1.0f / sqrtf(ss);
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+        const floatx4 gn = *reinterpret_cast<const floatx4*>(gain + 256 * c + 4 * lane);
+        half4_t h, l;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float y = v[c][e] * scale * gn[e];
+            h[e] = static_cast<half_t>(y);
+            l[e] = static_cast<half_t>(y - static_cast<float>(h[e]));
+        }
+        *reinterpret_cast<half4_t*>(hi + row + 256 * c + 4 * lane) = h;
+        *reinterpret_cast<half4_t*>(lo + row + 256 * c + 4 * lane) = l;
+    }
+}
+
 // RoPE on q and k of token t (ops.cpp:34-54), q kept in fp32, k and v written to the
 // caches as binary16 at position pos0 + t (model.cpp:171-176).  With `splits` > 1, qs/ks/vs are the
 // first of that many partial products, split_stride floats apart, and are summed in order here;
@@ -764,8 +829,11 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
 // The same attention on the matrix cores
 // ---------------------------------------------------------------------------
 //
-// A wavefront owns 32 query rows = (32 / gqa) consecutive tokens x the gqa query heads of one KV
-// head, and walks the cache in blocks of 32 positions:
+// A workgroup owns 32 query rows = (32 / gqa) consecutive tokens x the gqa query heads of one KV
+// head; its four wavefronts share the cache's blocks of 32 positions among them (wavefront w takes
+// blocks w, w + 4, ..: a row's work is a chain of dependent steps per block, so the longest rows
+// set the kernel's time), each with its own running maximum, sum and output, merged through
+// LDS at the end.  Per block:
 //   S^T[pos][row] = sum_d K[pos][d] Q[row][d]     A = K block (a lane's 8 d-values: one 16-byte
 //                                                 load from the cache row), B = Q (head + remainder)
 //   online softmax: in the result a LANE holds one query row (its column) and 16 of the block's 32
@@ -809,8 +877,8 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     const int lane = lane_id(), wave = wave_index();
     const int r = lane & 31, g = lane >> 5;
     const int tokens_per_tile = 32 / gqa;
-    const int t0 = (static_cast<int>(blockIdx.x) * 4 + wave) * tokens_per_tile;
-    if (t0 >= n_tokens) return;  // (wavefronts of a workgroup do not meet again)
+    const int t0 = static_cast<int>(blockIdx.x) * tokens_per_tile;
+    if (t0 >= n_tokens) return;  // (the whole workgroup)
     const int kvh = blockIdx.y;
     const int my_tok = t0 + r / gqa, my_head = r % gqa;
     const bool valid = my_tok < n_tokens;
@@ -842,17 +910,38 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         for (int e = 0; e < 16; ++e) o[dt][e] = 0.0f;
     float top = -INFINITY, lsum = 0.0f;
 
-    for (int p0 = 0; p0 < limit; p0 += 32) {
-        floatx16 st;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) st[e] = 0.0f;
+    // The K fragments of the next block and the V^T fragments of this one are requested before this
+    // block's products: a block would otherwise be two memory round trips with nothing in between.
+    auto fetch_k = [&](half8_t (&kf)[kKSteps], int p0) {
         const int prow = (p0 + r < seq_len) ? p0 + r : seq_len - 1;  // (rows past the tile's limit are masked below)
         const uint16_t* krow = kbase + static_cast<size_t>(prow) * kHs + 8 * g;
 #pragma unroll
+        for (int s = 0; s < kKSteps; ++s) kf[s] = as_half8(load16(krow + 16 * s));
+    };
+    half8_t k_next[kKSteps];
+    fetch_k(k_next, 32 * wave);
+    for (int p0 = 32 * wave; p0 < limit; p0 += 128) {
+        floatx16 st;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) st[e] = 0.0f;
+        half8_t kf[kKSteps];
+#pragma unroll
+        for (int s = 0; s < kKSteps; ++s) kf[s] = k_next[s];
+        half8_t vf[kDTiles][2];
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                const uint16_t* vrow = vtb + static_cast<size_t>(32 * dt + r) * vt_stride + p0 + 16 * s2 + 4 * g;
+                const half4_t a0 = *reinterpret_cast<const half4_t*>(vrow);
+                const half4_t a1 = *reinterpret_cast<const half4_t*>(vrow + 8);
+                vf[dt][s2] = half8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+            }
+        if (p0 + 128 < limit) fetch_k(k_next, p0 + 128);
+#pragma unroll
         for (int s = 0; s < kKSteps; ++s) {
-            const half8_t kf = as_half8(load16(krow + 16 * s));
-            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qh[s], st, 0, 0, 0);
-            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, ql[s], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], qh[s], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], ql[s], st, 0, 0, 0);
         }
         float sv[16];
         float block_top = -INFINITY;
@@ -884,22 +973,59 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
             for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-                const uint16_t* vrow = vtb + static_cast<size_t>(32 * dt + r) * vt_stride + p0 + 16 * s2 + 4 * g;
-                const half4_t a0 = *reinterpret_cast<const half4_t*>(vrow);
-                const half4_t a1 = *reinterpret_cast<const half4_t*>(vrow + 8);
-                const half8_t vf = half8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, ph[s2], o[dt], 0, 0, 0);
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pl[s2], o[dt], 0, 0, 0);
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[dt][s2], ph[s2], o[dt], 0, 0, 0);
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[dt][s2], pl[s2], o[dt], 0, 0, 0);
             }
         }
+    }
+    // merge: wavefronts 1..3 hand their (maximum, sum, output) to wavefront 0, lane for lane
+    __shared__ float merge_o[3][kDTiles * 16][64];
+    __shared__ float merge_ms[3][2][64];
+    if (wave > 0) {
+        merge_ms[wave - 1][0][lane] = top;
+        merge_ms[wave - 1][1][lane] = lsum;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) merge_o[wave - 1][dt * 16 + e][lane] = o[dt][e];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float all_top = top;  // finite: block 0 is wavefront 0's and position 0 is in every row's range
+#pragma unroll
+    for (int w = 0; w < 3; ++w) all_top = fmaxf(all_top, merge_ms[w][0][lane]);
+    const float own = exp_fast(top - all_top);
+    lsum *= own;
+#pragma unroll
+    for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[dt][e] *= own;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        const float their_top = merge_ms[w][0][lane];
+        const float weight = (their_top == -INFINITY) ? 0.0f : exp_fast(their_top - all_top);
+        lsum += merge_ms[w][1][lane] * weight;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[dt][e] += merge_o[w][dt * 16 + e][lane] * weight;
     }
     if (valid) {
         const size_t base = static_cast<size_t>(my_tok) * dim + (kvh * gqa + my_head) * kHs;
 #pragma unroll
         for (int dt = 0; dt < kDTiles; ++dt)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-                split_store(out_hi, out_lo, base + 32 * dt + 8 * (e >> 2) + 4 * g + (e & 3), o[dt][e] / lsum);
+            for (int e4 = 0; e4 < 4; ++e4) {
+                half4_t h, l;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const float v = o[dt][4 * e4 + u] / lsum;
+                    h[u] = static_cast<half_t>(v);
+                    l[u] = static_cast<half_t>(v - static_cast<float>(h[u]));
+                }
+                *reinterpret_cast<half4_t*>(out_hi + base + 32 * dt + 8 * e4 + 4 * g) = h;
+                *reinterpret_cast<half4_t*>(out_lo + base + 32 * dt + 8 * e4 + 4 * g) = l;
+            }
     }
 }
 
@@ -1093,6 +1219,21 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
     return LPP_OK;
 }
 
+lpp_status norm_split(float* x, const float* gain, pf::half_t* hi, pf::half_t* lo, int dim, int n, int t_pad, const float* partials,
+                      int splits, size_t split_stride, hipStream_t s) {
+    const dim3 rows_grid((t_pad + 3) / 4);
+    if (dim == 1024)
+        hipLaunchKernelGGL(pf::k_norm_split_rows<4>, rows_grid, dim3(256), 0, s, x, gain, hi, lo, n, t_pad, partials, splits, split_stride);
+    else if (dim == 2048)
+        hipLaunchKernelGGL(pf::k_norm_split_rows<8>, rows_grid, dim3(256), 0, s, x, gain, hi, lo, n, t_pad, partials, splits, split_stride);
+    else if (dim == 4096)
+        hipLaunchKernelGGL(pf::k_norm_split_rows<16>, rows_grid, dim3(256), 0, s, x, gain, hi, lo, n, t_pad, partials, splits, split_stride);
+    else
+        hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x, gain, hi, lo, dim, n, partials, splits, split_stride);
+    LPP_CHECK_LAUNCH("k_norm_split");
+    return LPP_OK;
+}
+
 // (hi, lo)[t][u] = SwiGLU(W1 x[t], W3 x[t])[u] in one launch: the gate and the up projection of a
 // feature share a workgroup, and the activation is applied to the accumulators.
 lpp_status gate_up_swiglu(const void* w1, const void* w3, int hidden, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad,
@@ -1150,24 +1291,24 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
     int pending = 0;  // ranges of the product before (W2's, then Wo's) still to be added to x
     for (int l = 0; l < c.n_layers; ++l) {
         // attention block, model.cpp:216-218
-        hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
-                           static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, gate,
-                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim);
-        LPP_CHECK_LAUNCH("k_norm_split");
+        LPP_TRY(norm_split(x, static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, t_pad, gate,
+                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s));
+        // What a prefill leaves behind is the cache: the last layer needs its K and V rows only, and
+        // nothing reads what the rest of that layer would compute.
+        const bool last_layer = l == c.n_layers - 1;
         const Product qkv[3] = {{layer_of(LPP_T_WQ, l, dim, dim), q, dim}, {layer_of(LPP_T_WK, l, kv, dim), k, kv},
                                 {layer_of(LPP_T_WV, l, kv, dim), v, kv}};
+        const int q_dim = last_layer ? 0 : dim;
         int qkv_split = 1;
-        LPP_TRY(gemm(qkv, 3, hi, lo, dim, t_pad, false, s, up, room, &qkv_split));
-        const size_t qkv_stride = static_cast<size_t>(t_pad) * (dim + 2 * kv);
+        LPP_TRY(gemm(qkv + (last_layer ? 1 : 0), last_layer ? 2 : 3, hi, lo, dim, t_pad, false, s, up, room, &qkv_split));
+        const size_t qkv_stride = static_cast<size_t>(t_pad) * (q_dim + 2 * kv);
         const float* qs = qkv_split > 1 ? up : q;
-        const float* ks = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * dim : k;
-        const float* vs = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * (dim + kv) : v;
+        const float* ks = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * q_dim : k;
+        const float* vs = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * (q_dim + kv) : v;
         hipLaunchKernelGGL(pf::k_rope_scatter, dim3(n), dim3(256), 0, s, q, qs, ks, vs, m->rope, m->key_cache, m->value_cache, l,
-                           pos0, dim, kv, hs, c.seq_len, qkv_split, qkv_stride);
+                           pos0, q_dim, kv, hs, c.seq_len, qkv_split, qkv_stride);
         LPP_CHECK_LAUNCH("k_rope_scatter");
-        // What a prefill leaves behind is the cache: the last layer's rows are in place here, and nothing
-        // reads what the rest of that layer would compute.
-        if (l == c.n_layers - 1) break;
+        if (last_layer) break;
         // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
         const bool matrix_cores = 32 % m->gqa == 0 && getenv("LPP_PREFILL_VALU_ATTENTION") == nullptr;
         if (matrix_cores) {
@@ -1177,7 +1318,7 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
                                c.seq_len, n_pos, vt_stride);
             LPP_CHECK_LAUNCH("k_transpose_v");
             const int tiles = (n + 32 / m->gqa - 1) / (32 / m->gqa);
-            const dim3 grid((tiles + 3) / 4, c.n_kv_heads);
+            const dim3 grid(tiles, c.n_kv_heads);
             if (hs == 64)
                 hipLaunchKernelGGL(pf::k_attention_mfma<64>, grid, dim3(256), 0, s, q, m->key_cache, vt, hi, lo, l, pos0, dim, kv,
                                    m->gqa, c.seq_len, n, vt_stride);
@@ -1195,10 +1336,8 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         const Product wo = {layer_of(LPP_T_WO, l, dim, dim), x, dim};
         LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s, gate, room, &pending));
         // feed-forward block, model.cpp:221-226
-        hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x,
-                           static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, gate,
-                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim);
-        LPP_CHECK_LAUNCH("k_norm_split");
+        LPP_TRY(norm_split(x, static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, t_pad, gate,
+                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s));
         if (fused_ffn) {
             LPP_TRY(gate_up_swiglu(layer_of(LPP_T_W1, l, hidden, dim), layer_of(LPP_T_W3, l, hidden, dim), hidden, hi, lo, dim, t_pad,
                                    hi2, lo2, s));
