@@ -494,14 +494,14 @@ struct PipeJob {
     int out_ld;
 };
 
-constexpr int kPipeTripK = 64;  // columns per trip
+constexpr int kPipeTripK = 64;  // columns per trip of the narrow tiles; K must be a multiple
 
-template <int kFi, int kTj>
+template <int kFi, int kTj, int kTripK>
 struct PipeShape {
-    static constexpr int kRowBytes = 2 * kPipeTripK;
+    static constexpr int kRowBytes = 2 * kTripK;
     static constexpr int kRowsA = 64 * kFi, kRowsB = 64 * kTj, kRows = kRowsA + 2 * kRowsB;
     static constexpr int kStageBytes = kRows * kRowBytes;
-    static constexpr int kStages = 3 * kStageBytes <= 144 * 1024 ? 3 : 2;
+    static constexpr int kStages = (160 * 1024) / kStageBytes > 5 ? 5 : (160 * 1024) / kStageBytes;
     static constexpr int kLoads = kStageBytes / 4096;  // requests of 1 KiB per wavefront and stage
     static constexpr int kLdsBytes = kStages * kStageBytes;
 };
@@ -526,12 +526,14 @@ __device__ __forceinline__ void swiglu_split4(half_t* hi, half_t* lo, const floa
     *reinterpret_cast<half4_t*>(lo) = half4_t{l[0], l[1], l[2], l[3]};
 }
 
-template <int kFi, int kTj, int kMode>
+template <int kFi, int kTj, int kMode, int kTripK>
 __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
-    typedef PipeShape<kFi, kTj> Shape;
+    typedef PipeShape<kFi, kTj, kTripK> Shape;
     constexpr int kRowsA = Shape::kRowsA, kRowsB = Shape::kRowsB, kStages = Shape::kStages, kLoads = Shape::kLoads;
     constexpr int kStageBytes = Shape::kStageBytes, kRowBytes = Shape::kRowBytes;
-    constexpr int kSteps = kPipeTripK / 16;  // k-steps per trip
+    constexpr int kSteps = kTripK / 16;      // k-steps per trip
+    constexpr int kPieces = kTripK / 8;      // 16-byte pieces of a row
+    constexpr int kSwizzleShift = kPieces == 8 ? 1 : 2;
     extern __shared__ __align__(1024) char pipe_lds[];
     const int lane = lane_id();
     const int wave_of_8 = __builtin_amdgcn_readfirstlane(wave_index());
@@ -553,12 +555,12 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
     constexpr int kFeaturesPerTile = kMode == 2 ? 32 * kFi : 64 * kFi;
     const int f_base = tile_x * kFeaturesPerTile, t_base = token_tile * kRowsB;
 
-    // what each lane requests: request q of this wavefront fills rows 8 (wave + 4 q) .. + 7 of a stage
+    // what each lane requests: request q of this wavefront fills 1 KiB = rows (64 / kPieces) (wave + 4 q) .. of a stage
     const char* src[kLoads];
 #pragma unroll
     for (int q = 0; q < kLoads; ++q) {
-        const int row = 8 * (wave + 4 * q) + (lane >> 3);
-        const int piece = (lane & 7) ^ ((row >> 1) & 7);
+        const int row = (64 / kPieces) * (wave + 4 * q) + lane / kPieces;
+        const int piece = (lane % kPieces) ^ ((row >> kSwizzleShift) & (kPieces - 1));
         const half_t* from;
         if (row < kRowsA) {
             if constexpr (kMode == 2) {
@@ -578,7 +580,7 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
     }
     const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(
         (__attribute__((address_space(3))) char*)pipe_lds));
-    const int trips = job.k_len / kPipeTripK;
+    const int trips = job.k_len / kTripK;
     auto request = [&](int trip) {
         const unsigned at = __builtin_amdgcn_readfirstlane(lds_base + (trip % kStages) * kStageBytes + wave * 1024);
         const int column = __builtin_amdgcn_readfirstlane(trip * kRowBytes);
@@ -591,7 +593,7 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
     int a_off[kSteps], b_off[kSteps];
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-        const int piece = (2 * s + g) ^ ((r >> 1) & 7);
+        const int piece = (2 * s + g) ^ ((r >> kSwizzleShift) & (kPieces - 1));
         a_off[s] = (wf * 32 * kFi + r) * kRowBytes + 16 * piece;
         b_off[s] = (kRowsA + wt * 32 * kTj + r) * kRowBytes + 16 * piece;
     }
@@ -1110,17 +1112,17 @@ struct Product {
     int n;
 };
 
-template <int kFi, int kTj, int kMode>
+template <int kFi, int kTj, int kMode, int kTripK = pf::kPipeTripK>
 lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
-    typedef pf::PipeShape<kFi, kTj> Shape;
+    typedef pf::PipeShape<kFi, kTj, kTripK> Shape;
     static bool sized = false;
     if (!sized) {
-        LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode>),
+        LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLdsBytes));
         sized = true;
     }
     const int per_die = (job.groups + 7) / 8;
-    hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
+    hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
     LPP_CHECK_LAUNCH("k_gemm_pipe");
     return LPP_OK;
 }
@@ -1180,8 +1182,8 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
         job.groups = feature_tiles * splits;
         const bool add_in_kernel = accumulate && splits == 1;
         if (wide) {
-            if (add_in_kernel) LPP_TRY((launch_pipe<4, 2, 1>(job, s)));
-            else LPP_TRY((launch_pipe<4, 2, 0>(job, s)));
+            if (add_in_kernel) LPP_TRY((launch_pipe<4, 2, 1, 32>(job, s)));
+            else LPP_TRY((launch_pipe<4, 2, 0, 32>(job, s)));
         } else {
             if (add_in_kernel) LPP_TRY((launch_pipe<2, 2, 1>(job, s)));
             else LPP_TRY((launch_pipe<2, 2, 0>(job, s)));
@@ -1254,7 +1256,7 @@ lpp_status gate_up_swiglu(const void* w1, const void* w3, int hidden, const pf::
     job.out_hi = out_hi;
     job.out_lo = out_lo;
     job.out_ld = hidden;
-    return launch_pipe<4, 2, 2>(job, s);
+    return launch_pipe<4, 2, 2, 32>(job, s);
 }
 
 // One chunk: tokens[0..n) at positions pos0 .. pos0 + n - 1; n <= kChunk.
