@@ -327,128 +327,6 @@ __global__ __launch_bounds__(256) void k_gemm(const half_t* __restrict__ w, cons
         }
 }
 
-// The same product with the operand tiles staged in LDS (K a multiple of 64).  A trip covers 64
-// columns: the workgroup copies its W, Xh and Xl tiles (rows of 128 bytes, 16 bytes per lane and
-// request, eight lanes per row) into registers while it multiplies the trip before out of LDS,
-// then stores them to LDS between two barriers.  Every byte comes from memory once per workgroup
-// (the direct kernel above fetches each fragment once per wavefront that uses it, and waits for
-// it with nothing else to do); rows are padded to 144 bytes in LDS so that the 32 rows of a
-// fragment do not all start in the same bank.
-//
-// One launch can serve up to three weight matrices that share the activations (Wq, Wk, Wv): the
-// feature tiles of the matrices are numbered one after the other along the grid's x.
-struct GemmOutputs {
-    const half_t* w[3];
-    float* y[3];
-    int ldy[3];
-    int first_tile[3];  // first feature tile of matrix i (first_tile[0] = 0); unused entries = INT_MAX
-    // Split K: workgroup z of the grid multiplies columns [z * k_len, (z + 1) * k_len) and writes its
-    // partial product to y + z * split_stride (rows of K_total columns in w and x; k_len of them used).
-    int k_len;
-    size_t split_stride;
-};
-
-template <bool kAccumulate, int kSub, int kTripK>
-__global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* __restrict__ xh,
-                                                  const half_t* __restrict__ xl, int K) {
-    constexpr int kTile = 64 * kSub;           // rows of each operand tile (features, tokens)
-    const int which = (static_cast<int>(blockIdx.x) >= o3.first_tile[2]) ? 2 : (static_cast<int>(blockIdx.x) >= o3.first_tile[1]) ? 1 : 0;
-    const half_t* __restrict__ w = which == 2 ? o3.w[2] : (which == 1 ? o3.w[1] : o3.w[0]);
-    float* __restrict__ y = which == 2 ? o3.y[2] : (which == 1 ? o3.y[1] : o3.y[0]);
-    const int ldy = which == 2 ? o3.ldy[2] : (which == 1 ? o3.ldy[1] : o3.ldy[0]);
-    const int tile_x = static_cast<int>(blockIdx.x) - (which == 2 ? o3.first_tile[2] : (which == 1 ? o3.first_tile[1] : 0));
-    const int k_first = static_cast<int>(blockIdx.z) * o3.k_len;  // K below is the row length; this workgroup covers k_len columns
-    y += static_cast<size_t>(blockIdx.z) * o3.split_stride;
-    constexpr int kRowBytes = 2 * kTripK + 16;             // a trip's columns of a row + 16 bytes of padding
-    constexpr int kRowChunks = kTripK / 8;                 // 16-byte pieces of it
-    constexpr int kChunks = kTile * kRowChunks / 256;      // pieces per thread and operand
-    __shared__ __align__(16) char tiles[3][kTile * kRowBytes];
-    const int tid = static_cast<int>(threadIdx.x);
-    const int lane = lane_id();
-    const int wave = wave_index();
-    const int f_base = tile_x * kTile, t_base = blockIdx.y * kTile;
-    const int r = lane & 31, g = lane >> 5;
-    const int wf = (wave & 1) * 32 * kSub, wt = (wave >> 1) * 32 * kSub;
-
-    const char* src[3][kChunks];
-    int dst[kChunks];
-#pragma unroll
-    for (int j = 0; j < kChunks; ++j) {
-        const int id = tid + 256 * j, row = id / kRowChunks, c = id % kRowChunks;
-        src[0][j] = reinterpret_cast<const char*>(w + static_cast<size_t>(f_base + row) * K + k_first) + 16 * c;
-        src[1][j] = reinterpret_cast<const char*>(xh + static_cast<size_t>(t_base + row) * K + k_first) + 16 * c;
-        src[2][j] = reinterpret_cast<const char*>(xl + static_cast<size_t>(t_base + row) * K + k_first) + 16 * c;
-        dst[j] = row * kRowBytes + 16 * c;
-    }
-    uintx4 stage[3][kChunks];
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int o = 0; o < 3; ++o)
-#pragma unroll
-            for (int j = 0; j < kChunks; ++j) stage[o][j] = load16(src[o][j] + 2 * static_cast<size_t>(k0));
-    };
-    auto commit = [&]() {
-#pragma unroll
-        for (int o = 0; o < 3; ++o)
-#pragma unroll
-            for (int j = 0; j < kChunks; ++j) *reinterpret_cast<uintx4*>(tiles[o] + dst[j]) = stage[o][j];
-    };
-
-    floatx16 acc[kSub][kSub];
-#pragma unroll
-    for (int i = 0; i < kSub; ++i)
-#pragma unroll
-        for (int j = 0; j < kSub; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-    fetch(0);
-    commit();
-    __syncthreads();
-    for (int k0 = 0; k0 < o3.k_len; k0 += kTripK) {
-        const bool more = k0 + kTripK < o3.k_len;
-        if (more) fetch(k0 + kTripK);
-#pragma unroll
-        for (int s = 0; s < kTripK / 16; ++s) {  // k-steps of 16 columns
-            half8_t a[kSub], bh[kSub], bl[kSub];
-#pragma unroll
-            for (int i = 0; i < kSub; ++i) {
-                a[i] = *reinterpret_cast<const half8_t*>(tiles[0] + (wf + 32 * i + r) * kRowBytes + 32 * s + 16 * g);
-                bh[i] = *reinterpret_cast<const half8_t*>(tiles[1] + (wt + 32 * i + r) * kRowBytes + 32 * s + 16 * g);
-                bl[i] = *reinterpret_cast<const half8_t*>(tiles[2] + (wt + 32 * i + r) * kRowBytes + 32 * s + 16 * g);
-            }
-#pragma unroll
-            for (int i = 0; i < kSub; ++i)
-#pragma unroll
-                for (int j = 0; j < kSub; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bh[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bl[j], acc[i][j], 0, 0, 0);
-                }
-        }
-        __syncthreads();  // every wavefront has read this trip's tiles
-        if (more) {
-            commit();
-            __syncthreads();
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < kSub; ++i)
-#pragma unroll
-        for (int j = 0; j < kSub; ++j) {
-            float* row = y + static_cast<size_t>(t_base + wt + 32 * j + r) * ldy + f_base + wf + 32 * i + 4 * g;
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-                floatx4* out = reinterpret_cast<floatx4*>(row + 8 * e4);
-                floatx4 v = floatx4{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
-                if constexpr (kAccumulate) {
-                    const floatx4 old = *out;
-                    v = floatx4{old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
-                }
-                *out = v;
-            }
-        }
-}
-
 // The same product as a pipeline of LDS stages filled by the memory system itself.
 //
 // A workgroup is eight wavefronts: four that multiply and four that only request data.  A request
@@ -460,16 +338,18 @@ __global__ __launch_bounds__(256) void k_gemm_lds(GemmOutputs o3, const half_t* 
 // The four multiplying wavefronts (2 x 2) own a tile of 64 kFi features x 64 kTj tokens; a wavefront
 // owns 32 kFi x 32 kTj of it (kFi x kTj MFMA tiles: the weight side is the longer one, because the
 // activations come twice, as head and remainder, and every fragment is read from LDS once per
-// wavefront that uses it).  A trip covers 64 columns = four k-steps of 16: the rows of the three
-// operand tiles, 128 bytes each (a whole cache line per row and trip), lie one after the other
-// in a stage of LDS, and a wavefront fills 8 rows with one global_load_lds_dwordx4 (lane i -> 16
-// bytes at M0 + 16 i): no registers are staged and nothing waits for the data but the s_waitcnt
-// of the trip that multiplies it.
+// wavefront that uses it).  A trip covers kTripK columns (64 = a whole cache line per row and
+// trip, or 32 where 64 would leave room for two stages only): the rows of the three operand
+// tiles lie one after the other in a stage of LDS, and a requesting wavefront fills 1 KiB of it
+// with one global_load_lds_dwordx4 (lane i -> 16 bytes at M0 + 16 i): no registers are staged
+// and nothing waits for the data but the s_waitcnt ahead of the trip that multiplies it.  As
+// many stages as 160 KiB hold, five at most.
 //
 // LDS banks: a fragment read takes 16 bytes per lane from 32 consecutive rows; with rows of 128
-// bytes every second row starts in the same bank, so the eight 16-byte pieces of row r are stored
-// in the order piece ^ ((r >> 1) & 7): 16 consecutive lanes then cover all 64 banks once.  The
-// permutation is applied on the way in, by the address each lane requests.
+// (64) bytes every second (fourth) row starts in the same bank, so the 16-byte pieces of row r
+// are stored in the order piece ^ ((r >> 1) & 7) (piece ^ ((r >> 2) & 3)): 16 consecutive lanes then
+// cover all 64 banks once.  The permutation is applied on the way in, by the address each lane
+// requests.
 //
 // The requests are inline assembly: written with the builtin, every LDS read of the loop would
 // wait for all outstanding requests (they may alias), which is the pipeline's whole depth.
