@@ -995,11 +995,13 @@ struct Product {
 template <int kFi, int kTj, int kMode, int kTripK = pf::kPipeTripK>
 lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
     typedef pf::PipeShape<kFi, kTj, kTripK> Shape;
-    static bool sized = false;
-    if (!sized) {
+    static bool sized[64] = {};  // (per device: the attribute belongs to the device's copy of the kernel)
+    int device = 0;
+    LPP_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= 64 || !sized[device]) {
         LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLdsBytes));
-        sized = true;
+        if (device >= 0 && device < 64) sized[device] = true;
     }
     const int per_die = (job.groups + 7) / 8;
     hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
