@@ -721,40 +721,25 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
 //   online softmax: in the result a LANE holds one query row (its column) and 16 of the block's 32
 //                   positions, the lane 32 further on the other 16 -- maximum, sum and rescaling are
 //                   per lane, with one exchange between the two halves of the wavefront
-//   O^T[d][row] += sum_pos V^T[d][pos] P^T[pos][row]   A = V transposed (k_transpose_v keeps a copy
-//                                                      of the layer's V with positions contiguous),
+//   O^T[d][row] += sum_pos V^T[d][pos] P^T[pos][row]   A = V transposed: the wavefront loads its block of
+//                                                      V as the cache holds it (a position's row at a
+//                                                      time, 16 bytes a lane), writes it into a tile of
+//                                                      LDS of its own with positions contiguous, and
+//                                                      reads its fragments from there,
 //                                                      B = P straight from the lane's own registers
 // A lane's 16 positions of a block are {8j + 4g .. 8j + 4g + 3 : j = 0..3} (g = lane / 32), so as
 // B operand of the second product it supplies, per 16-position step, positions 4g..4g+3 and
-// 8+4g..8+4g+3; the V^T fragment is loaded in the same order (two 8-byte loads).  Any such
+// 8+4g..8+4g+3; the V^T fragment is read in the same order (two 8-byte reads).  Any such
 // permutation of k is fine as long as both operands use it.
 // Probabilities and queries are split into binary16 head + remainder like every other activation.
-
-// vt[kvh][d][p] = V[kvh][p][d] of `layer` for p < n_pos, zero for n_pos <= p < vt_stride.
-__global__ __launch_bounds__(256) void k_transpose_v(const uint16_t* __restrict__ value_cache, uint16_t* __restrict__ vt,
-                                                     int layer, int kv_dim, int hs, int seq_len, int n_pos, int vt_stride) {
-    __shared__ uint16_t tile[32][128 + 2];
-    const int p0 = blockIdx.x * 32, kvh = blockIdx.y;
-    const uint16_t* src = value_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * hs;
-    for (int idx = threadIdx.x; idx < 32 * hs; idx += blockDim.x) {
-        const int p = idx / hs, d = idx - p * hs;
-        tile[p][d] = (p0 + p < n_pos) ? src[static_cast<size_t>(p0 + p) * hs + d] : static_cast<uint16_t>(0);
-    }
-    __syncthreads();
-    uint16_t* dst = vt + static_cast<size_t>(kvh) * hs * vt_stride;
-    for (int idx = threadIdx.x; idx < 32 * hs; idx += blockDim.x) {
-        const int d = idx >> 5, p = idx & 31;
-        dst[static_cast<size_t>(d) * vt_stride + p0 + p] = tile[p][d];
-    }
-}
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 template <int kHs>
 __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict__ q, const uint16_t* __restrict__ key_cache,
-                                                        const uint16_t* __restrict__ vt, half_t* __restrict__ out_hi,
+                                                        const uint16_t* __restrict__ value_cache, half_t* __restrict__ out_hi,
                                                         half_t* __restrict__ out_lo, int layer, int pos0, int dim, int kv_dim,
-                                                        int gqa, int seq_len, int n_tokens, int vt_stride) {
+                                                        int gqa, int seq_len, int n_tokens) {
     constexpr int kDTiles = kHs / 32, kKSteps = kHs / 16;
     const int lane = lane_id(), wave = wave_index();
     const int r = lane & 31, g = lane >> 5;
@@ -769,7 +754,12 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     const int limit = pos0 + last_tok + 1;    // positions the tile reads: [0, limit)
     const int my_limit = pos0 + tok_c + 1;    // positions this lane's row attends to: [0, my_limit)
     const uint16_t* kbase = key_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * kHs;
-    const uint16_t* vtb = vt + static_cast<size_t>(kvh) * kHs * vt_stride;
+    const uint16_t* vbase = value_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * kHs;
+    // this wavefront's tile of V^T: [d][32 positions], rows 72 bytes apart (8-byte reads, few shared banks)
+    constexpr int kTileRow = 36;  // binary16 per row
+    __shared__ __align__(16) uint16_t vt_tiles[4][kHs * kTileRow];
+    uint16_t* vt_tile = vt_tiles[wave];
+    constexpr int kVChunks = kHs / 16;  // 16-byte pieces of the block's V rows per lane
     const float scale = 1.0f / sqrtf(static_cast<float>(kHs));  // model.cpp:188
 
     half8_t qh[kKSteps], ql[kKSteps];
@@ -809,16 +799,14 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         half8_t kf[kKSteps];
 #pragma unroll
         for (int s = 0; s < kKSteps; ++s) kf[s] = k_next[s];
-        half8_t vf[kDTiles][2];
+        // this block's V rows: piece c of the block = 8 dimensions of one position (zero past the context)
+        uintx4 vrows[kVChunks];
 #pragma unroll
-        for (int dt = 0; dt < kDTiles; ++dt)
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2) {
-                const uint16_t* vrow = vtb + static_cast<size_t>(32 * dt + r) * vt_stride + p0 + 16 * s2 + 4 * g;
-                const half4_t a0 = *reinterpret_cast<const half4_t*>(vrow);
-                const half4_t a1 = *reinterpret_cast<const half4_t*>(vrow + 8);
-                vf[dt][s2] = half8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-            }
+        for (int i = 0; i < kVChunks; ++i) {
+            const int c = lane + 64 * i, p = c / (kHs / 8), d0 = (c % (kHs / 8)) * 8;
+            const int pos = p0 + p;
+            vrows[i] = pos < limit ? load16(vbase + static_cast<size_t>(pos) * kHs + d0) : uintx4{0u, 0u, 0u, 0u};
+        }
         if (p0 + 128 < limit) fetch_k(k_next, p0 + 128);
 #pragma unroll
         for (int s = 0; s < kKSteps; ++s) {
@@ -849,14 +837,27 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         block_sum += __shfl_xor(block_sum, 32);
         lsum = lsum * corr + block_sum;
         top = grown;
+        // V rows into the tile, a position's 8 dimensions down a column; the LDS serves a wavefront's accesses
+        // in order, so the fragment reads below see them (and the next block's writes come after these reads)
+#pragma unroll
+        for (int i = 0; i < kVChunks; ++i) {
+            const int c = lane + 64 * i, p = c / (kHs / 8), d0 = (c % (kHs / 8)) * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                vt_tile[(d0 + e) * kTileRow + p] = static_cast<uint16_t>(vrows[i][e >> 1] >> (16 * (e & 1)));
+        }
 #pragma unroll
         for (int dt = 0; dt < kDTiles; ++dt) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[dt][s2], ph[s2], o[dt], 0, 0, 0);
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[dt][s2], pl[s2], o[dt], 0, 0, 0);
+                const uint16_t* vrow = vt_tile + (32 * dt + r) * kTileRow + 16 * s2 + 4 * g;
+                const half4_t a0 = *reinterpret_cast<const half4_t*>(vrow);
+                const half4_t a1 = *reinterpret_cast<const half4_t*>(vrow + 8);
+                const half8_t vf = half8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, ph[s2], o[dt], 0, 0, 0);
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pl[s2], o[dt], 0, 0, 0);
             }
         }
     }
@@ -941,7 +942,7 @@ __global__ __launch_bounds__(256) void k_split(const float* __restrict__ x, half
 namespace {
 
 // Buffers of a chunk of t_pad tokens, in lpp_model::pf_buf order.
-enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufVt, kBufHi2, kBufLo2, kBufCount };
+enum { kBufTokens, kBufX, kBufQ, kBufK, kBufV, kBufGate, kBufUp, kBufHi, kBufLo, kBufHi2, kBufLo2, kBufCount };
 static_assert(kBufCount <= static_cast<int>(sizeof(lpp_model::pf_buf) / sizeof(void*)), "lpp_model::pf_buf is too small");
 
 const char* unsupported_reason(const lpp_model* m) {
@@ -969,8 +970,6 @@ lpp_status ensure_scratch(lpp_model* m, int t_pad) {
                                      t * c.hidden_dim * sizeof(float),
                                      t * widest * sizeof(pf::half_t),
                                      t * widest * sizeof(pf::half_t),
-                                     // one layer's V with positions contiguous: [kv_dim][seq_len rounded up to 32]
-                                     static_cast<size_t>(m->kv_dim) * ((c.seq_len + 31) / 32 * 32) * sizeof(uint16_t),
                                      // the feed-forward activations, written while hi/lo are still being read
                                      t * c.hidden_dim * sizeof(pf::half_t),
                                      t * c.hidden_dim * sizeof(pf::half_t)};
@@ -1196,19 +1195,14 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
         const bool matrix_cores = 32 % m->gqa == 0 && getenv("LPP_PREFILL_VALU_ATTENTION") == nullptr;
         if (matrix_cores) {
-            const int n_pos = pos0 + n, vt_stride = (n_pos + 31) / 32 * 32;
-            uint16_t* vt = static_cast<uint16_t*>(m->pf_buf[kBufVt]);
-            hipLaunchKernelGGL(pf::k_transpose_v, dim3(vt_stride / 32, c.n_kv_heads), dim3(256), 0, s, m->value_cache, vt, l, kv, hs,
-                               c.seq_len, n_pos, vt_stride);
-            LPP_CHECK_LAUNCH("k_transpose_v");
             const int tiles = (n + 32 / m->gqa - 1) / (32 / m->gqa);
             const dim3 grid(tiles, c.n_kv_heads);
             if (hs == 64)
-                hipLaunchKernelGGL(pf::k_attention_mfma<64>, grid, dim3(256), 0, s, q, m->key_cache, vt, hi, lo, l, pos0, dim, kv,
-                                   m->gqa, c.seq_len, n, vt_stride);
+                hipLaunchKernelGGL(pf::k_attention_mfma<64>, grid, dim3(256), 0, s, q, m->key_cache, m->value_cache, hi, lo, l, pos0,
+                                   dim, kv, m->gqa, c.seq_len, n);
             else
-                hipLaunchKernelGGL(pf::k_attention_mfma<128>, grid, dim3(256), 0, s, q, m->key_cache, vt, hi, lo, l, pos0, dim, kv,
-                                   m->gqa, c.seq_len, n, vt_stride);
+                hipLaunchKernelGGL(pf::k_attention_mfma<128>, grid, dim3(256), 0, s, q, m->key_cache, m->value_cache, hi, lo, l, pos0,
+                                   dim, kv, m->gqa, c.seq_len, n);
             LPP_CHECK_LAUNCH("k_attention_mfma");
         } else if (hs == 64)
             hipLaunchKernelGGL(pf::k_attention<8>, dim3((n + 3) / 4, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache,
