@@ -203,14 +203,15 @@ def test_run_with_batched_prefill_matches_run(temperature):
     m.close()
 
 
-def test_prefill_at_full_size_against_decode():
-    """Llama-3.2-1B shape: 300 prompt ids; caches and the next steps' logits against the
-    same model prefilled by decode."""
-    shape = CONFIGS["c3_llama32_1b_fp16"]
+@pytest.mark.parametrize("config,n", [("c3_llama32_1b_fp16", 300), ("c2_tinyllama_1b_fp16", 200), ("c5_llama3_8b_fp16", 140)])
+def test_prefill_at_full_size_against_decode(config, n):
+    """The benchmark shapes (1B: 300 prompt ids; TinyLlama: 44 feature tiles of the fused gate/up launch, not a
+    multiple of the eight dies; 8B: head size 128, hidden 14336): caches and the next steps' logits
+    against the same model prefilled by decode."""
+    shape = CONFIGS[config]
     a = Model(shape)
     a.load_synthetic(1)
     a.set_path(capi.PATH_PERSISTENT)
-    n = 300
     prompt = capi.synth_token_ids(n, 4, shape.vocab_size)
     decode_prompt(a, prompt)
     la = []
@@ -229,8 +230,9 @@ def test_prefill_at_full_size_against_decode():
         scale = np.abs(y).max()
         assert np.all(np.abs(x - y) <= np.maximum(np.abs(y) * 2.0 ** -9, scale * 2.0 ** -11))
         # (16 layers deep the two summation orders differ by about 1e-4 relative, a fifth of a binary16
-        # step: about that share of the entries rounds to the neighbouring value, none further)
-        assert np.mean(x == y) > 0.6
+        # step: about that share of the entries rounds to the neighbouring value, none further; 32 layers
+        # deep the share that rounds the same way is 57 %)
+        assert np.mean(x == y) > (0.6 if shape.n_layers <= 22 else 0.45)
     tok = int(prompt[-1])
     for pos, (want_tok, want) in zip(range(n, n + 4), la):
         got_tok = b.forward(tok, pos, 0.0)
