@@ -991,17 +991,24 @@ struct Product {
     int n;
 };
 
-template <int kFi, int kTj, int kMode, int kTripK = pf::kPipeTripK>
-lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
-    typedef pf::PipeShape<kFi, kTj, kTripK> Shape;
-    static bool sized[64] = {};  // (per device: the attribute belongs to the device's copy of the kernel)
+// The kernel's LDS need, told to the runtime once per device (the attribute belongs to the device's copy of the kernel).
+template <int kFi, int kTj, int kMode, int kTripK>
+lpp_status size_pipe() {
+    static bool sized[64] = {};
     int device = 0;
     LPP_HIP(hipGetDevice(&device));
     if (device < 0 || device >= 64 || !sized[device]) {
         LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, Shape::kLdsBytes));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, pf::PipeShape<kFi, kTj, kTripK>::kLdsBytes));
         if (device >= 0 && device < 64) sized[device] = true;
     }
+    return LPP_OK;
+}
+
+template <int kFi, int kTj, int kMode, int kTripK = pf::kPipeTripK>
+lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
+    typedef pf::PipeShape<kFi, kTj, kTripK> Shape;
+    LPP_TRY((size_pipe<kFi, kTj, kMode, kTripK>()));
     const int per_die = (job.groups + 7) / 8;
     hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
     LPP_CHECK_LAUNCH("k_gemm_pipe");
@@ -1330,6 +1337,12 @@ lpp_status scratch_address(void** out) {
 }  // namespace
 
 lpp_status prefill_gemm_scratch_setup() {
+    // (everything the allocation-free entry point would otherwise set up on its first call: a caller under
+    // graph capture finds it done)
+    LPP_TRY((size_pipe<4, 2, 0, 32>()));
+    LPP_TRY((size_pipe<4, 2, 1, 32>()));
+    LPP_TRY((size_pipe<2, 2, 0, pf::kPipeTripK>()));
+    LPP_TRY((size_pipe<2, 2, 1, pf::kPipeTripK>()));
     void* p = nullptr;
     return scratch_address(&p);
 }
