@@ -396,7 +396,9 @@ __device__ __forceinline__ void swiglu_split4(half_t* hi, half_t* lo, const floa
     half_t h[4], l[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const float sigma = 1.0f / (1.0f + expf(-g[e]));
+        // (v_exp_f32 and v_rcp_f32, an ulp each: 64 of these per lane follow every tile, and what they feed is
+        // rounded to binary16 + remainder right below)
+        const float sigma = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g[e] * -1.44269504088896341f));
         const float v = (g[e] * sigma) * u[e];
         h[e] = static_cast<half_t>(v);
         l[e] = static_cast<half_t>(v - static_cast<float>(h[e]));
