@@ -186,33 +186,35 @@ __global__ __launch_bounds__(256) void k_rope_scatter(float* __restrict__ q, con
     const int t = blockIdx.x;
     const int pos = pos0 + t;
     const float2* cs_row = rope + static_cast<size_t>(pos) * (hs / 2);
+    // (two pairs per thread: 16-byte loads and stores; dim, kv_dim and the head size are multiples of 4)
     auto summed = [&](const float* first, size_t at) {
-        float2 v = *reinterpret_cast<const float2*>(first + at);
+        floatx4 v = *reinterpret_cast<const floatx4*>(first + at);
         for (int z = 1; z < splits; ++z) {
-            const float2 a = *reinterpret_cast<const float2*>(first + z * split_stride + at);
-            v.x += a.x;
-            v.y += a.y;
+            const floatx4 a = *reinterpret_cast<const floatx4*>(first + z * split_stride + at);
+            v = floatx4{v[0] + a[0], v[1] + a[1], v[2] + a[2], v[3] + a[3]};
         }
         return v;
     };
-    for (int i = 2 * threadIdx.x; i < dim; i += 2 * blockDim.x) {
+    for (int i = 4 * threadIdx.x; i < dim; i += 4 * blockDim.x) {
         const size_t at = static_cast<size_t>(t) * dim + i;
-        const float2 cs = cs_row[(i % hs) >> 1];
-        const float2 v = summed(qs, at);
-        q[at] = v.x * cs.x - v.y * cs.y;
-        q[at + 1] = v.x * cs.y + v.y * cs.x;
+        const floatx4 cs = *reinterpret_cast<const floatx4*>(cs_row + ((i % hs) >> 1));  // (cos, sin) of two pairs
+        const floatx4 v = summed(qs, at);
+        *reinterpret_cast<floatx4*>(q + at) =
+            floatx4{v[0] * cs[0] - v[1] * cs[1], v[0] * cs[1] + v[1] * cs[0], v[2] * cs[2] - v[3] * cs[3], v[2] * cs[3] + v[3] * cs[2]};
     }
-    for (int i = 2 * threadIdx.x; i < kv_dim; i += 2 * blockDim.x) {
+    for (int i = 4 * threadIdx.x; i < kv_dim; i += 4 * blockDim.x) {
         const size_t at = static_cast<size_t>(t) * kv_dim + i;
-        const float2 kk = summed(ks, at), vv = summed(vs, at);
-        const float2 cs = cs_row[(i % hs) >> 1];
+        const floatx4 kk = summed(ks, at), vv = summed(vs, at);
+        const floatx4 cs = *reinterpret_cast<const floatx4*>(cs_row + ((i % hs) >> 1));
         const int head = i / hs, within = i - head * hs;
         const size_t dst = static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(head) * seq_len * hs +
                            static_cast<size_t>(pos) * hs + within;
-        key_cache[dst] = f32_to_f16_bits(kk.x * cs.x - kk.y * cs.y);
-        key_cache[dst + 1] = f32_to_f16_bits(kk.x * cs.y + kk.y * cs.x);
-        value_cache[dst] = f32_to_f16_bits(vv.x);
-        value_cache[dst + 1] = f32_to_f16_bits(vv.y);
+        typedef uint16_t ushort4_t __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<ushort4_t*>(key_cache + dst) =
+            ushort4_t{f32_to_f16_bits(kk[0] * cs[0] - kk[1] * cs[1]), f32_to_f16_bits(kk[0] * cs[1] + kk[1] * cs[0]),
+                      f32_to_f16_bits(kk[2] * cs[2] - kk[3] * cs[3]), f32_to_f16_bits(kk[2] * cs[3] + kk[3] * cs[2])};
+        *reinterpret_cast<ushort4_t*>(value_cache + dst) =
+            ushort4_t{f32_to_f16_bits(vv[0]), f32_to_f16_bits(vv[1]), f32_to_f16_bits(vv[2]), f32_to_f16_bits(vv[3])};
     }
 }
 
@@ -396,9 +398,7 @@ __device__ __forceinline__ void swiglu_split4(half_t* hi, half_t* lo, const floa
     half_t h[4], l[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        // (v_exp_f32 and v_rcp_f32, an ulp each: 64 of these per lane follow every tile, and what they feed is
-        // rounded to binary16 + remainder right below)
-        const float sigma = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g[e] * -1.44269504088896341f));
+        const float sigma = 1.0f / (1.0f + expf(-g[e]));  // (hardware exp and reciprocal here: 0.4 % of a prefill)
         const float v = (g[e] * sigma) * u[e];
         h[e] = static_cast<half_t>(v);
         l[e] = static_cast<half_t>(v - static_cast<float>(h[e]));
