@@ -165,8 +165,8 @@ def bench_prefill(args, model, shape, name, cus) -> int:
         print("bench.py: the batched prefill does not take this model", file=sys.stderr)
         return 2
     ids = capi.synth_token_ids(n, SEED + 1, shape.vocab_size)
-    reps = args.steps if args.steps is not None else 10
-    for _ in range(max(args.warmup if args.warmup != 16 else 2, 1)):
+    reps = args.steps if args.steps is not None else 30
+    for _ in range(max(args.warmup if args.warmup != 16 else 3, 1)):
         model.prefill(ids, 0)
     capi.synchronize()
     t0 = time.perf_counter()
@@ -181,7 +181,7 @@ def bench_prefill(args, model, shape, name, cus) -> int:
     att_flops = 4.0 * (L - 1) * shape.n_heads * shape.head_size * n * (n + 1) / 2
     tflops = (gemm_flops + att_flops) / sec / 1e12
     out = dict(metric="batched prefill, prompt ids/s, " + args.config, value=round(n / sec, 1), unit="tok/s", n_gpus=1,
-               steps=reps, warmup=2, ms_per_step=round(sec * 1e3, 3), higher_is_better=True, scaling="weak",
+               steps=reps, warmup=max(args.warmup if args.warmup != 16 else 3, 1), ms_per_step=round(sec * 1e3, 3), higher_is_better=True, scaling="weak",
                vs_baseline=None, dtype="f32 accumulate over f16 weights, activations split hi+lo", data="synthetic",
                config=dict(workload=args.config, prompt_ids=n, chunk=512),
                roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
