@@ -108,68 +108,71 @@ __global__ __launch_bounds__(256) void k_norm_split(float* __restrict__ x, const
     }
 }
 
-// The same with a wavefront per row and the row in registers (dim = 256 kChunks): one pass over
-// the memory, no barrier.  The sum of squares runs over the lane's elements in order, then across
-// the lanes.
-template <int kChunks>
-__global__ __launch_bounds__(256) void k_norm_split_rows(float* __restrict__ x, const float* __restrict__ gain,
+// The same with a workgroup per row (dim = 1024 kPer) and the number of partial products known to
+// the compiler: a thread's kPer x (1 + kSplits) loads are all requested before the first is used, so
+// a row costs one round trip to memory and is read once.  Residual sum in the same order; the sum of squares runs over a thread's elements in
+// order, across the lanes, then over the four wavefronts as (0 + 1) + (2 + 3).
+template <int kPer, int kSplits>
+__global__ __launch_bounds__(256) void k_norm_split_wide(float* __restrict__ x, const float* __restrict__ gain,
                                                          half_t* __restrict__ hi, half_t* __restrict__ lo, int n_tokens,
-                                                         int rows, const float* __restrict__ partials, int splits,
-                                                         size_t split_stride) {
+                                                         const float* __restrict__ partials, size_t split_stride) {
 #pragma clang fp contract(off)
-    constexpr int kDim = 256 * kChunks;
-    const int lane = lane_id();
-    const int t = static_cast<int>(blockIdx.x) * 4 + wave_index();
-    if (t >= rows) return;
-    const size_t row = static_cast<size_t>(t) * kDim;
+    constexpr int kDim = 1024 * kPer;
+    __shared__ float scratch[4];
     typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    const int t = blockIdx.x;
+    const size_t row = static_cast<size_t>(t) * kDim;
+    const int first = 4 * threadIdx.x;
     if (t >= n_tokens) {
         const half4_t zero = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
 #pragma unroll
-        for (int c = 0; c < kChunks; ++c) {
-            *reinterpret_cast<half4_t*>(hi + row + 256 * c + 4 * lane) = zero;
-            *reinterpret_cast<half4_t*>(lo + row + 256 * c + 4 * lane) = zero;
+        for (int c = 0; c < kPer; ++c) {
+            *reinterpret_cast<half4_t*>(hi + row + 1024 * c + first) = zero;
+            *reinterpret_cast<half4_t*>(lo + row + 1024 * c + first) = zero;
         }
         return;
     }
-    floatx4 v[kChunks];
+    floatx4 v[kPer], a[kSplits > 0 ? kSplits : 1][kPer], gn[kPer];
 #pragma unroll
-    for (int c = 0; c < kChunks; ++c) v[c] = *reinterpret_cast<const floatx4*>(x + row + 256 * c + 4 * lane);
-    if (splits > 0) {
-        for (int z = 0; z < splits; ++z) {
+    for (int c = 0; c < kPer; ++c) v[c] = *reinterpret_cast<const floatx4*>(x + row + 1024 * c + first);
 #pragma unroll
-            for (int c = 0; c < kChunks; ++c) {
-                const floatx4 a = *reinterpret_cast<const floatx4*>(partials + z * split_stride + row + 256 * c + 4 * lane);
-                v[c] = floatx4{v[c][0] + a[0], v[c][1] + a[1], v[c][2] + a[2], v[c][3] + a[3]};
-            }
+    for (int z = 0; z < kSplits; ++z)
+#pragma unroll
+        for (int c = 0; c < kPer; ++c) a[z][c] = *reinterpret_cast<const floatx4*>(partials + z * split_stride + row + 1024 * c + first);
+#pragma unroll
+    for (int c = 0; c < kPer; ++c) gn[c] = *reinterpret_cast<const floatx4*>(gain + 1024 * c + first);
+    if (kSplits > 0) {
+#pragma unroll
+        for (int c = 0; c < kPer; ++c) {
+#pragma unroll
+            for (int z = 0; z < kSplits; ++z)
+                v[c] = floatx4{v[c][0] + a[z][c][0], v[c][1] + a[z][c][1], v[c][2] + a[z][c][2], v[c][3] + a[z][c][3]};
+            *reinterpret_cast<floatx4*>(x + row + 1024 * c + first) = v[c];
         }
-#pragma unroll
-        for (int c = 0; c < kChunks; ++c) *reinterpret_cast<floatx4*>(x + row + 256 * c + 4 * lane) = v[c];
     }
     float ss = 0.0f;
 #pragma unroll
-    for (int c = 0; c < kChunks; ++c) {
+    for (int c = 0; c < kPer; ++c) {
         ss += v[c][0] * v[c][0];
         ss += v[c][1] * v[c][1];
         ss += v[c][2] * v[c][2];
         ss += v[c][3] * v[c][3];
     }
-    ss = wave_sum(ss);
+    ss = block_sum256(ss, scratch);
     ss /= static_cast<float>(kDim);
     ss += 1e-5f;
     const float scale = 1.0f / sqrtf(ss);
 #pragma unroll
-    for (int c = 0; c < kChunks; ++c) {
-        const floatx4 gn = *reinterpret_cast<const floatx4*>(gain + 256 * c + 4 * lane);
+    for (int c = 0; c < kPer; ++c) {
         half4_t h, l;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float y = v[c][e] * scale * gn[e];
+            const float y = v[c][e] * scale * gn[c][e];
             h[e] = static_cast<half_t>(y);
             l[e] = static_cast<half_t>(y - static_cast<float>(h[e]));
         }
-        *reinterpret_cast<half4_t*>(hi + row + 256 * c + 4 * lane) = h;
-        *reinterpret_cast<half4_t*>(lo + row + 256 * c + 4 * lane) = l;
+        *reinterpret_cast<half4_t*>(hi + row + 1024 * c + first) = h;
+        *reinterpret_cast<half4_t*>(lo + row + 1024 * c + first) = l;
     }
 }
 
@@ -393,19 +396,18 @@ __device__ __forceinline__ void wait_requests() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCount) : "memory");
 }
 
-__device__ __forceinline__ void swiglu_split4(half_t* hi, half_t* lo, const float* g, const float* u) {
+typedef _Float16 half4_pf_t __attribute__((ext_vector_type(4)));
+
+// (hi, lo) = SwiGLU of four (gate, up) pairs, ops.cpp:78-87
+__device__ __forceinline__ void swiglu_split4(half4_pf_t& hi, half4_pf_t& lo, const float* g, const float* u) {
 #pragma clang fp contract(off)
-    half_t h[4], l[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const float sigma = 1.0f / (1.0f + expf(-g[e]));  // (hardware exp and reciprocal here: 0.4 % of a prefill)
         const float v = (g[e] * sigma) * u[e];
-        h[e] = static_cast<half_t>(v);
-        l[e] = static_cast<half_t>(v - static_cast<float>(h[e]));
+        hi[e] = static_cast<half_t>(v);
+        lo[e] = static_cast<half_t>(v - static_cast<float>(hi[e]));
     }
-    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-    *reinterpret_cast<half4_t*>(hi) = half4_t{h[0], h[1], h[2], h[3]};
-    *reinterpret_cast<half4_t*>(lo) = half4_t{l[0], l[1], l[2], l[3]};
 }
 
 template <int kFi, int kTj, int kMode, int kTripK>
@@ -558,34 +560,68 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    // D[m][n]: a lane holds column n = lane % 32 (a token) and rows m = 8 (e / 4) + 4 (lane / 32) + e % 4 (features)
+    // D[m][n]: a lane holds column n = lane % 32 (a token) and rows m = 8 (e / 4) + 4 (lane / 32) + e % 4 (features):
+    // stored from there, an instruction would write 16 or 32 bytes to each of 32 rows of the output.  Every 32 x 32
+    // tile therefore passes through LDS, [token][feature], and leaves as whole 128-byte lines, eight lanes to a
+    // token's row.  The room is the wavefront's quarter of a stage that neither the last trip nor the read past
+    // it uses; a wavefront's LDS accesses are served in order, so no barrier is needed between a tile's writes, its
+    // reads and the next tile's writes.
+    static_assert(kStages >= 3 && kStageBytes / 4 >= 32 * 144, "room for a transposed tile per wavefront");
+    char* room = pipe_lds + ((trips + 1) % kStages) * kStageBytes + wave * (kStageBytes / 4);
+    const int row8 = lane >> 3, part8 = lane & 7;
     if constexpr (kMode == 2) {
+        static_assert(kFi == 4, "a wavefront's gate and up tiles: two of each");
+        typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+        constexpr int kPitch = 72;  // binary16 per token row of the transposed tile: 64 features + padding
+        half_t* tile = reinterpret_cast<half_t*>(room);
 #pragma unroll
-        for (int i = 0; i < kFi / 2; ++i)
+        for (int j = 0; j < kTj; ++j) {
+            half4_t h[2][4], l[2][4];
 #pragma unroll
-            for (int j = 0; j < kTj; ++j) {
-                const size_t at = static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j + r) * job.out_ld + f_base + wf * 16 * kFi +
-                                  32 * i + 4 * g;
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
                     const float gate[4] = {acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
-                    const float up[4] = {acc[i + kFi / 2][j][4 * e4], acc[i + kFi / 2][j][4 * e4 + 1],
-                                         acc[i + kFi / 2][j][4 * e4 + 2], acc[i + kFi / 2][j][4 * e4 + 3]};
-                    swiglu_split4(job.out_hi + at + 8 * e4, job.out_lo + at + 8 * e4, gate, up);
+                    const float up[4] = {acc[i + 2][j][4 * e4], acc[i + 2][j][4 * e4 + 1], acc[i + 2][j][4 * e4 + 2],
+                                         acc[i + 2][j][4 * e4 + 3]};
+                    swiglu_split4(h[i][e4], l[i][e4], gate, up);
+                }
+            const size_t at = static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j) * job.out_ld + f_base + wf * 64 + 8 * part8;
+#pragma unroll
+            for (int part = 0; part < 2; ++part) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4)
+                        *reinterpret_cast<half4_t*>(tile + r * kPitch + 32 * i + 8 * e4 + 4 * g) = part == 0 ? h[i][e4] : l[i][e4];
+                half_t* out = part == 0 ? job.out_hi : job.out_lo;
+#pragma unroll
+                for (int pass = 0; pass < 4; ++pass) {
+                    const int n = 8 * pass + row8;
+                    *reinterpret_cast<half8_t*>(out + at + static_cast<size_t>(n) * job.out_ld) =
+                        *reinterpret_cast<const half8_t*>(tile + n * kPitch + 8 * part8);
                 }
             }
+        }
     } else {
+        constexpr int kPitch = 36;  // floats per token row of the transposed tile: 32 features + padding
+        float* tile = reinterpret_cast<float*>(room);
         float* __restrict__ y = (which == 2 ? job.y[2] : (which == 1 ? job.y[1] : job.y[0])) + static_cast<size_t>(split) * job.split_stride;
         const int ldy = which == 2 ? job.ldy[2] : (which == 1 ? job.ldy[1] : job.ldy[0]);
 #pragma unroll
         for (int i = 0; i < kFi; ++i)
 #pragma unroll
             for (int j = 0; j < kTj; ++j) {
-                float* row = y + static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j + r) * ldy + f_base + wf * 32 * kFi + 32 * i + 4 * g;
 #pragma unroll
-                for (int e4 = 0; e4 < 4; ++e4) {
-                    floatx4* out = reinterpret_cast<floatx4*>(row + 8 * e4);
-                    floatx4 v = floatx4{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                for (int e4 = 0; e4 < 4; ++e4)
+                    *reinterpret_cast<floatx4*>(tile + r * kPitch + 8 * e4 + 4 * g) =
+                        floatx4{acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]};
+                float* first = y + static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j) * ldy + f_base + wf * 32 * kFi + 32 * i + 4 * part8;
+#pragma unroll
+                for (int pass = 0; pass < 4; ++pass) {
+                    const int n = 8 * pass + row8;
+                    floatx4* out = reinterpret_cast<floatx4*>(first + static_cast<size_t>(n) * ldy);
+                    floatx4 v = *reinterpret_cast<const floatx4*>(tile + n * kPitch + 4 * part8);
                     if constexpr (kMode == 1) {
                         const floatx4 old = *out;
                         v = floatx4{old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
@@ -764,6 +800,28 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     constexpr int kVChunks = kHs / 16;  // 16-byte pieces of the block's V rows per lane
     const float scale = 1.0f / sqrtf(static_cast<float>(kHs));  // model.cpp:188
 
+    // The K rows and the V rows of a wavefront's next block are requested a block ahead (the first block's
+    // before q is read): a block would otherwise be a memory round trip with nothing in between.
+    auto fetch_k = [&](half8_t (&kf)[kKSteps], int p0) {
+        const int prow = (p0 + r < seq_len) ? p0 + r : seq_len - 1;  // (rows past the tile's limit are masked below)
+        const uint16_t* krow = kbase + static_cast<size_t>(prow) * kHs + 8 * g;
+#pragma unroll
+        for (int s = 0; s < kKSteps; ++s) kf[s] = as_half8(load16(krow + 16 * s));
+    };
+    // a block's V rows: piece c of the block = 8 dimensions of one position (zero past the context)
+    auto fetch_v = [&](uintx4 (&vr)[kVChunks], int p0) {
+#pragma unroll
+        for (int i = 0; i < kVChunks; ++i) {
+            const int c = lane + 64 * i, p = c / (kHs / 8), d0 = (c % (kHs / 8)) * 8;
+            const int pos = p0 + p;
+            vr[i] = pos < limit ? load16(vbase + static_cast<size_t>(pos) * kHs + d0) : uintx4{0u, 0u, 0u, 0u};
+        }
+    };
+    half8_t k_next[kKSteps];
+    uintx4 v_next[kVChunks];
+    fetch_k(k_next, 32 * wave);
+    fetch_v(v_next, 32 * wave);
+
     half8_t qh[kKSteps], ql[kKSteps];
     {
         const float* qrow = q + static_cast<size_t>(tok_c) * dim + (kvh * gqa + my_head) * kHs + 8 * g;
@@ -784,16 +842,6 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         for (int e = 0; e < 16; ++e) o[dt][e] = 0.0f;
     float top = -INFINITY, lsum = 0.0f;
 
-    // The K fragments of the next block and the V^T fragments of this one are requested before this
-    // block's products: a block would otherwise be two memory round trips with nothing in between.
-    auto fetch_k = [&](half8_t (&kf)[kKSteps], int p0) {
-        const int prow = (p0 + r < seq_len) ? p0 + r : seq_len - 1;  // (rows past the tile's limit are masked below)
-        const uint16_t* krow = kbase + static_cast<size_t>(prow) * kHs + 8 * g;
-#pragma unroll
-        for (int s = 0; s < kKSteps; ++s) kf[s] = as_half8(load16(krow + 16 * s));
-    };
-    half8_t k_next[kKSteps];
-    fetch_k(k_next, 32 * wave);
     for (int p0 = 32 * wave; p0 < limit; p0 += 128) {
         floatx16 st;
 #pragma unroll
@@ -801,15 +849,13 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         half8_t kf[kKSteps];
 #pragma unroll
         for (int s = 0; s < kKSteps; ++s) kf[s] = k_next[s];
-        // this block's V rows: piece c of the block = 8 dimensions of one position (zero past the context)
         uintx4 vrows[kVChunks];
 #pragma unroll
-        for (int i = 0; i < kVChunks; ++i) {
-            const int c = lane + 64 * i, p = c / (kHs / 8), d0 = (c % (kHs / 8)) * 8;
-            const int pos = p0 + p;
-            vrows[i] = pos < limit ? load16(vbase + static_cast<size_t>(pos) * kHs + d0) : uintx4{0u, 0u, 0u, 0u};
+        for (int i = 0; i < kVChunks; ++i) vrows[i] = v_next[i];
+        if (p0 + 128 < limit) {
+            fetch_k(k_next, p0 + 128);
+            fetch_v(v_next, p0 + 128);
         }
-        if (p0 + 128 < limit) fetch_k(k_next, p0 + 128);
 #pragma unroll
         for (int s = 0; s < kKSteps; ++s) {
             st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], qh[s], st, 0, 0, 0);
@@ -1113,15 +1159,28 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
 
 lpp_status norm_split(float* x, const float* gain, pf::half_t* hi, pf::half_t* lo, int dim, int n, int t_pad, const float* partials,
                       int splits, size_t split_stride, hipStream_t s) {
-    const dim3 rows_grid((t_pad + 3) / 4);
-    if (dim == 1024)
-        hipLaunchKernelGGL(pf::k_norm_split_rows<4>, rows_grid, dim3(256), 0, s, x, gain, hi, lo, n, t_pad, partials, splits, split_stride);
-    else if (dim == 2048)
-        hipLaunchKernelGGL(pf::k_norm_split_rows<8>, rows_grid, dim3(256), 0, s, x, gain, hi, lo, n, t_pad, partials, splits, split_stride);
-    else if (dim == 4096)
-        hipLaunchKernelGGL(pf::k_norm_split_rows<16>, rows_grid, dim3(256), 0, s, x, gain, hi, lo, n, t_pad, partials, splits, split_stride);
-    else
+#define LPP_NORM_WIDE(PER, SPLITS) \
+    hipLaunchKernelGGL((pf::k_norm_split_wide<PER, SPLITS>), dim3(t_pad), dim3(256), 0, s, x, gain, hi, lo, n, partials, split_stride)
+#define LPP_NORM_WIDE_DIM(PER)          \
+    switch (splits) {                   \
+        case 0: LPP_NORM_WIDE(PER, 0); break; \
+        case 2: LPP_NORM_WIDE(PER, 2); break; \
+        case 4: LPP_NORM_WIDE(PER, 4); break; \
+        default: LPP_NORM_WIDE(PER, 8); break; \
+    }
+    // (gemm() cuts K into 1, 2, 4 or 8 ranges)
+    const bool wide = (dim == 1024 || dim == 2048 || dim == 4096) && (splits == 0 || splits == 2 || splits == 4 || splits == 8);
+    if (wide && dim == 1024) {
+        LPP_NORM_WIDE_DIM(1)
+    } else if (wide && dim == 2048) {
+        LPP_NORM_WIDE_DIM(2)
+    } else if (wide) {
+        LPP_NORM_WIDE_DIM(4)
+    } else {
         hipLaunchKernelGGL(pf::k_norm_split, dim3(t_pad), dim3(256), 0, s, x, gain, hi, lo, dim, n, partials, splits, split_stride);
+    }
+#undef LPP_NORM_WIDE_DIM
+#undef LPP_NORM_WIDE
     LPP_CHECK_LAUNCH("k_norm_split");
     return LPP_OK;
 }
