@@ -110,8 +110,9 @@ __global__ __launch_bounds__(256) void k_norm_split(float* __restrict__ x, const
 
 // The same with a workgroup per row (dim = 1024 kPer) and the number of partial products known to
 // the compiler: a thread's kPer x (1 + kSplits) loads are all requested before the first is used, so
-// a row costs one round trip to memory and is read once.  Residual sum in the same order; the sum of squares runs over a thread's elements in
-// order, across the lanes, then over the four wavefronts as (0 + 1) + (2 + 3).
+// a row costs one round trip to memory and is read once.  Residual sum in the same order; the sum
+// of squares runs over a thread's elements in order, across the lanes, then over the four
+// wavefronts as (0 + 1) + (2 + 3).
 template <int kPer, int kSplits>
 __global__ __launch_bounds__(256) void k_norm_split_wide(float* __restrict__ x, const float* __restrict__ gain,
                                                          half_t* __restrict__ hi, half_t* __restrict__ lo, int n_tokens,
@@ -801,7 +802,8 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     const float scale = 1.0f / sqrtf(static_cast<float>(kHs));  // model.cpp:188
 
     // The K rows and the V rows of a wavefront's next block are requested a block ahead (the first block's
-    // before q is read): a block would otherwise be a memory round trip with nothing in between.
+    // before q is read), so that they travel while this block is worked on.  (Four blocks ahead measures
+    // slower: a block's time is its ~400 vector instructions, and the registers cost more than the wait.)
     auto fetch_k = [&](half8_t (&kf)[kKSteps], int p0) {
         const int prow = (p0 + r < seq_len) ? p0 + r : seq_len - 1;  // (rows past the tile's limit are masked below)
         const uint16_t* krow = kbase + static_cast<size_t>(prow) * kHs + 8 * g;
