@@ -43,7 +43,8 @@ def rel_err(got, want):
     return float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
 
 
-@pytest.mark.parametrize("n,k,t", [(128, 32, 128), (256, 2048, 128), (384, 1024, 256), (128, 8192, 512), (16384, 256, 512)])
+@pytest.mark.parametrize("n,k,t", [(128, 32, 128), (256, 2048, 128), (384, 1024, 256), (128, 8192, 512), (16384, 256, 512),
+                                   (256, 64, 128), (16384, 64, 512)])  # the last two: one and two trips through the staged kernels
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_gemm_against_float64(lib, n, k, t, accumulate):
     rng = np.random.default_rng(1000 * n + k + t)
