@@ -200,11 +200,18 @@ lpp_status lpp_model_set_path(lpp_model *m, int path);
 /* Test hooks of LPP_PATH_PERSISTENT (no counterpart in the reference).  Its kernel waits
  * for values other workgroups publish with a bounded number of polls (default 2^20, far
  * beyond any real wait): a wait that runs out raises a flag that ends every other wait,
- * all workgroups leave the kernel normally, and lpp_forward / lpp_generate return
- * LPP_ERR_HIP ("gave up waiting"); the model is usable again after lpp_model_reset or
- * simply at the next call, because values carry sequence numbers that never repeat.
+ * all workgroups leave the kernel normally, no token is delivered and the device's step
+ * record stays as the launch found it, and lpp_forward / lpp_generate return LPP_ERR_HIP
+ * ("gave up waiting"); the model is usable again at the next call (lpp_generate: from the
+ * position the caller chooses; the cache holds every position decoded before the failed
+ * launch), because values carry sequence numbers that never repeat.  One cause is
+ * handled inside the library and never reaches the caller: a launch whose workgroups
+ * the device dealt out unevenly over its XCDs (the per-XCD hand-overs assume equal
+ * shares) switches those hand-overs off for the model and launches the same token again.
+ * A give-up while the per-XCD hand-overs are in use switches them off as well.
  * set_spin_limit changes the bound; set_sequence_base moves the 32-bit sequence count
- * (the library re-zeroes its exchange slots and restarts the count before it can wrap). */
+ * (the library re-zeroes its exchange slots and restarts the count before it can wrap).
+ * Both are test hooks, like lpp_set_test_option in section C. */
 lpp_status lpp_model_set_spin_limit(lpp_model *m, unsigned polls);
 lpp_status lpp_model_set_sequence_base(lpp_model *m, unsigned base);
 /* Forget the KV cache contents (zero-fill, as malloc_run_state leaves it). */
@@ -446,6 +453,35 @@ lpp_status lpp_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes);
 lpp_status lpp_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes);
 /* Device facts used by the benchmark report. */
 lpp_status lpp_device_info(char *name, size_t name_cap, int *compute_units, size_t *hbm_bytes);
+
+/* Test hooks (no counterpart in the reference).  The library picks among alternative
+ * plans and kernels by itself -- from the model's shape, the position, and what it
+ * measured on the device at the first launch.  Each option below takes one of those
+ * choices away so that a test can run the alternative the library would otherwise not
+ * have taken on the machine at hand; none changes what is computed.  Process-wide;
+ * a model picks a change up at its next launch (the persistent path rebuilds its step
+ * lists then).  Defaults in brackets. */
+enum lpp_test_option {
+    /* LPP_PATH_PERSISTENT */
+    LPP_OPT_DECODE_XCD_HANDOVERS = 0,   /* [1] number workgroups by XCD and hand hb / q,k,v over inside an XCD when the
+                                               device deals workgroups out to its XCDs in turn; 0: as if it did not */
+    LPP_OPT_DECODE_XCD_QKV = 1,         /* [1] deal the Wq/Wk/Wv rows out per XCD where the KV heads divide among them   */
+    LPP_OPT_DECODE_PARKING = 2,         /* [1] keep gate/up rows in LDS at short contexts                               */
+    LPP_OPT_DECODE_LANE_ITEM = 3,       /* [1] one-pass attention item for heads of size 64; 0: the walking item        */
+    LPP_OPT_DECODE_FAIL_TICKETS = 4,    /* [0] n > 0: the n-th launch from now that uses the per-XCD numbering is told a
+                                               wrong ticket base, so every workgroup reports an unevenly dealt XCD (the
+                                               kernel drains normally) and the library's recovery runs; counts down to 0 */
+    LPP_OPT_DECODE_XCD_ATTENTION = 5,   /* [1] split a KV head's context over the workgroups of its XCD at long contexts;
+                                               0: work items dealt out over the whole device                            */
+    /* batched prefill */
+    LPP_OPT_PREFILL_STAGED_GEMM = 6,    /* [1] LDS-pipelined GEMM; 0: fragments straight from memory + separate SwiGLU   */
+    LPP_OPT_PREFILL_WIDE_TILES = 7,     /* [1] 256 x 128 tiles where they fill the device                               */
+    LPP_OPT_PREFILL_FUSED_FFN = 8,      /* [1] W1, W3 and SwiGLU in one launch                                          */
+    LPP_OPT_PREFILL_MFMA_ATTENTION = 9, /* [1] matrix-core attention; 0: one wavefront per token and KV head            */
+    LPP_OPT_COUNT = 10
+};
+lpp_status lpp_set_test_option(int option, int value);
+lpp_status lpp_get_test_option(int option, int *value);
 
 /* Deterministic synthetic tensors (host side): element i of a stream named by
  * seed is N(0, std) from a counter-based generator (splitmix64 -> Box-Muller in

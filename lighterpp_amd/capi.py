@@ -34,6 +34,13 @@ TENSOR_NAMES = ["token_embedding", "rms_att", "wq", "wk", "wv", "wo", "rms_ffn",
 
 PATH_OPS, PATH_FUSED, PATH_PERSISTENT = 0, 1, 2
 GGML_F32, GGML_F16 = 0, 1
+# enum lpp_test_option
+(OPT_DECODE_XCD_HANDOVERS, OPT_DECODE_XCD_QKV, OPT_DECODE_PARKING, OPT_DECODE_LANE_ITEM, OPT_DECODE_FAIL_TICKETS,
+ OPT_DECODE_XCD_ATTENTION, OPT_PREFILL_STAGED_GEMM, OPT_PREFILL_WIDE_TILES, OPT_PREFILL_FUSED_FFN,
+ OPT_PREFILL_MFMA_ATTENTION, OPT_COUNT) = range(11)
+OPT_DEFAULTS = {OPT_DECODE_XCD_HANDOVERS: 1, OPT_DECODE_XCD_QKV: 1, OPT_DECODE_PARKING: 1, OPT_DECODE_LANE_ITEM: 1,
+                OPT_DECODE_FAIL_TICKETS: 0, OPT_DECODE_XCD_ATTENTION: 1, OPT_PREFILL_STAGED_GEMM: 1,
+                OPT_PREFILL_WIDE_TILES: 1, OPT_PREFILL_FUSED_FFN: 1, OPT_PREFILL_MFMA_ATTENTION: 1}
 TOKENIZER_SENTENCEPIECE, TOKENIZER_BPE = 0, 1
 
 
@@ -143,6 +150,8 @@ SIGNATURES = {
     "lpp_malloc_host": (_i, [C.POINTER(_vp), _sz]),
     "lpp_free_host": (_i, [_vp]),
     "lpp_device_info": (_i, [C.c_char_p, _sz, _ip, C.POINTER(_sz)]),
+    "lpp_set_test_option": (_i, [_i, _i]),
+    "lpp_get_test_option": (_i, [_i, _ip]),
     "lpp_synth_normal_f32": (_i, [_vp, _sz, _u64, _u64, _f]),
     "lpp_synth_normal_f16": (_i, [_vp, _sz, _u64, _u64, _f]),
     "lpp_synth_uniform_f32": (_i, [_vp, _sz, _u64, _u64]),
@@ -236,6 +245,21 @@ class DeviceBuffer:
 
 def synchronize() -> None:
     check(load().lpp_synchronize())
+
+
+def set_test_option(option: int, value: int) -> None:
+    check(load().lpp_set_test_option(option, value))
+
+
+def get_test_option(option: int) -> int:
+    v = C.c_int(0)
+    check(load().lpp_get_test_option(option, C.byref(v)))
+    return v.value
+
+
+def reset_test_options() -> None:
+    for option, value in OPT_DEFAULTS.items():
+        set_test_option(option, value)
 
 
 # ---- synthetic data -------------------------------------------------------------

@@ -63,16 +63,8 @@ constexpr int kPollBatch = 8;                      // tagged values one thread r
 constexpr int kItemPositions = 1024;               // a one-head attention work item stays within twice this many positions
 constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS copy of the penalty window
 constexpr int kMaxHeadPad = 128;
-#ifndef LPP_IDLE_WAITS_FOR_Q
-#define LPP_IDLE_WAITS_FOR_Q 0
-#endif
-#ifndef LPP_PACED_STEPS
-#define LPP_PACED_STEPS 2
-#endif
-#ifndef LPP_SHORT_ROUNDS
-#define LPP_SHORT_ROUNDS 2
-#endif
-constexpr int kShortRounds = LPP_SHORT_ROUNDS;          // cache rows per lane group a one-head work item requests at once
+constexpr int kShortRounds = 2;                    // cache rows per lane group a one-head work item requests at once
+constexpr int kPacedSteps = 2;                     // next-phase rows a streaming wavefront sends out early after a burst
 constexpr int kMaxAttHeads = 2;                    // query heads of one KV head a long-context work item covers
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
 
@@ -96,6 +88,11 @@ __device__ __forceinline__ u64 peek(const u64* slot) {
 // The same inside one XCD: a plain store stays in the XCD's L2 (a device-scope one writes through and drops the line),
 // and a non-temporal load is not kept by the compute unit's L1, so it is served by that L2.  Only for slots that no
 // other XCD touches.
+// (Both statements take their address as a VECTOR operand.  An asm statement that hands a memory instruction a
+// SCALAR address operand must begin with s_nop 4: the compiler may have written that register pair with a vector
+// instruction (v_readlane from where it keeps spilled scalars) immediately before, a memory instruction reading it
+// needs five wait states after such a write, and nobody counts wait states inside an asm statement -- the first
+// request would go to whatever the pair held before.)
 __device__ __forceinline__ void publish_near(u64* slot, float v, unsigned tag) {
     const u64 both = pack(v, tag);
     asm volatile("global_store_dwordx2 %0, %1, off sc0" ::"v"(slot), "v"(both) : "memory");
@@ -437,7 +434,6 @@ __device__ __forceinline__ void gemv_role(const DecodeArgs& a, Control& ctl, con
     unsigned pace = 0u;
     int paced = 0;  // next-phase rows sent out early since the last burst
     constexpr int kPaceSleep = 15;
-    constexpr int kPacedSteps = LPP_PACED_STEPS;
     auto run_round = [&](const uintx4& batch, int slot0) {
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) {
@@ -651,11 +647,17 @@ __device__ __forceinline__ void mark(Ctx& c, const Io& io, int which) {
 // Polling
 // ---------------------------------------------------------------------------
 
+// What went wrong in a launch, for the host: 1 a wait for tagged values ran out, 2 an LDS wait did, 3 an XCD was
+// dealt more than its share of the workgroups.  The highest code reported stays (the host's recovery differs for 3).
+__device__ __forceinline__ void report_error(StepParams* step, int code) {
+    __hip_atomic_fetch_max(&step->error, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ bool poll_give_up(const Ctx& c, unsigned& spins) {
     if ((spins & 63u) == 63u && __hip_atomic_load(c.t.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return true;
     if (++spins > c.t.spin_limit) {
         __hip_atomic_store(c.t.abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        c.a.step->error = 1;
+        report_error(c.a.step, 1);
         return true;
     }
     __builtin_amdgcn_s_sleep(1);
@@ -1703,11 +1705,6 @@ __host__ __device__ inline int item_splits(int npos, int cap, int n_heads, int n
 // q, k and v are out (one value stands for all: they are published within a microsecond of one
 // another), so that what those held back goes out while the items are computed, not before.
 __device__ __forceinline__ void idle_attention_received(Ctx& c, const Io& io, int layer) {
-#if LPP_IDLE_WAITS_FOR_Q
-    float unused[1];
-    const u64* one = c.t.q + (c.wg % c.a.dim);
-    poll_n<1>([&](int) -> const u64* { return one; }, unused, c.seq(layer, kQkv), c);
-#endif
     (void)io;
     (void)layer;
     signal_received(c.ctl);
@@ -1982,7 +1979,10 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     if (it == 0) {
         const int target = lds_ld(&ctl.target);
         const bool finisher = (target == wg) || (target < 0 && wg == nwg - 1);
-        if (finisher) finish_token(a, lds_ld(&ctl.token), 0u);
+        // A launch in which some wait was given up delivers nothing: the step record stays as it was, so the
+        // host can launch the same token again.
+        if (finisher && __hip_atomic_load(c.t.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u)
+            finish_token(a, lds_ld(&ctl.token), 0u);
     }
     mark(c, io, 4);
     ++c.phase_index;
@@ -2011,7 +2011,7 @@ __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
     }
     fresh();
     io_classify_sample(c, io, l);
-    if (io.it == 0 && lds_peek(&c.ctl.error) != 0u) a.step->error = 2;
+    if (io.it == 0 && lds_peek(&c.ctl.error) != 0u) report_error(a.step, 2);
 }
 
 // ---------------------------------------------------------------------------
@@ -2038,7 +2038,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
                 number = static_cast<int>(order) * t.n_xcc + x;
             } else {
                 __hip_atomic_store(t.abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                a.step->error = 3;
+                __hip_atomic_fetch_max(&a.step->error, 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
         numbered = number;
@@ -2111,7 +2111,7 @@ Plan plan_for(const lpp_model* m, bool parking) {
     b.qkv_by_xcc = 0;
     {
         // Per XCD where the KV heads divide among the XCDs (qkv_row): whole KV heads with their query heads.
-        static const bool allowed = getenv("LPP_NO_XCD_QKV") == nullptr;
+        const bool allowed = test_option(LPP_OPT_DECODE_XCD_QKV) != 0;
         const int n = m->df_xcc;
         if (allowed && n > 1 && c.n_kv_heads % n == 0 && p.grid % n == 0 && c.n_heads / n <= p.grid / n) {
             const int rows = (c.dim + 2 * m->kv_dim) / n, wgs = p.grid / n;
@@ -2157,8 +2157,7 @@ Plan plan_for(const lpp_model* m, bool parking) {
         const size_t row_bytes = static_cast<size_t>(c.dim) * 2;
         int rows = used + kReserve < kLdsBytes ? static_cast<int>((kLdsBytes - kReserve - used) / row_bytes) : 0;
         rows &= ~1;                                 // whole hidden units
-        static const int env_cap = getenv("LPP_PARK_ROWS") ? atoi(getenv("LPP_PARK_ROWS")) : 0;
-        const int cap = env_cap > 0 ? env_cap : 4 * df::kIoWaves;  // a handful of rows per exchange wavefront is plenty
+        const int cap = 4 * df::kIoWaves;  // a handful of rows per exchange wavefront is plenty
         if (rows > cap) rows = cap;
         // units of an ordinary workgroup if the first n_heads own rows / 2 fewer
         const int gu = (c.hidden_dim + c.n_heads * (rows / 2) + p.grid - 1) / p.grid;
@@ -2194,7 +2193,7 @@ size_t tagged_count(const lpp_model* m, int grid_cap) {
 // blocks per 64 positions in the parked rows' area and the staged-activation area of plan p, whole blocks of 64
 // positions inside the cache; 0 where that item does not apply.
 int lane_item_positions(const lpp_model* m, const Plan& p) {
-    static const bool off = getenv("LPP_NO_LANE_ITEM") != nullptr;
+    const bool off = test_option(LPP_OPT_DECODE_LANE_ITEM) == 0;
     if (off || m->head_size != 64 || m->cfg.n_heads > p.grid) return 0;
     const int blocks = p.blocks.park_floats / df::kLaneBlockFloats + p.blocks.xs_floats / df::kLaneBlockFloats;
     int cap = blocks / 2 * df::kWave;
@@ -2414,11 +2413,16 @@ const char* dataflow_unsupported_reason(const lpp_model* m) {
 template <bool kF16>
 static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
     if (const char* why = dataflow_unsupported_reason(m)) return fail(LPP_ERR_UNSUPPORTED, "%s", why);
+    if (m->df_options_epoch != test_options_epoch()) {
+        // A test hook changed what the plans may use: forget what was derived under the old settings.
+        LPP_TRY(dataflow_forget_plans(m, s, 0));
+        m->df_options_epoch = test_options_epoch();
+    }
     if (m->df_xcc == 0) {
         // Workgroups are handed to the XCDs in turn.  The per-XCD hand-overs rely on every XCD getting an equal share
         // of them, so it is measured, not assumed: anything but workgroup w on XCD (first + w) % n switches them off.
         m->df_xcc = 1;
-        if (getenv("LPP_NO_XCD_LOCAL") == nullptr) {
+        if (test_option(LPP_OPT_DECODE_XCD_HANDOVERS) != 0) {
             const int grid = compute_units();
             void* d = nullptr;
             LPP_TRY(lpp_malloc(&d, static_cast<size_t>(grid) * sizeof(int)));
@@ -2434,14 +2438,11 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
             bool in_turn = n > 1 && n <= kMaxXcc && grid % n == 0;
             for (int w = 0; w < grid && in_turn; ++w) in_turn = where[w] == (where[0] + w) % n;
             if (in_turn) m->df_xcc = n;
-            if (getenv("LPP_DEBUG") != nullptr)
-                fprintf(stderr, "persistent decode: %d XCDs seen, workgroups %s; per-XCD hand-overs %s\n", n,
-                        in_turn ? "in turn" : "not in turn", m->df_xcc > 1 ? "on" : "off");
         }
     }
     // Two plans: with parked gate/up rows while only the first n_heads workgroups hold an attention item
     // (one split per head), without them at longer contexts.  Each has its own step lists.
-    static const bool parking_allowed = getenv("LPP_NO_PARKING") == nullptr;
+    const bool parking_allowed = test_option(LPP_OPT_DECODE_PARKING) != 0;
     const Plan parked_plan = plan_for(m, parking_allowed);
     const int lane_cap = lane_item_positions(m, parked_plan);
     df::Tagged tagged = tagged_of(m, a.uniforms != nullptr, lane_cap);
@@ -2488,6 +2489,8 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     if (m->df_rows[which] == nullptr) LPP_TRY(build_step_lists(m, p, which));
     if (parked_plan.blocks.park_rows > 0 && m->df_rows[1 - which] == nullptr)
         LPP_TRY(build_step_lists(m, use_parked ? plan_for(m, false) : parked_plan, 1 - which));
+    // (test hook: a ticket base one launch behind makes every workgroup's ticket look like one too many for its XCD)
+    if (tagged.n_xcc > 1 && take_forced_ticket_failure()) tagged.ticket_base -= static_cast<unsigned>(m->persist_grid / tagged.n_xcc);
     hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a, tagged,
                        p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
     LPP_CHECK_LAUNCH("k_decode_dataflow");
@@ -2505,19 +2508,43 @@ lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s)
     return m->cfg.weight_precision == LPP_WEIGHT_FP16 ? launch_impl<true>(m, a, s) : launch_impl<false>(m, a, s);
 }
 
-// What a launch left in StepParams::error, as a status.  Code 3 (an XCD did not get its share of the workgroups)
-// also switches the per-XCD hand-overs off for this model: the next launch runs without them.
-lpp_status dataflow_report_error(lpp_model* m, int code) {
-    if (code == 0) return LPP_OK;
-    if (code == 3) {
-        m->df_xcc = 1;
-        for (int i = 0; i < 2; ++i) {  // the step lists were dealt out per XCD
-            lpp_free(m->df_rows[i]);
-            m->df_rows[i] = nullptr;
-        }
-        return fail(LPP_ERR_HIP, "decode kernel: workgroups unevenly spread over the XCDs; per-XCD hand-overs switched off");
+// Forget the step lists, the launch sizing and the per-XCD ticket counts; df_xcc = 0 has the next launch probe the
+// device again, 1 leaves the per-XCD hand-overs off for this model.
+lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc) {
+    LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the lists and drawing tickets
+    for (int i = 0; i < 2; ++i) {
+        lpp_free(m->df_rows[i]);
+        m->df_rows[i] = nullptr;
     }
-    return fail(LPP_ERR_HIP, "decode kernel gave up waiting for its inputs");
+    m->df_xcc = df_xcc;
+    m->persist_grid = 0;
+    m->df_ticket_base = 0;
+    if (m->sync_words != nullptr) LPP_TRY(lpp_memset(m->sync_words + 96, 0, kMaxXcc * sizeof(unsigned)));
+    return LPP_OK;
+}
+
+// After a launch that left a code in StepParams::error (the stream is idle, the step record is as the launch found it:
+// a launch that gave up delivers no token).  Whatever the code, the ticket counters and the abort flag start afresh.
+// Code 3 (an XCD was dealt more than its share of the workgroups): the per-XCD hand-overs are switched off for this
+// model and *relaunch is set -- sequence numbers never repeat, so the same token can simply be launched again.
+// Code 1 (a wait for inputs ran out) under the per-XCD scheme switches it off as well: the hand-overs inside an XCD
+// rest on how its L2 serves plain stores and non-temporal loads, and the device-scope path does not.
+lpp_status dataflow_after_error(lpp_model* m, int code, bool* relaunch) {
+    *relaunch = false;
+    if (code == 0) return LPP_OK;
+    hipStream_t s = stream();
+    const bool had_xcd_scheme = m->df_xcc > 1;
+    LPP_TRY(dataflow_forget_plans(m, s, (code == 3 || had_xcd_scheme) ? 1 : m->df_xcc));
+    LPP_TRY(lpp_memset(m->sync_words + 64, 0, 2 * sizeof(unsigned)));
+    int zero = 0;
+    LPP_HIP(hipMemcpyAsync(&m->step->error, &zero, sizeof zero, hipMemcpyHostToDevice, s));
+    LPP_HIP(hipStreamSynchronize(s));
+    if (code == 3) {
+        *relaunch = true;
+        return LPP_OK;
+    }
+    return fail(LPP_ERR_HIP, code == 2 ? "decode kernel: a wait inside a workgroup ran out"
+                                       : "decode kernel gave up waiting for its inputs");
 }
 
 unsigned dataflow_phases_per_token(int n_layers) { return df::phases_per_token(n_layers); }

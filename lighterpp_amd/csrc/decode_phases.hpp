@@ -868,6 +868,7 @@ size_t dataflow_tagged_bytes(const lpp_model* m);
 lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s);
 unsigned dataflow_phases_per_token(int n_layers);
 unsigned dataflow_trace_marks();
-lpp_status dataflow_report_error(lpp_model* m, int code);
+lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc);
+lpp_status dataflow_after_error(lpp_model* m, int code, bool* relaunch);
 
 }  // namespace lpp

@@ -150,11 +150,7 @@ DecodeArgs make_args(const lpp_model* m, bool with_arrays) {
 
 int blocks_for_tiles(int ntiles) {
     int blocks = (ntiles + kWavesPerWg - 1) / kWavesPerWg;
-    static const int per_cu = [] {
-        const char* e = std::getenv("LPP_BLOCKS_PER_CU");  // tuning aid
-        const int v = e ? std::atoi(e) : 0;
-        return v > 0 ? v : 8;
-    }();
+    constexpr int per_cu = 8;
     const int cap = compute_units() * per_cu;
     if (blocks > cap) blocks = cap;
     return blocks < 1 ? 1 : blocks;
@@ -394,16 +390,22 @@ lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, fl
     sp.temperature = temperature;
     sp.penalty = penalty;
     sp.r = r;
-    LPP_TRY(begin_run(m, sp, s));
-    if (use_history)
-        LPP_HIP(hipMemcpyAsync(m->history, history, static_cast<size_t>(history_len) * sizeof(int),
-                               hipMemcpyHostToDevice, s));
-    LPP_TRY(launch_token(m, false, s));
-    LPP_HIP(hipMemcpyAsync(next_token, m->sampled_token, sizeof(int), hipMemcpyDeviceToHost, s));
-    LPP_HIP(hipStreamSynchronize(s));
-    if (m->path == LPP_PATH_PERSISTENT) {
+    for (int attempt = 0;; ++attempt) {
+        LPP_TRY(begin_run(m, sp, s));
+        if (use_history)
+            LPP_HIP(hipMemcpyAsync(m->history, history, static_cast<size_t>(history_len) * sizeof(int),
+                                   hipMemcpyHostToDevice, s));
+        LPP_TRY(launch_token(m, false, s));
+        LPP_HIP(hipMemcpyAsync(next_token, m->sampled_token, sizeof(int), hipMemcpyDeviceToHost, s));
+        LPP_HIP(hipStreamSynchronize(s));
+        if (m->path != LPP_PATH_PERSISTENT) break;
         LPP_HIP(hipMemcpy(m->step_host, m->step, sizeof(StepParams), hipMemcpyDeviceToHost));
-        if (m->step_host->error != 0) return dataflow_report_error(m, m->step_host->error);
+        if (m->step_host->error == 0) break;
+        // The persistent kernel drained without a token.  Where the cause is the per-XCD numbering, that is
+        // switched off and the same token launched once more (values carry sequence numbers that never repeat).
+        bool relaunch = false;
+        LPP_TRY(dataflow_after_error(m, m->step_host->error, &relaunch));
+        if (!relaunch || attempt > 0) return fail(LPP_ERR_HIP, "decode kernel: workgroups unevenly spread over the XCDs");
     }
     return LPP_OK;
 }
@@ -446,15 +448,34 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     // on the host.
     LPP_HIP(hipEventRecord(m->ev_a, s));
     const auto t0 = std::chrono::steady_clock::now();
+    int launched = 0;
+    bool relaunched = false;
     for (int i = 0; i < n_steps; ++i) {
-        LPP_TRY(launch_token(m, true, s));
-        if (i > 0) {
-            LPP_TRY(await_token(m, i - 1, s));
-            out_tokens[i - 1] = m->pinned_tokens[i - 1];
+        while (launched < n_steps && launched <= i + 1) {
+            LPP_TRY(launch_token(m, true, s));
+            ++launched;
         }
+        if (await_token(m, i, s) != LPP_OK) {
+            // The stream went idle without token i: a persistent launch drained with an error code.  Such a launch
+            // leaves the device's step record as it found it, so the record says where to pick up.
+            if (m->path != LPP_PATH_PERSISTENT) return LPP_ERR_HIP;
+            StepParams rec{};
+            LPP_HIP(hipMemcpy(&rec, m->step, sizeof rec, hipMemcpyDeviceToHost));
+            if (rec.error == 0) return LPP_ERR_HIP;  // (await_token's own message stands)
+            bool again = false;
+            LPP_TRY(dataflow_after_error(m, rec.error, &again));
+            if (!again || relaunched || rec.step_index != i)
+                return fail(LPP_ERR_HIP, "decode kernel: workgroups unevenly spread over the XCDs");
+            relaunched = true;
+            m->df_pos = rec.pos;
+            m->df_history_len = rec.history_len;
+            m->df_step_index = rec.step_index;
+            launched = i;
+            --i;
+            continue;
+        }
+        out_tokens[i] = m->pinned_tokens[i];
     }
-    LPP_TRY(await_token(m, n_steps - 1, s));
-    out_tokens[n_steps - 1] = m->pinned_tokens[n_steps - 1];
     m->df_uniforms_host = nullptr;
     const auto t1 = std::chrono::steady_clock::now();
     LPP_HIP(hipEventRecord(m->ev_b, s));
@@ -463,7 +484,11 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
     // Hand the penalty window back in the reference's order (oldest first).
     StepParams done{};
     LPP_HIP(hipMemcpy(&done, m->step, sizeof done, hipMemcpyDeviceToHost));
-    if (done.error != 0) return dataflow_report_error(m, done.error);
+    if (done.error != 0) {
+        bool again = false;
+        LPP_TRY(dataflow_after_error(m, done.error, &again));
+        return fail(LPP_ERR_HIP, "decode kernel reported error %d after the last token", done.error);
+    }
     if (history_cap > 0) {
         std::vector<int> ring(static_cast<size_t>(history_cap));
         LPP_HIP(hipMemcpy(ring.data(), m->history, ring.size() * sizeof(int), hipMemcpyDeviceToHost));

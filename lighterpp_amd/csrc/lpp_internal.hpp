@@ -55,8 +55,16 @@ int compute_units();
 lpp_status rope_table(int head_size, float rope_base, int min_positions, const float2** d_table);
 
 // Resolves, for the current device, the address of the device-resident scratch that
-// lpp_prefill_gemm_noalloc works in (prefill.hip); lpp_init calls it once per device.
+// lpp_prefill_gemm_noalloc works in (prefill.hip); lpp_init calls it once per device.  What it
+// returned is kept per device and handed out by prefill_gemm_scratch_status(): the allocation-free
+// entry point reports a failed set-up, nothing else in the library depends on it.
 lpp_status prefill_gemm_scratch_setup();
+
+// Test hooks (lpp_set_test_option).  The epoch changes whenever an option a model has acted on changes.
+int test_option(int option);
+unsigned test_options_epoch();
+// LPP_OPT_DECODE_FAIL_TICKETS: counts a launch; true for the launch that is to fail.
+bool take_forced_ticket_failure();
 
 // Launch helpers implemented in the .hip files and used by the model code.
 namespace k {

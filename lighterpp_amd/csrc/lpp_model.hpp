@@ -67,6 +67,7 @@ struct lpp_model {
     int persist_grid = 0;                    // workgroups of the persistent kernel (0: not sized yet)
     unsigned df_ticket_base = 0;             // what the per-XCD workgroup counters read before the next persistent launch
     int df_xcc = 0;                          // XCDs the persistent kernel's workgroups go round (1: near copies off; 0: not probed)
+    unsigned df_options_epoch = 0;           // test_options_epoch() the plans and lists were made under
     unsigned spin_limit = 1u << 20;          // polls a wait for tagged inputs may take before giving up
     const float2* rope = nullptr;            // [seq_len][head_size/2] (cos, sin)
     int max_splits = 1;

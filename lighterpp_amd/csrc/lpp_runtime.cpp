@@ -33,7 +33,19 @@ struct RopeTable {
 };
 std::map<std::tuple<int, int, uint32_t>, RopeTable> g_rope;  // key: device, head_size, base bits
 
+// Test hooks (lpp_set_test_option): which of its alternatives the library may pick by itself.
+int g_test_options[LPP_OPT_COUNT] = {1, 1, 1, 1, 0, 1, 1, 1, 1, 1};
+unsigned g_test_epoch = 1;  // advanced by every change a model has to act on
+
 }  // namespace
+
+int test_option(int option) { return (option >= 0 && option < LPP_OPT_COUNT) ? g_test_options[option] : 0; }
+unsigned test_options_epoch() { return g_test_epoch; }
+bool take_forced_ticket_failure() {
+    if (g_test_options[LPP_OPT_DECODE_FAIL_TICKETS] <= 0) return false;
+    g_test_options[LPP_OPT_DECODE_FAIL_TICKETS] -= 1;
+    return g_test_options[LPP_OPT_DECODE_FAIL_TICKETS] == 0;
+}
 
 lpp_status fail(lpp_status code, const char* fmt, ...) {
     va_list ap;
@@ -134,7 +146,10 @@ lpp_status lpp_init(int device) {
     lpp::g_rt.device = device;
     lpp::g_rt.cus = prop.multiProcessorCount;
     lpp::g_rt.ready = true;
-    return lpp::prefill_gemm_scratch_setup();
+    // What the allocation-free prefill GEMM needs on this device is set up here, so that it never has to do so
+    // itself; a failure is that entry point's to report (prefill_gemm_scratch_status), not the whole library's.
+    lpp::prefill_gemm_scratch_setup();
+    return LPP_OK;
 }
 
 lpp_status lpp_set_stream(void* hip_stream) {
@@ -220,6 +235,21 @@ lpp_status lpp_memcpy_d2d(void* d_dst, const void* d_src, size_t bytes) {
     LPP_REQUIRE(d_dst && d_src, "lpp_memcpy_d2d: null pointer");
     if (!lpp::g_rt.ready) LPP_TRY(lpp_init(0));
     LPP_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, lpp::g_rt.current));
+    return LPP_OK;
+}
+
+lpp_status lpp_set_test_option(int option, int value) {
+    LPP_REQUIRE(option >= 0 && option < LPP_OPT_COUNT, "lpp_set_test_option: no option %d", option);
+    if (lpp::g_test_options[option] != value) {
+        lpp::g_test_options[option] = value;
+        if (option != LPP_OPT_DECODE_FAIL_TICKETS) lpp::g_test_epoch += 1;
+    }
+    return LPP_OK;
+}
+
+lpp_status lpp_get_test_option(int option, int* value) {
+    LPP_REQUIRE(option >= 0 && option < LPP_OPT_COUNT && value != nullptr, "lpp_get_test_option: no option %d", option);
+    *value = lpp::g_test_options[option];
     return LPP_OK;
 }
 

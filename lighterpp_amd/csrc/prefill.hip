@@ -1083,10 +1083,10 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
         total_n += prods[i].n;
         wide = wide && prods[i].n % 256 == 0;
     }
-    const bool staged = K % pf::kPipeTripK == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr;
+    const bool staged = K % pf::kPipeTripK == 0 && test_option(LPP_OPT_PREFILL_STAGED_GEMM) != 0;
     if (staged) {
         const int token_tiles = t_pad / pf::kTileTokens;
-        wide = wide && (total_n / 256) * token_tiles >= compute_units() && getenv("LPP_PREFILL_NO_WIDE") == nullptr;
+        wide = wide && (total_n / 256) * token_tiles >= compute_units() && test_option(LPP_OPT_PREFILL_WIDE_TILES) != 0;
         const int tile = wide ? 256 : 128;
         const int feature_tiles = total_n / tile;
         const size_t stride = static_cast<size_t>(t_pad) * total_n;
@@ -1239,8 +1239,8 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
     // The fp32 gate and up buffers double as room for the partial products of the GEMMs whose K is
     // split (each is t_pad * hidden floats): up for Wq/Wk/Wv, gate for Wo and then for W2.
     const size_t room = static_cast<size_t>(t_pad) * hidden;
-    const bool fused_ffn = dim % pf::kPipeTripK == 0 && hidden % 128 == 0 && getenv("LPP_PREFILL_DIRECT") == nullptr &&
-                           getenv("LPP_PREFILL_NO_FUSED_FFN") == nullptr;
+    const bool fused_ffn = dim % pf::kPipeTripK == 0 && hidden % 128 == 0 && test_option(LPP_OPT_PREFILL_STAGED_GEMM) != 0 &&
+                           test_option(LPP_OPT_PREFILL_FUSED_FFN) != 0;
     int pending = 0;  // ranges of the product before (W2's, then Wo's) still to be added to x
     for (int l = 0; l < c.n_layers; ++l) {
         // attention block, model.cpp:216-218
@@ -1263,7 +1263,7 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         LPP_CHECK_LAUNCH("k_rope_scatter");
         if (last_layer) break;
         // (rows n .. t_pad of hi/lo are still the zeros k_norm_split wrote: the attention writes rows < n only)
-        const bool matrix_cores = 32 % m->gqa == 0 && getenv("LPP_PREFILL_VALU_ATTENTION") == nullptr;
+        const bool matrix_cores = 32 % m->gqa == 0 && test_option(LPP_OPT_PREFILL_MFMA_ATTENTION) != 0;
         if (matrix_cores) {
             const int tiles = (n + 32 / m->gqa - 1) / (32 / m->gqa);
             const dim3 grid(tiles, c.n_kv_heads);
@@ -1399,15 +1399,42 @@ lpp_status scratch_address(void** out) {
 
 }  // namespace
 
-lpp_status prefill_gemm_scratch_setup() {
-    // (everything the allocation-free entry point would otherwise set up on its first call: a caller under
-    // graph capture finds it done)
+namespace {
+// What the set-up returned on each device: 0 not run yet, 1 done, 2 failed (message kept).
+int g_setup_state[kMaxDevices] = {};
+char g_setup_message[kMaxDevices][256] = {};
+
+lpp_status run_scratch_setup() {
     LPP_TRY((size_pipe<4, 2, 0, 32>()));
     LPP_TRY((size_pipe<4, 2, 1, 32>()));
     LPP_TRY((size_pipe<2, 2, 0, pf::kPipeTripK>()));
     LPP_TRY((size_pipe<2, 2, 1, pf::kPipeTripK>()));
     void* p = nullptr;
     return scratch_address(&p);
+}
+}  // namespace
+
+lpp_status prefill_gemm_scratch_setup() {
+    // (everything the allocation-free entry point would otherwise set up on its first call: a caller under
+    // graph capture finds it done)
+    int device = -1;
+    LPP_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(LPP_ERR_UNSUPPORTED, "device ordinal %d beyond %d", device, kMaxDevices - 1);
+    const lpp_status st = run_scratch_setup();
+    g_setup_state[device] = st == LPP_OK ? 1 : 2;
+    if (st != LPP_OK) std::snprintf(g_setup_message[device], sizeof g_setup_message[device], "%s", lpp_last_error());
+    return st;
+}
+
+// The set-up's outcome on the current device; runs it if this is the first call on the device.
+static lpp_status prefill_gemm_scratch_status() {
+    int device = -1;
+    LPP_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(LPP_ERR_UNSUPPORTED, "device ordinal %d beyond %d", device, kMaxDevices - 1);
+    if (g_setup_state[device] == 0) return prefill_gemm_scratch_setup();
+    if (g_setup_state[device] == 2)
+        return fail(LPP_ERR_HIP, "lpp_prefill_gemm_noalloc: set-up failed on this device: %s", g_setup_message[device]);
+    return LPP_OK;
 }
 
 }  // namespace lpp
@@ -1424,6 +1451,7 @@ lpp_status lpp_prefill_gemm_noalloc(float* d_y, const void* d_w, const float* d_
     LPP_REQUIRE(count <= kNoAllocElements, "lpp_prefill_gemm_noalloc: n_tokens * k = %zu exceeds the built-in scratch of %zu elements",
                 count, kNoAllocElements);
     hipStream_t s = stream();
+    LPP_TRY(prefill_gemm_scratch_status());
     void* base = nullptr;
     LPP_TRY(scratch_address(&base));
     pf::half_t* hi = static_cast<pf::half_t*>(base);

@@ -10,3 +10,14 @@ for p in (str(ROOT), str(ROOT / "tests")):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+import pytest  # noqa: E402
+
+
+@pytest.fixture
+def test_options():
+    """Setter for the library's test hooks (lpp_set_test_option); every option is back at its default afterwards."""
+    from lighterpp_amd import capi
+    yield capi.set_test_option
+    capi.reset_test_options()

@@ -247,6 +247,10 @@ ONE_PASS = {
     # (one wavefront alone up to 64 positions).  Eight KV heads: q, k and v are also handed over inside each XCD.
     "gqa4_8kv": Shape(2048, 512, 1, 32, 8, 500, 640, 500000.0, fp16=True, tied=True),
     "gqa2_4kv": Shape(512, 768, 2, 8, 4, 500, 640, 10000.0, fp16=True, tied=False),
+    # Sixteen KV heads: two per XCD (with their query heads), so a workgroup's rows of the stacked Wq/Wk/Wv run across
+    # KV-head boundaries and an XCD's first workgroups hold the items of two KV heads.
+    "mha_16kv": Shape(1024, 512, 1, 16, 16, 500, 640, 10000.0, fp16=True, tied=True),
+    "gqa2_16kv": Shape(2048, 512, 1, 32, 16, 500, 640, 500000.0, fp16=True, tied=False),
 }
 
 
@@ -283,6 +287,89 @@ def test_one_pass_attention_item_matches_oracle(name):
             assert np.all(np.isfinite(got)), (start, pos)
             assert rel_err(got, want) <= LOGIT_TOL, (start, pos)
             tok = int(np.argmax(want))
+    m.close()
+    o.close()
+
+
+# A 1B-shaped layer: wide enough for parked gate/up rows, eight KV heads for the per-XCD hand-overs, heads of size 64
+# for the one-pass attention item.
+SELF_SELECTED = Shape(2048, 8192, 1, 32, 8, 500, 640, 500000.0, fp16=True, tied=True)
+VARIANTS = {
+    "as_selected": {},
+    "xcd_handovers_off": {capi.OPT_DECODE_XCD_HANDOVERS: 0},
+    "xcd_qkv_off": {capi.OPT_DECODE_XCD_QKV: 0},
+    "no_parking": {capi.OPT_DECODE_PARKING: 0},
+    "walking_attention_item": {capi.OPT_DECODE_LANE_ITEM: 0},
+    "xcd_attention_off": {capi.OPT_DECODE_XCD_ATTENTION: 0},
+}
+
+
+@pytest.mark.parametrize("variant", list(VARIANTS))
+def test_persistent_alternatives_the_library_selects_by_itself(variant, test_options):
+    """Every plan the persistent path may pick by itself -- from the probe of the device, the shape and the position
+    -- decodes the same tokens as the oracle: each is forced here through a test hook, also switched in the middle
+    of a decode (the step lists are rebuilt), positions 0..7 and 515..518 (past the range of the parked-rows plan and of the one-pass item)."""
+    shape = SELF_SELECTED
+    m, o = build(shape, 31)
+    m.set_path(capi.PATH_PERSISTENT)
+    tok, greedy = 5, []
+    for pos in range(8):
+        if pos == 3:
+            for option, value in VARIANTS[variant].items():
+                test_options(option, value)
+        nxt = m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL, (variant, pos)
+        assert nxt == int(np.argmax(want)), (variant, pos)
+        greedy.append(nxt)
+        tok = nxt
+    # past the range of the plan with parked rows and of the one-pass item (the cache in between holds zeros on both sides)
+    for pos in range(515, 519):
+        nxt = m.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL, (variant, pos)
+        assert nxt == int(np.argmax(want)), (variant, pos)
+        tok = nxt
+    # the same plan through the generation loop, from a fresh cache
+    m.reset()
+    toks, _, _ = m.generate(5, 0, 8, temperature=0.0)
+    assert toks.tolist() == greedy, variant
+    m.close()
+    o.close()
+
+
+def test_persistent_relaunches_a_token_when_an_xcd_is_dealt_unevenly(test_options):
+    """A launch in which an XCD draws more tickets than its share ends with every workgroup leaving the kernel
+    normally and no token delivered; the library switches the per-XCD hand-overs off and launches the same token
+    again.  Forced from the host through the ticket base, in lpp_forward and in the middle of lpp_generate: the
+    caller sees the oracle's tokens and no error."""
+    shape = SELF_SELECTED
+    m, o = build(shape, 32)
+    m.set_path(capi.PATH_PERSISTENT)
+    tok, fed, wants = 5, [], []
+    for pos in range(10):
+        if pos == 2:
+            test_options(capi.OPT_DECODE_FAIL_TICKETS, 1)
+        nxt = m.forward(tok, pos, 0.0)
+        if pos == 2:
+            assert capi.get_test_option(capi.OPT_DECODE_FAIL_TICKETS) == 0, "the forced failure was not taken"
+        want = o.forward_logits(tok, pos)
+        fed.append(tok)
+        wants.append(want)
+        assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL, pos
+        assert nxt == int(np.argmax(want)), pos
+        tok = nxt
+    greedy = [int(np.argmax(w)) for w in wants]
+    # the generation loop: the failure hits the n-th launch, with the launch after it already queued
+    for nth in (1, 4, 10):
+        m.reset()
+        # per-XCD hand-overs back on: a changed option has the next launch probe the device again
+        test_options(capi.OPT_DECODE_XCD_HANDOVERS, 0)
+        test_options(capi.OPT_DECODE_XCD_HANDOVERS, 1)
+        test_options(capi.OPT_DECODE_FAIL_TICKETS, nth)
+        toks, _, _ = m.generate(5, 0, 10, temperature=0.0)
+        assert capi.get_test_option(capi.OPT_DECODE_FAIL_TICKETS) == 0, "the forced failure was not taken"
+        assert toks.tolist() == greedy, (nth, toks.tolist(), greedy)
     m.close()
     o.close()
 

@@ -96,12 +96,12 @@ def assert_caches_agree(a, b, shape, upto):
 
 @pytest.mark.parametrize("variant", ["matrix_cores", "fallback_kernels"])
 @pytest.mark.parametrize("name", list(SHAPES))
-def test_prefill_leaves_what_decode_leaves(name, variant, monkeypatch):
+def test_prefill_leaves_what_decode_leaves(name, variant, test_options):
     if variant == "fallback_kernels":
         # the attention on the vector ALUs and the GEMM with fragments straight from memory (what
         # shapes outside the fast kernels' conditions get)
-        monkeypatch.setenv("LPP_PREFILL_VALU_ATTENTION", "1")
-        monkeypatch.setenv("LPP_PREFILL_DIRECT", "1")
+        test_options(capi.OPT_PREFILL_MFMA_ATTENTION, 0)
+        test_options(capi.OPT_PREFILL_STAGED_GEMM, 0)
     shape = SHAPES[name]
     a, b = Model(shape), Model(shape)
     w = a.load_synthetic(7, keep=True)

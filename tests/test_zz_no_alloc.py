@@ -41,6 +41,45 @@ def test_noalloc_gemm_matches_allocating_gemm_twice_in_a_row():
     _case(lib, 13, 128, 32, 128, 0)     # smallest shape the GEMM takes
 
 
+def _free_device_bytes():
+    """hipMemGetInfo of the HIP runtime the library itself is linked against."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_noalloc_gemm_allocates_nothing_and_queues_without_a_sync():
+    """What the entry point is for: device memory in use does not move across its calls (nothing allocated, nothing
+    freed), and two calls of different shapes queued back to back, with no synchronisation between them, both give
+    the allocating entry point's bits (the second overwrites the scratch the first is still being read from only
+    after it: one stream)."""
+    lib = capi.load()
+    capi.check(lib.lpp_init(0))
+    rng = np.random.default_rng(21)
+    cases = []
+    for n, k, t, acc in [(256, 2048, 256, 0), (128, 512, 128, 1)]:
+        w = (rng.standard_normal((n, k)) * 0.05).astype(np.float16)
+        x = (rng.standard_normal((t, k)) * 3.0).astype(F)
+        y0 = rng.standard_normal((t, n)).astype(F)
+        dw, dx = DB.from_numpy(w), DB.from_numpy(x)
+        d_ref, d_new = DB.from_numpy(y0), DB.from_numpy(y0)
+        capi.check(lib.lpp_prefill_gemm(d_ref.ptr, dw.ptr, dx.ptr, n, k, t, acc))
+        cases.append((n, k, t, acc, dw, dx, d_ref, d_new))
+    capi.check(lib.lpp_synchronize())
+    before = _free_device_bytes()
+    for n, k, t, acc, dw, dx, d_ref, d_new in cases:  # queued one behind the other
+        capi.check(lib.lpp_prefill_gemm_noalloc(d_new.ptr, dw.ptr, dx.ptr, n, k, t, acc))
+    after_queue = _free_device_bytes()
+    capi.check(lib.lpp_synchronize())
+    after = _free_device_bytes()
+    assert before == after_queue == after, (before, after_queue, after)
+    for n, k, t, acc, dw, dx, d_ref, d_new in cases:
+        want, got = d_ref.to_numpy(F, t * n), d_new.to_numpy(F, t * n)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (n, k, t)
+
+
 def test_noalloc_gemm_rejects_what_does_not_fit():
     lib = capi.load()
     capi.check(lib.lpp_init(0))
