@@ -394,11 +394,14 @@ lpp_status lpp_prefill_gemm(float *d_y, const void *d_w, const float *d_x, int n
 lpp_status lpp_prefill_gemm_noalloc(float *d_y, const void *d_w, const float *d_x, int n, int k,
                                     int n_tokens, int accumulate);
 
-/* Per-kernel timing of the fused path, measured with HIP events on the launch
- * stream: each kernel class is recorded n_layers times (one launch per layer,
- * so every launch streams different weights) into a graph that is replayed
- * `reps` times between two events.  avg_ms is the mean duration of one launch,
- * bytes the algorithmic HBM bytes of one launch at position `pos`. */
+/* Per-kernel timing of the model's current path, measured with HIP events on the
+ * launch stream.  LPP_PATH_FUSED: each kernel class is recorded n_layers times (one
+ * launch per layer, so every launch streams different weights) into a graph that is
+ * replayed `reps` times between two events.  LPP_PATH_PERSISTENT: `reps` launches of
+ * the one kernel at a frozen position.  LPP_PATH_OPS: every operator of section A as
+ * forward() launches it, stand-alone, one launch per layer, `reps` tokens' worth per
+ * class (the run state is left holding whatever they wrote).  avg_ms is the mean
+ * duration of one launch, bytes the algorithmic HBM bytes of one launch at `pos`. */
 typedef struct lpp_kernel_time {
     char name[32];
     int launches_per_token;

@@ -623,9 +623,10 @@ extern "C" lpp_status lpp_profile_kernels(lpp_model* m, int pos, int reps, lpp_k
     using namespace lpp;
     LPP_REQUIRE(m && out && count && capacity > 0 && reps > 0, "lpp_profile_kernels: bad argument");
     LPP_REQUIRE(pos >= 0 && pos < m->cfg.seq_len, "lpp_profile_kernels: pos %d outside [0, %d)", pos, m->cfg.seq_len);
-    if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
     for (int t = 0; t < LPP_T_COUNT; ++t)
         if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
+    if (m->path == LPP_PATH_OPS) return ops_profile(m, pos, reps, out, capacity, count);
+    if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
     StepParams sp{};
     sp.pos = pos;
     sp.temperature = 0.8f;

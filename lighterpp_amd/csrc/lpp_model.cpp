@@ -326,6 +326,96 @@ lpp_status forward_ops(lpp_model* m, int token, int pos, float temperature, floa
 
 }  // namespace
 
+}  // extern "C"
+
+// Stand-alone timing of the operators of section A as forward_ops launches them at position `pos`: every class is
+// launched as often as one token launches it (one launch per layer, so successive launches stream different weights),
+// `reps` tokens' worth between two events on the launch stream.  bytes = what the operator has to move at least once
+// (weights or cache rows once, vectors in and out).  The run state is left holding whatever the operators wrote.
+lpp_status lpp::ops_profile(lpp_model* m, int pos, int reps, lpp_kernel_time* out, int capacity, int* count) {
+    const lpp_config& c = m->cfg;
+    const int L = c.n_layers, dim = c.dim, kv = m->kv_dim, hidden = c.hidden_dim, hs = m->head_size, prec = c.weight_precision;
+    const double wb = prec == LPP_WEIGHT_FP16 ? 2.0 : 4.0;
+    const int npos = pos + 1;
+    hipStream_t s = lpp::stream();
+    int n = 0;
+    auto timed = [&](const char* name, int per_token, double bytes, auto launch_layer) -> lpp_status {
+        for (int l = 0; l < (per_token > 0 ? L : 1); ++l) LPP_TRY(launch_layer(l));  // warm-up: code objects, tables
+        LPP_HIP(hipStreamSynchronize(s));
+        LPP_HIP(hipEventRecord(m->ev_a, s));
+        int launches = 0;
+        for (int r = 0; r < reps; ++r)
+            for (int l = 0; l < L; ++l) {
+                const int before = launches;
+                LPP_TRY(launch_layer(l));
+                launches = before + 1;
+            }
+        LPP_HIP(hipEventRecord(m->ev_b, s));
+        LPP_HIP(hipEventSynchronize(m->ev_b));
+        float ms = 0.0f;
+        LPP_HIP(hipEventElapsedTime(&ms, m->ev_a, m->ev_b));
+        if (n < capacity) {
+            std::snprintf(out[n].name, sizeof out[n].name, "%s", name);
+            out[n].launches_per_token = per_token;
+            out[n].avg_ms = static_cast<double>(ms) / launches;
+            out[n].bytes_per_launch = bytes;
+        }
+        ++n;
+        return LPP_OK;
+    };
+    auto gemv_bytes = [&](double rows, double cols) { return rows * cols * wb + 4.0 * cols + 4.0 * rows; };
+    const float* rms_att = static_cast<const float*>(m->w[LPP_T_RMS_ATT]);
+    LPP_TRY(lpp_memset(m->att, 0, static_cast<size_t>(c.n_heads) * c.seq_len * sizeof(float)));
+    LPP_TRY(timed("gemv Wq", L, gemv_bytes(dim, dim), [&](int l) {
+        return lpp_gemv(m->q, m->xb, lpp::weight_at(m, LPP_T_WQ, static_cast<size_t>(l) * dim * dim), m->workspace_f16, dim, dim, prec);
+    }));
+    LPP_TRY(timed("gemv Wk, Wv", 2 * L, gemv_bytes(kv, dim), [&](int l) {
+        return lpp_gemv(m->k, m->xb, lpp::weight_at(m, (l & 1) ? LPP_T_WV : LPP_T_WK, static_cast<size_t>(l) * kv * dim), m->workspace_f16, kv, dim, prec);
+    }));
+    LPP_TRY(timed("gemv Wo", L, gemv_bytes(dim, dim), [&](int l) {
+        return lpp_gemv(m->xb2, m->xb, lpp::weight_at(m, LPP_T_WO, static_cast<size_t>(l) * dim * dim), m->workspace_f16, dim, dim, prec);
+    }));
+    LPP_TRY(timed("gemv W1, W3", 2 * L, gemv_bytes(hidden, dim), [&](int l) {
+        return lpp_gemv(m->hb, m->xb, lpp::weight_at(m, (l & 1) ? LPP_T_W3 : LPP_T_W1, static_cast<size_t>(l) * hidden * dim), m->workspace_f16, hidden, dim, prec);
+    }));
+    LPP_TRY(timed("gemv W2", L, gemv_bytes(dim, hidden), [&](int l) {
+        return lpp_gemv(m->xb2, m->hb, lpp::weight_at(m, LPP_T_W2, static_cast<size_t>(l) * hidden * dim), m->workspace_f16, dim, hidden, prec);
+    }));
+    LPP_TRY(timed("gemv classifier", 1, gemv_bytes(c.vocab_size, dim), [&](int) {
+        return lpp_gemv(m->logits, m->x, m->w[LPP_T_WCLS], m->workspace_f16, c.vocab_size, dim, prec);
+    }));
+    LPP_TRY(timed("convert_f32_to_f16", 0, 6.0 * hidden, [&](int) {  // (never launched by forward: x stays fp32)
+        return lpp_convert_f32_to_f16(static_cast<lpp_half*>(m->workspace_f16), m->hb, hidden);
+    }));
+    LPP_TRY(timed("rmsnorm", 2 * L + 1, 12.0 * dim, [&](int l) { return lpp_rmsnorm(m->xb, m->x, rms_att + static_cast<size_t>(l) * dim, dim); }));
+    LPP_TRY(timed("rope", L, 8.0 * (dim + kv), [&](int) { return lpp_rope(m->q, m->k, pos, dim, kv, hs, c.rope_base); }));
+    LPP_TRY(timed("scatter_kv", L, 12.0 * kv, [&](int l) {
+        return lpp_scatter_kv(m->key_cache, m->value_cache, m->k, m->v, l, pos, c.n_kv_heads, hs, c.seq_len);
+    }));
+    LPP_TRY(timed("multihead_gemv", L, 2.0 * kv * npos + 4.0 * dim + 4.0 * c.n_heads * npos, [&](int l) {
+        return lpp_multihead_gemv(m->att, m->q, m->key_cache, l, pos, c.n_heads, c.n_kv_heads, hs, c.seq_len);
+    }));
+    LPP_TRY(timed("scale_multihead", L, 8.0 * c.n_heads * npos, [&](int) {
+        return lpp_scale_multihead(m->att, 1.0f / sqrtf(static_cast<float>(hs)), c.n_heads, npos, c.seq_len);
+    }));
+    LPP_TRY(timed("softmax_multihead", L, 8.0 * c.n_heads * npos, [&](int) {
+        return lpp_softmax_multihead(m->att, m->att, c.n_heads, npos, c.seq_len);
+    }));
+    LPP_TRY(timed("aggregation_multihead", L, 2.0 * kv * npos + 4.0 * c.n_heads * npos + 4.0 * dim, [&](int l) {
+        return lpp_aggregation_multihead(m->xb, m->value_cache + static_cast<size_t>(l) * kv * c.seq_len, m->att, c.n_heads, npos, hs,
+                                         m->gqa, c.seq_len);
+    }));
+    LPP_TRY(timed("residual_add", 2 * L, 12.0 * dim, [&](int) { return lpp_residual_add(m->x, m->x, m->xb2, dim); }));
+    LPP_TRY(timed("swiglu", L, 12.0 * hidden, [&](int) { return lpp_swiglu(m->hb, m->hb, m->he, hidden); }));
+    LPP_TRY(timed("sample", 1, 8.0 * c.vocab_size, [&](int) {
+        return lpp_sample(m->logits, c.vocab_size, 0.8f, 1.0f, 1.0f, nullptr, 0, m->sampled_token, nullptr, 0.5f);
+    }));
+    *count = n < capacity ? n : capacity;
+    return LPP_OK;
+}
+
+extern "C" {
+
 lpp_status lpp_forward(lpp_model* m, int token, int pos, float temperature, float topp, float penalty,
                        const int* history, int history_len, float r, int* next_token) {
     LPP_TRY(lpp::check_ready(m));

@@ -108,6 +108,9 @@ void prefill_release(lpp_model* m);
 // Implemented in dataflow_decode.hip: why LPP_PATH_PERSISTENT cannot take this model's shape, or nullptr.
 const char* dataflow_unsupported_reason(const lpp_model* m);
 
+// Implemented in lpp_model.cpp: stand-alone timing of the operators of lpp.h section A (lpp_profile_kernels on LPP_PATH_OPS).
+lpp_status ops_profile(lpp_model* m, int pos, int reps, lpp_kernel_time* out, int capacity, int* count);
+
 // Implemented in fused_decode.hip.
 lpp_status fused_prepare(lpp_model* m);
 lpp_status fused_release(lpp_model* m);

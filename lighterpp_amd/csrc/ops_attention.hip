@@ -148,6 +148,105 @@ __global__ __launch_bounds__(kAggThreads) void aggregate_kernel(float* __restric
         out[static_cast<size_t>(h) * head_size + e] = part[e];
 }
 
+// Long contexts: kSplit workgroups per query head, each over a contiguous run of positions, so that the launch has
+// work for every compute unit (one workgroup per head leaves most of them idle and takes 29 us for 8193 positions
+// of the 1B shape).  A workgroup leaves its partial sums in a scratch area that lives in the library's device image
+// (the operator allocates nothing and takes no workspace argument); the workgroup of a head that finishes last adds
+// the partials up, always in split order, so the result does not depend on who finished when.  Calls on different
+// streams would share the scratch: like the reference's operators, these are for one stream.
+constexpr int kAggSplitThreads = 512;
+constexpr int kAggMaxHeads = 256, kAggMaxSplits = 16, kAggPad = 128;
+static __device__ float agg_partials[kAggMaxHeads * kAggMaxSplits * kAggPad];
+static __device__ unsigned agg_tickets[kAggMaxHeads];  // back at zero after every launch
+
+template <int kGroup>
+__global__ __launch_bounds__(kAggSplitThreads) void aggregate_split_kernel(float* __restrict__ out,
+                                                                           const uint16_t* __restrict__ v_layer,
+                                                                           const float* __restrict__ att, int npos,
+                                                                           int head_size, int gqa, int att_stride,
+                                                                           float* partials, unsigned* tickets) {
+    extern __shared__ __align__(16) float part[];  // [ngroups][hs_pad]
+    __shared__ int is_last;
+    constexpr int kGroups = kAggSplitThreads / kGroup;
+    constexpr int hs_pad = kGroup * 8;
+    const int h = blockIdx.x, split = blockIdx.y, nsplits = gridDim.y;
+    const int sub = static_cast<int>(threadIdx.x) % kGroup;
+    const int grp = static_cast<int>(threadIdx.x) / kGroup;
+    const int chunk = (npos + nsplits - 1) / nsplits;
+    const int t_begin = split * chunk, t_end = min(npos, t_begin + chunk);
+    const uint16_t* vh = v_layer + static_cast<size_t>(h / gqa) * att_stride * head_size + sub * 8;
+    const float* ah = att + static_cast<size_t>(h) * att_stride;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (sub * 8 < head_size) {
+        constexpr int kUnroll = 4;  // rows requested before the first is used
+        for (int t0 = t_begin + grp; t0 < t_end; t0 += kUnroll * kGroups) {
+            uintx4 rows[kUnroll];
+            float w[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int t = t0 + u * kGroups;
+                const bool live = t < t_end;
+                rows[u] = load16(vh + static_cast<size_t>(live ? t : t_begin) * head_size);
+                w[u] = live ? ah[t] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const half8_t vv = as_half8(rows[u]);
+                // (a weight of zero must not meet whatever the clamped row holds)
+                if (w[u] != 0.0f) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = fmaf(static_cast<float>(vv[e]), w[u], acc[e]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[grp * hs_pad + sub * 8 + e] = acc[e];
+    __syncthreads();
+    for (int width = kGroups / 2; width >= 1; width >>= 1) {
+        for (int i = threadIdx.x; i < width * hs_pad; i += kAggSplitThreads) part[i] += part[i + width * hs_pad];
+        __syncthreads();
+    }
+    float* mine = partials + (static_cast<size_t>(h) * kAggMaxSplits + split) * kAggPad;
+    for (int e = threadIdx.x; e < head_size; e += kAggSplitThreads) Mem<true>::st(mine + e, part[e]);
+    // (the barrier waits for this workgroup's stores; the ticket is drawn after it)
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned ticket = __hip_atomic_fetch_add(&tickets[h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = ticket == static_cast<unsigned>(nsplits - 1) ? 1 : 0;
+        if (is_last) __hip_atomic_store(&tickets[h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    const float* all = partials + static_cast<size_t>(h) * kAggMaxSplits * kAggPad;
+    for (int e = threadIdx.x; e < head_size; e += kAggSplitThreads) {
+        float s = Mem<true>::ld(all + e);
+        for (int k = 1; k < nsplits; ++k) s += Mem<true>::ld(all + k * kAggPad + e);
+        out[static_cast<size_t>(h) * head_size + e] = s;
+    }
+}
+
+// Device addresses of the scratch above, per device (the arrays' names are host-side handles only).
+constexpr int kMaxDevices = 64;
+float* g_agg_partials[kMaxDevices] = {};
+unsigned* g_agg_tickets[kMaxDevices] = {};
+lpp_status agg_scratch(float** partials, unsigned** tickets) {
+    int device = -1;
+    LPP_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(LPP_ERR_UNSUPPORTED, "device ordinal %d beyond %d", device, kMaxDevices - 1);
+    if (g_agg_partials[device] == nullptr) {
+        void* p = nullptr;
+        void* t = nullptr;
+        LPP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(agg_partials)));
+        LPP_HIP(hipGetSymbolAddress(&t, HIP_SYMBOL(agg_tickets)));
+        g_agg_partials[device] = static_cast<float*>(p);
+        g_agg_tickets[device] = static_cast<unsigned*>(t);
+    }
+    *partials = g_agg_partials[device];
+    *tickets = g_agg_tickets[device];
+    return LPP_OK;
+}
+
 __global__ __launch_bounds__(kAttThreads) void aggregate_generic_kernel(float* __restrict__ out,
                                                                         const uint16_t* __restrict__ v_layer,
                                                                         const float* __restrict__ att,
@@ -252,6 +351,29 @@ lpp_status lpp_aggregation_multihead(float* d_out, const lpp_half* d_v, const fl
         hipLaunchKernelGGL(aggregate_generic_kernel, dim3(n_heads), dim3(kAttThreads), 0, stream(), d_out,
                            d_v, d_att, seq_len, head_size, gqa_factor, att_stride);
         LPP_CHECK_LAUNCH("aggregate_generic_kernel");
+        return LPP_OK;
+    }
+    // Enough workgroups for the device once a head's context is long (two per compute unit, a few hundred positions each).
+    int splits = (2 * compute_units() + n_heads - 1) / n_heads;
+    if (splits > kAggMaxSplits) splits = kAggMaxSplits;
+    if (splits > seq_len / 256) splits = seq_len / 256;
+    if (splits > 1 && n_heads <= kAggMaxHeads && g >= 1) {
+        float* partials = nullptr;
+        unsigned* tickets = nullptr;
+        LPP_TRY(agg_scratch(&partials, &tickets));
+        const size_t lds_split = static_cast<size_t>(kAggSplitThreads) * 8 * sizeof(float);
+#define LPP_AGG_SPLIT(G)                                                                                              \
+    hipLaunchKernelGGL((aggregate_split_kernel<G>), dim3(n_heads, splits), dim3(kAggSplitThreads), lds_split, stream(), \
+                       d_out, d_v, d_att, seq_len, head_size, gqa_factor, att_stride, partials, tickets)
+        switch (g) {
+            case 1: LPP_AGG_SPLIT(1); break;
+            case 2: LPP_AGG_SPLIT(2); break;
+            case 4: LPP_AGG_SPLIT(4); break;
+            case 8: LPP_AGG_SPLIT(8); break;
+            default: LPP_AGG_SPLIT(16); break;
+        }
+#undef LPP_AGG_SPLIT
+        LPP_CHECK_LAUNCH("aggregate_split_kernel");
         return LPP_OK;
     }
     const size_t lds = static_cast<size_t>(kAggThreads) * 8 * sizeof(float);  // 32 KiB

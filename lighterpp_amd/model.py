@@ -373,10 +373,11 @@ class Model:
         return out[:res.n_tokens].copy(), res
 
     def profile_kernels(self, pos: int, reps: int = 20) -> list:
-        """[(name, launches_per_token, avg_ms, bytes_per_launch)] for the fused path."""
-        arr = (capi.LppKernelTime * 16)()
+        """[(name, launches_per_token, avg_ms, bytes_per_launch)] of the model's current path: the fused kernels, the
+        persistent kernel, or (operator path) each operator of lpp.h section A as a stand-alone launch."""
+        arr = (capi.LppKernelTime * 32)()
         n = C.c_int(0)
-        capi.check(self.lib.lpp_profile_kernels(self.handle, pos, reps, arr, 16, C.byref(n)))
+        capi.check(self.lib.lpp_profile_kernels(self.handle, pos, reps, arr, 32, C.byref(n)))
         return [(arr[i].name.decode(), arr[i].launches_per_token, arr[i].avg_ms, arr[i].bytes_per_launch)
                 for i in range(n.value)]
 
