@@ -65,8 +65,18 @@ constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS 
 constexpr int kMaxHeadPad = 128;
 constexpr int kShortRounds = 2;                    // cache rows per lane group a one-head work item requests at once
 constexpr int kPacedSteps = 2;                     // next-phase rows a streaming wavefront sends out early after a burst
-constexpr int kMaxAttHeads = 2;                    // query heads of one KV head a long-context work item covers
+constexpr int kMaxAttHeads = 4;                    // query heads of one KV head a work item covers at most
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
+
+// The calling thread's lane, worked out on the spot (two instructions the optimiser can neither hoist nor share).
+// Hides dev::lane_id() in this file on purpose: that one is threadIdx.x & 63, a value that then stays live from the
+// kernel's first instruction to its last and is the first thing to be spilled when registers run short -- and a
+// reload from spill space waits for ALL of the wavefront's outstanding memory operations.
+__device__ __forceinline__ int lane_id() {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
 
 typedef unsigned long long u64;
 // Sequence-number base beyond which the host re-zeroes the tagged slots and restarts the count
@@ -132,6 +142,12 @@ struct Tagged {
     int att_group_splits;  // is a few dozen integer divisions); > 0: items cover two heads of a KV head, this many splits
     float inv_sqrt_head;   // 1 / sqrt(head_size), formed on the host (on the device it would sit in a vector register all token long)
     int lane_item_cap;     // contexts up to this many positions take the one-pass item of a head of size 64 (att_lane_item)
+    // A KV head's context split over the workgroups of its XCD (att_xcd_item): xa_chunk > 0 switches it on.
+    int xa_chunk;          // positions per workgroup (a multiple of 8, at most 8 * 64)
+    int xa_active;         // workgroups of a KV head that hold positions at this context length
+    int xa_ppw;            // positions per exchange wavefront: xa_chunk / 8
+    u64* near_part;        // [n_xcc][workgroups per XCD][near_part_stride] partial results, read inside the XCD only
+    int near_part_stride;
     // the step record, except the token id (which the previous launch left in device memory)
     int pos, history_len;
     float temperature, penalty, r;
@@ -151,6 +167,9 @@ struct Blocks {
     int park_rows;  // gate/up rows a workgroup from gu_split on keeps in LDS instead of streaming them (even; 0: none)
     int park_floats;
     int qkv_by_xcc; // > 0: the stacked [Wq; Wk; Wv] rows are dealt out per XCD, this many KV heads (with their query heads) to each
+    int xa_cu_shift;  // att_xcd_item: log2 of the workgroups that share a KV head
+    int xa_opc;       // att_xcd_item: attention outputs each of them combines
+    int kv_floats;    // LDS for the K and V rows of a workgroup's share of a context
     int slice_dim;  // columns per slice of a dim-column row (slice_width)
     int down;   // rows of W2
     int cls;    // rows of the classifier
@@ -838,6 +857,8 @@ struct Lds {
     float* red;      // [kIoWaves][kMaxAttHeads][kRedStride] attention cross-wavefront reduction
     float* gather;   // [gather_floats] attention split partials
     float* park;     // [park_floats] parked gate/up rows (binary16), row after row
+    float* kv;       // [kv_floats] K and V rows of this workgroup's share of a KV head's context (att_xcd_item)
+    unsigned kv_lds; // the same area as an LDS byte address (what M0 takes for loads that land in LDS)
 };
 
 // xs = the tagged vector itself, zero padded to a multiple of 8.  (The streaming
@@ -935,6 +956,10 @@ __device__ __forceinline__ int block_rows(int total, int block, int wg) {
     return n < 0 ? 0 : (n > block ? block : n);
 }
 
+// (defined with the attention items below)
+template <int kHs>
+__device__ __forceinline__ void xcd_att_prefetch(const Ctx& c, const Io& io, const Lds& l, int layer);
+
 __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) {
 #pragma clang fp contract(off)
     const DecodeArgs& a = c.a;
@@ -956,6 +981,14 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     // (a valid address either way, so that the request does not sit behind a branch)
     float first_cos, first_sin;
     pinned_load(cs_row + (first_rotates ? mod_hs(((first_g < dim) ? first_g : first_g - dim) & ~1) >> 1 : 0), first_cos, first_sin);
+    // This layer's share of the context, on its way into LDS while the rows of this phase are multiplied: the phase
+    // is bound by latency, the memory system has room for the bytes, and the attention's inputs are three
+    // hand-over steps away.  (Requested a layer ahead, during the gate/up phase, the same bytes make that phase,
+    // which is bound by bandwidth, longer by more than they take here.)
+    if (c.t.xa_chunk > 0) {
+        if (hs == 64) xcd_att_prefetch<64>(c, io, l, layer);
+        else xcd_att_prefetch<128>(c, io, l, layer);
+    }
     // (a plain loop, not finished_rows with a closure: a local captured by reference is kept in
     // private memory across the wait, and private memory shares the load counter)
     wait_gemv(c.ctl, 4 * layer + kGQkv);
@@ -1654,6 +1687,349 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
     }
 }
 
+// ---------------------------------------------------------------------------
+// A KV head's context split over the workgroups of its XCD
+// ---------------------------------------------------------------------------
+//
+// Where every KV head belongs to one XCD (its rows of Wq/Wk/Wv are formed there: qkv_row), long contexts are
+// shared out among ALL workgroups of that XCD, 2^xa_cu_shift of them per KV head: workgroup `slot` of a KV head
+// takes positions slot * chunk .. slot * chunk + chunk - 1, for all the query heads that read the KV head, so
+// every K and V row is fetched once.  The rows do not depend on this token: each exchange wavefront requests its
+// xa_ppw = chunk / 8 positions straight into LDS (global_load_lds) while the QKV rows of the layer are still
+// being multiplied, so when q arrives the context is on the compute unit and what is left is arithmetic on LDS:
+// a lane holds one position's whole K row and forms its scores for the heads alone; the values are summed with a
+// lane per two dimensions; wavefronts, and then the workgroups of the KV head, are merged by the max-rescale
+// rule of att_group_item.  The partial results and q, k, v travel inside the XCD (publish_near / peek_near); the
+// second merge is itself shared out, xa_opc outputs to each workgroup, and publishes the attention output to
+// the whole device.  An item's cost depends on chunk, not on the context: 8448 positions of the 1B shape are 264
+// per workgroup.  model.cpp:186-198 with the softmax of ops.cpp:56-75, regrouped.
+
+// One 16-byte request per lane straight into LDS: lane i's bytes land at lds_bytes + 16 i.  Inline assembly on
+// purpose: requests made through the builtin have the compiler drain every outstanding memory operation before
+// any later LDS read of the wavefront.  (The address is a vector operand; M0 is written by a scalar move.)
+__device__ __forceinline__ void lds_request16(const void* from, unsigned lds_bytes) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n" ::"v"(from), "s"(lds_bytes) : "memory");
+}
+
+struct XcdShare {
+    int kvh;         // the KV head this workgroup works for
+    int slot;        // its index among that KV head's workgroups
+    int group0;      // rank (within the XCD) of the KV head's first workgroup
+    int t0;          // first position of the calling wavefront
+    int count;       // positions of the calling wavefront at this context length (0: none)
+    bool holds_current;  // the workgroup's share ends with the current position
+};
+__device__ __forceinline__ XcdShare xcd_share(const Ctx& c, int iw) {
+    XcdShare x;
+    const int shift = c.b.xa_cu_shift;
+    const int j = c.rank_in_xcc >> shift;
+    x.slot = c.rank_in_xcc - (j << shift);
+    x.group0 = j << shift;
+    x.kvh = c.xcc * c.b.qkv_by_xcc + j;
+    const int npos = c.pos + 1, chunk = c.t.xa_chunk, ppw = c.t.xa_ppw;
+    const int begin = x.slot * chunk;
+    const int end = min(npos, begin + chunk);
+    x.t0 = begin + iw * ppw;
+    const int n = min(ppw, end - x.t0);
+    x.count = n > 0 ? n : 0;
+    x.holds_current = begin < npos && npos <= begin + chunk;
+    return x;
+}
+// (does this workgroup work for a KV head at all?  An XCD with fewer KV heads than 32 >> shift leaves none idle.)
+
+// LDS image of a workgroup's share (chunk positions p = 0 .. chunk-1): K piece-major -- the 16-byte piece i of
+// position p at i * chunk * 16 + p * 16, so that a lane which holds a position reads its whole row without bank
+// conflicts -- then V as the cache holds it, a position's row after the other.
+template <int kHs>
+__device__ __forceinline__ unsigned xcd_v_offset(int chunk) {
+    return static_cast<unsigned>(chunk) * kHs * 2u;
+}
+
+// The calling wavefront's K and V rows of `layer` (its xa_ppw positions of the share, those before the current
+// position: the current one's rows come with this token's k and v) on their way into l.kv.
+template <int kHs>
+__device__ __forceinline__ void xcd_att_prefetch(const Ctx& c, const Io& io, const Lds& l, int layer) {
+    const DecodeArgs& a = c.a;
+    const XcdShare x = xcd_share(c, io.iw);
+    const int before = min(x.count, c.pos - x.t0);  // rows earlier tokens left in the cache
+    if (before <= 0) return;
+    const int chunk = c.t.xa_chunk, ppw = c.t.xa_ppw;
+    const int lane = fresh_lane();
+    const size_t first = ((static_cast<size_t>(layer) * a.n_kv_heads + x.kvh) * a.seq_len + x.t0) * kHs;
+    const unsigned k_lds = __builtin_amdgcn_readfirstlane(l.kv_lds + static_cast<unsigned>(io.iw * ppw * 16));
+    const unsigned v_lds = __builtin_amdgcn_readfirstlane(l.kv_lds + xcd_v_offset<kHs>(chunk) + static_cast<unsigned>(io.iw * ppw * kHs * 2));
+    if (lane < before) {
+        const char* row = reinterpret_cast<const char*>(a.key_cache + first + static_cast<size_t>(lane) * kHs);
+#pragma unroll
+        for (int i = 0; i < kHs / 8; ++i) lds_request16(row + 16 * i, k_lds + static_cast<unsigned>(i * chunk * 16));
+    }
+    const char* vsrc = reinterpret_cast<const char*>(a.value_cache + first);
+    const int bytes = before * kHs * 2;
+    for (int at = 0; at < bytes; at += 1024)  // (uniform)
+        if (at + lane * 16 < bytes) lds_request16(vsrc + at + lane * 16, v_lds + static_cast<unsigned>(at));
+}
+
+template <int kHs, int kG>
+__device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int layer) {
+    const DecodeArgs& a = c.a;
+    static_assert(kG <= kMaxAttHeads && kG * kHs <= kIoThreads && kIoWaves % kG == 0, "one thread per (head, dimension) in the merge");
+    constexpr int kPieces = kHs / 8;
+    constexpr int kParts = kIoWaves / kG;        // the share's positions in kParts runs of kG wavefronts' worth each
+    constexpr int kStreams = kHs == 64 ? 2 : 1;  // positions a wavefront adds up side by side (a V row is 32 or 64 lanes wide)
+    const int lane = fresh_lane();
+    const XcdShare x = xcd_share(c, io.iw);
+    const int chunk = c.t.xa_chunk, ppw = c.t.xa_ppw;
+    const int share_count = min(c.pos + 1 - x.slot * chunk, chunk);  // positions of the whole share (<= 0: none)
+    const bool active = x.slot < c.t.xa_active;  // (uniform over the workgroup)
+    const unsigned tag_in = c.seq(layer, kQkv), tag_out = c.seq(layer, kAtt);
+    u64* part_all = c.t.near_part + static_cast<size_t>(c.xcc) * (c.nwg / c.t.n_xcc) * c.t.near_part_stride;
+    char* kbase = reinterpret_cast<char*>(l.kv);
+    char* vbase = kbase + xcd_v_offset<kHs>(chunk);
+    float* weights = l.gather;  // [kG][chunk] softmax weights relative to the maximum of the position's part
+    float* stats = l.sc;        // [kG][kParts][2] maximum and sum of weights of head h over part
+
+    if (active) {
+        // q of the KV head's kG query heads into LDS rows 0 .. kG-1 and, where the share ends with the current
+        // position, this token's k and v into that position's rows of the image, rounded as the cache store rounds
+        const u64* near = c.t.near_qkv + static_cast<size_t>(c.xcc) * c.t.near_qkv_stride;
+        const int wanted = (kG + (x.holds_current ? 2 : 0)) * kHs;  // at most 6 * 128 <= 2 * kIoThreads
+        if (io.it < wanted) {
+            auto source = [&](int idx) -> const u64* {
+                const int which = idx / kHs, e = idx - which * kHs;
+                return near + (which < kG ? static_cast<size_t>(x.kvh * kG + which) * kHs + e
+                                          : a.dim + (which == kG ? 0 : a.kv_dim) + static_cast<size_t>(x.kvh) * kHs + e);
+            };
+            const int second = io.it + kIoThreads < wanted ? io.it + kIoThreads : io.it;
+            float in[2];
+            poll_near_2([&](int j) -> const u64* { return source(j == 0 ? io.it : second); }, in, tag_in, c);
+            const int lc = share_count - 1;  // the current position within the share
+            for (int j = 0; j < (second != io.it ? 2 : 1); ++j) {
+                const int idx = j == 0 ? io.it : second;
+                const int which = idx / kHs, e = idx - which * kHs;
+                if (which < kG) {
+                    l.qkv[which * kMaxHeadPad + e] = in[j];
+                } else {
+                    const uint16_t bits = f32_to_f16_bits(in[j]);
+                    char* at = which == kG ? kbase + (e >> 3) * chunk * 16 + lc * 16 + (e & 7) * 2 : vbase + lc * (kHs * 2) + e * 2;
+                    *reinterpret_cast<uint16_t*>(at) = bits;
+                }
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's requested rows are in LDS
+    mark(c, io, 5);
+    signal_received(c.ctl);
+    io_sync(c.ctl, io);
+    mark(c, io, 1);
+    mark(c, io, 6);
+    mark(c, io, 2);
+
+    if (active) {
+        // Scores: wavefront (h, part) takes head h over the part's positions, a LANE per position: the lane reads
+        // its position's K row (pieces side by side in LDS) and forms the dot product alone; q is read once per
+        // wavefront, four pieces at a time, and kept while the part's passes of 64 positions go by.
+        {
+            const int h = io.iw % kG, part = io.iw / kG;
+            const int first = part * kG * ppw;
+            const int n = min(share_count - first, kG * ppw);  // positions of the part (<= 0: none)
+            float sc[kG];
+#pragma unroll
+            for (int j = 0; j < kG; ++j) sc[j] = 0.0f;
+            if (n > 0) {  // (uniform)
+#pragma unroll
+                for (int r = 0; r < kPieces / 4; ++r) {
+                    compiler_fence();
+                    __builtin_amdgcn_sched_barrier(0);
+                    floatx4 qa[4], qb[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        qa[i] = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + 8 * (4 * r + i));
+                        qb[i] = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + 8 * (4 * r + i) + 4);
+                    }
+#pragma unroll
+                    for (int j = 0; j < kG; ++j) {
+                        if (j * kWave < n) {  // (uniform)
+                            const int p = j * kWave + lane;
+                            const int my = first + (p < n ? p : 0);  // (lanes past the part read its first row; their scores are dropped)
+                            uintx4 kbits[4];
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) kbits[i] = *reinterpret_cast<const uintx4*>(kbase + (4 * r + i) * chunk * 16 + my * 16);
+                            __builtin_amdgcn_sched_barrier(0);  // (left alone, the scheduler pairs every read with its use)
+                            float part4[4];
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) part4[i] = dot8(kbits[i], qa[i], qb[i], 0.0f);
+                            sc[j] += (part4[0] + part4[1]) + (part4[2] + part4[3]);
+                            // (the sum is wanted HERE: without a use in place the multiply-adds are sunk to where the
+                            // score is first needed, behind every other round's reads, and all the rows wait in registers)
+                            asm volatile("" : "+v"(sc[j]));
+                        }
+                    }
+                }
+            }
+            float top = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < kG; ++j) {
+                sc[j] = (j * kWave + lane < n) ? sc[j] * c.t.inv_sqrt_head : -INFINITY;  // model.cpp:188
+                top = fmaxf(top, sc[j]);
+            }
+            top = wave_max(top);
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < kG; ++j) {
+                const float w = (sc[j] == -INFINITY) ? 0.0f : exp_fast(sc[j] - top);
+                sum += w;
+                if (j * kWave + lane < kG * ppw) weights[h * chunk + first + j * kWave + lane] = w;
+            }
+            sum = wave_sum(sum);
+            if (lane == 0) {
+                stats[(h * kParts + part) * 2] = top;
+                stats[(h * kParts + part) * 2 + 1] = sum;
+            }
+        }
+        io_sync(c.ctl, io);
+        // Values: wavefront w takes its own xa_ppw positions for all heads; lane (stream, pair) adds up dimensions
+        // 2 pair, 2 pair + 1 over positions stream, stream + kStreams, ...: four positions' values and weights are
+        // requested before the first is used.
+        float out[kG][2];
+#pragma unroll
+        for (int h = 0; h < kG; ++h) out[h][0] = out[h][1] = 0.0f;
+        if (x.count > 0) {  // (uniform over the wavefront)
+            const int stream = kStreams == 2 ? lane >> 5 : 0, pair = kStreams == 2 ? (lane & 31) : lane;
+            const int w0 = io.iw * ppw;
+            const int iters = (x.count + kStreams - 1) / kStreams;
+            for (int i0 = 0; i0 < iters; i0 += 4) {
+                __builtin_amdgcn_sched_barrier(0);
+                unsigned bits[4];
+                float wv[kG][4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int p = (i0 + u) * kStreams + stream;
+                    const int at = w0 + (p < x.count ? p : 0);
+                    bits[u] = *reinterpret_cast<const unsigned*>(vbase + at * (kHs * 2) + pair * 4);
+#pragma unroll
+                    for (int h = 0; h < kG; ++h) wv[h][u] = weights[h * chunk + at];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int p = (i0 + u) * kStreams + stream;
+                    // (what lies past the share may be anything, NaN included: its weight is zero, the value must be too)
+                    const unsigned b = p < x.count ? bits[u] : 0u;
+                    const float lo = f16_bits_to_f32(static_cast<uint16_t>(b & 0xffffu)), hi = f16_bits_to_f32(static_cast<uint16_t>(b >> 16));
+#pragma unroll
+                    for (int h = 0; h < kG; ++h) {
+                        const float wgt = p < x.count ? wv[h][u] : 0.0f;
+                        out[h][0] = fmaf(wgt, lo, out[h][0]);
+                        out[h][1] = fmaf(wgt, hi, out[h][1]);
+                    }
+                }
+            }
+            if (kStreams == 2) {
+#pragma unroll
+                for (int h = 0; h < kG; ++h) {
+                    out[h][0] += lane_xor(out[h][0], 32, lane);
+                    out[h][1] += lane_xor(out[h][1], 32, lane);
+                }
+            }
+        }
+        {
+            const int pair = kStreams == 2 ? (lane & 31) : lane;
+            if (kStreams == 1 || lane < 32) {
+#pragma unroll
+                for (int h = 0; h < kG; ++h) {
+                    float* r = l.red + (io.iw * kMaxAttHeads + h) * kRedStride;
+                    r[2 * pair] = out[h][0];
+                    r[2 * pair + 1] = out[h][1];
+                }
+            }
+        }
+    }
+    mark(c, io, 7);
+    io_sync(c.ctl, io);
+    mark(c, io, 3);
+    if (active && io.it < kG * kHs) {  // thread (h, e): this workgroup's partial result, to the XCD's copy
+        const int h = io.it / kHs, e = io.it - h * kHs;
+        float ptop[kParts], psum[kParts], wout[kIoWaves];
+#pragma unroll
+        for (int q = 0; q < kParts; ++q) {
+            ptop[q] = stats[(h * kParts + q) * 2];
+            psum[q] = stats[(h * kParts + q) * 2 + 1];
+        }
+#pragma unroll
+        for (int w = 0; w < kIoWaves; ++w) wout[w] = l.red[(w * kMaxAttHeads + h) * kRedStride + e];
+        __builtin_amdgcn_sched_barrier(0);
+        float all = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < kParts; ++q) all = fmaxf(all, ptop[q]);
+        float o = 0.0f, ls = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kParts; ++q) {
+            const float f = (ptop[q] == -INFINITY) ? 0.0f : exp_fast(ptop[q] - all);
+            ls += psum[q] * f;
+#pragma unroll
+            for (int w = q * kG; w < (q + 1) * kG; ++w) o += wout[w] * f;  // (a part's wavefronts: q * kG ..)
+        }
+        u64* mine = part_all + static_cast<size_t>(c.rank_in_xcc) * c.t.near_part_stride + h * (kHs + 2);
+        publish_near(mine + e, o, tag_out);
+        if (e == 0) {
+            publish_near(mine + kHs, all, tag_out);
+            publish_near(mine + kHs + 1, ls, tag_out);
+        }
+    }
+    // The second merge, shared out: this workgroup combines outputs slot * opc .. of the KV head's kG * kHs, all of
+    // one query head.  Thread (e, s) fetches output e of workgroup s's partial result with that result's maximum
+    // and sum, all three requested at once; the 32 workgroups of an output sit in the two 16-lane rows of half a
+    // wavefront and are merged by lane exchange: no LDS, no barrier.
+    const int opc = c.b.xa_opc;
+    const int first_out = x.slot * opc;
+    const int hd = first_out / kHs, e0 = first_out - hd * kHs;
+    const int it = exchange_thread_index(io.iw);
+    const int s = it & 31, e = it >> 5;
+    if (e < opc) {  // (whole wavefronts)
+        float val = 0.0f, top = -INFINITY, sum = 0.0f;
+        if (s < c.t.xa_active) {
+            const u64* theirs = part_all + static_cast<size_t>(x.group0 + s) * c.t.near_part_stride + hd * (kHs + 2);
+            const u64* p0 = theirs + e0 + e;
+            const u64* p1 = theirs + kHs;
+            const u64* p2 = theirs + kHs + 1;
+            u64 g0, g1, g2;
+            unsigned spins = 0;
+            while (true) {
+                asm volatile(
+                    "global_load_dwordx2 %0, %3, off nt\n\tglobal_load_dwordx2 %1, %4, off nt\n\t"
+                    "global_load_dwordx2 %2, %5, off nt\n\ts_waitcnt vmcnt(0)"
+                    : "=&v"(g0), "=&v"(g1), "=&v"(g2)
+                    : "v"(p0), "v"(p1), "v"(p2)
+                    : "memory");
+                if (tag_of(g0) == tag_out && tag_of(g1) == tag_out && tag_of(g2) == tag_out) break;
+                if (poll_give_up(c, spins)) break;
+            }
+            val = value_of(g0);
+            top = value_of(g1);
+            sum = value_of(g2);
+        }
+        const int lane = fresh_lane();
+        auto half_max = [&](float v) {
+            v = fmaxf(v, dpp_move<kDppXor1>(v));
+            v = fmaxf(v, dpp_move<kDppXor2>(v));
+            v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+            v = fmaxf(v, dpp_move<kDppMirror>(v));
+            return fmaxf(v, lane_xor(v, 16, lane));
+        };
+        auto half_sum = [&](float v) {
+            v += dpp_move<kDppXor1>(v);
+            v += dpp_move<kDppXor2>(v);
+            v += dpp_move<kDppHalfMirror>(v);
+            v += dpp_move<kDppMirror>(v);
+            return v + lane_xor(v, 16, lane);
+        };
+        const float all = half_max(top);
+        const float f = (top == -INFINITY) ? 0.0f : exp_fast(top - all);
+        const float o = half_sum(val * f), ls = half_sum(sum * f);
+        if (s == 0) publish(c.t.xb + static_cast<size_t>(x.kvh * kG + hd) * kHs + e0 + e, o / ls, tag_out);
+    }
+}
+
 // Combine the context splits of head h: collect every split's (output, max,
 // sum), rescale to the common maximum and normalise.  Runs after the workgroup
 // has published all of its own partials, so a workgroup waiting here never
@@ -1739,6 +2115,22 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
     mark(c, io, 0);
     // Long contexts of grouped-query models: one item covers the heads that share a KV head (four at a
     // time), so that the cache is read once.  Short contexts keep one item per head and no combine pass.
+    if (c.t.xa_chunk > 0) {
+        io.it = exchange_thread_index(io.iw);
+        if (hs == 64) {
+            if (a.gqa == 4) att_xcd_item<64, 4>(c, io, l, layer);
+            else if (a.gqa == 2) att_xcd_item<64, 2>(c, io, l, layer);
+            else att_xcd_item<64, 1>(c, io, l, layer);
+        } else {
+            if (a.gqa == 4) att_xcd_item<128, 4>(c, io, l, layer);
+            else if (a.gqa == 2) att_xcd_item<128, 2>(c, io, l, layer);
+            else att_xcd_item<128, 1>(c, io, l, layer);
+        }
+        park_fetch(c, io, l, layer);
+        mark(c, io, 4);
+        ++c.phase_index;
+        return;
+    }
     constexpr int heads_per_item = 2;
     if (c.t.att_group_splits > 0) {
         const int n_chunks = a.n_heads / heads_per_item;
@@ -2053,6 +2445,11 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.red = l.qkv + (kMaxAttHeads + 2) * kMaxHeadPad;
     l.gather = l.red + kIoWaves * kMaxAttHeads * kRedStride;
     l.park = l.gather + b.gather_floats;
+    l.kv = l.park + b.park_floats;
+    // (the LDS address is taken from the array itself, where the address space is plain to the compiler, and the
+    // area's offset added as a number: a pointer that has been through a structure is not reliably traced back)
+    l.kv_lds = static_cast<unsigned>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)) +
+               static_cast<unsigned>((l.kv - lds) * sizeof(float));
     for (unsigned i = threadIdx.x; i < sizeof(Control) / sizeof(unsigned); i += blockDim.x)
         reinterpret_cast<unsigned*>(&ctl)[i] = 0u;
     __syncthreads();  // the only workgroup-wide barrier: the two kinds of wavefronts part ways here
@@ -2139,6 +2536,12 @@ Plan plan_for(const lpp_model* m, bool parking) {
     if (b.cls * b.ns_dim > slots) slots = b.cls * b.ns_dim;
     b.results_floats = (slots + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
+    // (att_xcd_item keeps its softmax weights and the second merge's table there)
+    const int xcd_att_floats = df::kIoWaves * df::kMaxAttHeads * df::kWave + 32 * (df::kMaxHeadPad / 8 + 2);
+    if (b.gather_floats < xcd_att_floats) b.gather_floats = xcd_att_floats;
+    b.xa_cu_shift = 0;
+    b.xa_opc = 0;
+    b.kv_floats = 0;
     b.slice_dim = df::slice_width(c.dim, chunk_cols);
     b.gu_a = b.gu;
     b.gu_split = 0;
@@ -2147,7 +2550,7 @@ Plan plan_for(const lpp_model* m, bool parking) {
     auto lds_floats = [&]() {
         return static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
                                    (df::kMaxAttHeads + 2) * df::kMaxHeadPad + df::kIoWaves * df::kMaxAttHeads * df::kRedStride +
-                                   b.gather_floats + b.park_floats);
+                                   b.gather_floats + b.park_floats + b.kv_floats);
     };
     // Parked gate/up rows: whatever LDS is left (binary16 models; the workgroups that hold the attention
     // items of a short context, one per query head, park nothing and own that many fewer hidden units).
@@ -2179,6 +2582,7 @@ Plan plan_for(const lpp_model* m, bool parking) {
 
 constexpr int kGridCap = 1024;  // workgroups the statistics table has room for
 constexpr int kMaxXcc = 8;
+constexpr int kMaxPerXcc = 32;  // workgroups of one XCD the XCD-wide attention split is laid out for
 // Tagged values of one XCD's copy of an n-value vector: whole 128-byte lines.
 size_t near_stride(int n) { return (static_cast<size_t>(n) + 15) / 16 * 16; }
 
@@ -2186,7 +2590,8 @@ size_t tagged_count(const lpp_model* m, int grid_cap) {
     const lpp_config& c = m->cfg;
     return static_cast<size_t>(c.dim) * 3 + static_cast<size_t>(m->kv_dim) * 2 + c.hidden_dim +
            static_cast<size_t>(c.n_heads) * splits_cap_for(m) * (m->head_size + 2) + 4u * grid_cap +
-           32u + static_cast<size_t>(kMaxXcc) * (near_stride(c.hidden_dim) + near_stride(c.dim + 2 * m->kv_dim));
+           32u + static_cast<size_t>(kMaxXcc) * (near_stride(c.hidden_dim) + near_stride(c.dim + 2 * m->kv_dim)) +
+           static_cast<size_t>(kMaxXcc) * kMaxPerXcc * near_stride(m->gqa * (m->head_size + 2));
 }
 
 // Positions a one-head attention item of a head of size 64 can keep on the compute unit (att_lane_item): two 8-KiB
@@ -2200,6 +2605,33 @@ int lane_item_positions(const lpp_model* m, const Plan& p) {
     if (cap > df::kLaneItemPositions) cap = df::kLaneItemPositions;
     const int in_cache = m->cfg.seq_len / df::kWave * df::kWave;
     return cap < in_cache ? cap : in_cache;
+}
+
+// The split of a KV head's context over the workgroups of its XCD (att_xcd_item) at npos positions, for a plan whose
+// Wq/Wk/Wv rows are dealt out per XCD; chunk 0 where it does not apply.
+struct XcdAttention {
+    int chunk, active, ppw, cu_shift, opc, kv_floats;
+};
+XcdAttention xcd_attention_for(const lpp_model* m, const df::Blocks& b, int grid, int npos) {
+    XcdAttention x = {};
+    if (test_option(LPP_OPT_DECODE_XCD_ATTENTION) == 0 || b.qkv_by_xcc <= 0 || m->df_xcc <= 1) return x;
+    const int hs = m->head_size, g = m->gqa;
+    if ((hs != 64 && hs != 128) || (g != 1 && g != 2 && g != 4)) return x;
+    const int per_xcc = grid / m->df_xcc;
+    if (per_xcc > kMaxPerXcc || per_xcc % b.qkv_by_xcc != 0) return x;
+    const int n_cu = per_xcc / b.qkv_by_xcc;  // workgroups that share a KV head
+    if ((n_cu & (n_cu - 1)) != 0 || (g * hs) % n_cu != 0) return x;
+    const int opc = g * hs / n_cu;            // outputs each of them combines: all of one head, at most 16
+    if (opc > hs || hs % opc != 0 || opc > df::kMaxHeadPad / 8) return x;
+    const int chunk = ((npos + n_cu - 1) / n_cu + 7) & ~7;
+    if (chunk > df::kIoWaves * df::kWave) return x;
+    while ((1 << x.cu_shift) < n_cu) ++x.cu_shift;
+    x.chunk = chunk;
+    x.active = (npos + chunk - 1) / chunk;
+    x.ppw = chunk / df::kIoWaves;
+    x.opc = opc;
+    x.kv_floats = chunk * hs;  // eight wavefronts x ppw positions x (K row + V row) of binary16
+    return x;
 }
 
 df::Tagged tagged_of(const lpp_model* m, bool generating, int lane_item_cap) {
@@ -2218,7 +2650,10 @@ df::Tagged tagged_of(const lpp_model* m, bool generating, int lane_item_cap) {
     t.near_hidden_stride = static_cast<int>(near_stride(c.hidden_dim));
     t.near_hb = p;      p += static_cast<size_t>(kMaxXcc) * t.near_hidden_stride;
     t.near_qkv_stride = static_cast<int>(near_stride(c.dim + 2 * m->kv_dim));
-    t.near_qkv = p;
+    t.near_qkv = p;     p += static_cast<size_t>(kMaxXcc) * t.near_qkv_stride;
+    t.near_part_stride = static_cast<int>(near_stride(m->gqa * (m->head_size + 2)));
+    t.near_part = p;
+    t.xa_chunk = t.xa_active = t.xa_ppw = 0;
     t.tickets = m->sync_words + 96;
     t.ticket_base = m->df_ticket_base;
     {
@@ -2446,8 +2881,35 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     const Plan parked_plan = plan_for(m, parking_allowed);
     const int lane_cap = lane_item_positions(m, parked_plan);
     df::Tagged tagged = tagged_of(m, a.uniforms != nullptr, lane_cap);
-    const bool use_parked = parked_plan.blocks.park_rows > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0;
-    const Plan p = use_parked ? parked_plan : plan_for(m, false);
+    // Contexts beyond what the plan with parked gate/up rows covers (one work item per head: the one-pass item's
+    // reach for heads of size 64, the cost model's choice otherwise): a KV head's context is split over the
+    // workgroups of its XCD, if the shape allows and the rows fit LDS.  That plan parks no gate/up rows (the rows'
+    // LDS holds the context instead: at the 8B shape the parked rows are worth more than the faster attention, 3087
+    // against 2844 us per token at 100 positions) and shares the step lists of the plan without parking.
+    constexpr size_t kLdsLimit = 160 * 1024 - 2048;
+    Plan xcd_plan = plan_for(m, false);
+    XcdAttention xa = {};
+    {
+        const int npos = m->df_pos + 1;
+        const bool wanted = m->head_size == 64 ? npos > lane_cap : (tagged.att_splits > 1 || tagged.att_group_splits > 0);
+        if (wanted) xa = xcd_attention_for(m, xcd_plan.blocks, xcd_plan.grid, npos);
+        if (xa.chunk > 0) {
+            xcd_plan.blocks.kv_floats = xa.kv_floats;
+            xcd_plan.blocks.xa_cu_shift = xa.cu_shift;
+            xcd_plan.blocks.xa_opc = xa.opc;
+            xcd_plan.lds_bytes += static_cast<size_t>(xa.kv_floats) * sizeof(float);
+            if (xcd_plan.lds_bytes > kLdsLimit) xa.chunk = 0;
+        }
+    }
+    if (xa.chunk > 0) {
+        tagged.xa_chunk = xa.chunk;
+        tagged.xa_active = xa.active;
+        tagged.xa_ppw = xa.ppw;
+        tagged.att_splits = 1;
+        tagged.att_group_splits = 0;
+    }
+    const bool use_parked = xa.chunk == 0 && parked_plan.blocks.park_rows > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0;
+    const Plan p = xa.chunk > 0 ? xcd_plan : (use_parked ? parked_plan : plan_for(m, false));
     const int which = use_parked ? 1 : 0;
     // q, k and v stay inside the XCD that formed them while every head's item sits on that XCD: one item per head
     tagged.local_qkv = (p.blocks.qkv_by_xcc > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0) ? 1 : 0;
@@ -2465,7 +2927,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
         LPP_REQUIRE(p.grid <= kGridCap, "persistent decode: %d compute units exceed the statistics table", p.grid);
         LPP_REQUIRE(m->head_size <= df::kMaxHeadPad, "persistent decode: head_size %d exceeds %d", m->head_size,
                     df::kMaxHeadPad);
-        const size_t lds_most = parked_plan.lds_bytes > p.lds_bytes ? parked_plan.lds_bytes : p.lds_bytes;
+        const size_t lds_most = kLdsLimit;  // (every launch brings its own size, up to what a compute unit has)
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&df::k_decode_dataflow<kF16>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_most)) != hipSuccess)
             return fail(LPP_ERR_UNSUPPORTED, "persistent decode needs %zu bytes of LDS per workgroup", lds_most);
@@ -2491,6 +2953,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
         LPP_TRY(build_step_lists(m, use_parked ? plan_for(m, false) : parked_plan, 1 - which));
     // (test hook: a ticket base one launch behind makes every workgroup's ticket look like one too many for its XCD)
     if (tagged.n_xcc > 1 && take_forced_ticket_failure()) tagged.ticket_base -= static_cast<unsigned>(m->persist_grid / tagged.n_xcc);
+    LPP_REQUIRE(p.lds_bytes <= kLdsLimit, "persistent decode: %zu bytes of LDS per workgroup", p.lds_bytes);
     hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a, tagged,
                        p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
     LPP_CHECK_LAUNCH("k_decode_dataflow");

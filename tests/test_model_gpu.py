@@ -374,6 +374,57 @@ def test_persistent_relaunches_a_token_when_an_xcd_is_dealt_unevenly(test_option
     o.close()
 
 
+XCD_SPLIT = {
+    # name: (shape, first positions of the runs).  Where every KV head belongs to one XCD, contexts beyond the
+    # one-pass item's 512 positions (heads of size 64) or beyond 96 (size 128) are split over that XCD's workgroups.
+    "hs64_gqa4_8kv_long": (Shape(2048, 512, 1, 32, 8, 500, 9000, 500000.0, fp16=True, tied=True), (600, 4093, 8441)),
+    "hs128_gqa4_8kv": (Shape(4096, 512, 1, 32, 8, 500, 1300, 500000.0, fp16=True, tied=False), (93, 500, 1050)),
+    "hs128_mha_8kv": (Shape(1024, 512, 1, 8, 8, 500, 700, 10000.0, fp16=True, tied=True), (120, 640)),
+    "hs64_mha_32kv": (Shape(2048, 512, 1, 32, 32, 500, 4200, 10000.0, fp16=True, tied=True), (520, 4090)),
+    "hs64_gqa2_16kv": (Shape(2048, 512, 1, 32, 16, 500, 1100, 500000.0, fp16=True, tied=False), (515, 1000)),
+}
+
+
+@pytest.mark.parametrize("name", list(XCD_SPLIT))
+def test_context_split_over_an_xcd_matches_oracle(name):
+    """The long-context attention of the persistent path (a KV head's context shared out among the workgroups of its
+    XCD, rows resident in LDS): six steps from each start on a cache of seeded values, NaN bit patterns past the
+    context on the GPU (whole rows are fetched ahead, nothing past the current position may be used), logits and
+    greedy ids against the oracle.  Starts sit on both sides of where the library switches to this item, at
+    share sizes that fill an exchange wavefront's 64 positions unevenly, and next to the largest context a shape takes."""
+    shape, starts = XCD_SPLIT[name]
+    m, o = build(shape, 17)
+    m.set_path(capi.PATH_PERSISTENT)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    n = L * nkv * shape.seq_len * hs
+    kfill = capi.synth_normal_f16(n, 701, 1.0).reshape(L, nkv, shape.seq_len, hs)
+    vfill = capi.synth_normal_f16(n, 702, 1.0).reshape(L, nkv, shape.seq_len, hs)
+    for start in starts:
+        k_gpu, v_gpu = kfill.copy(), vfill.copy()
+        k_gpu[:, :, start:, :] = 0x7e00  # binary16 NaN
+        v_gpu[:, :, start:, :] = 0x7e00
+        m.reset()
+        m.write_buffer(capi.B_KEY_CACHE, k_gpu)
+        m.write_buffer(capi.B_VALUE_CACHE, v_gpu)
+        k_cpu, v_cpu = kfill.copy(), vfill.copy()
+        k_cpu[:, :, start:, :] = 0
+        v_cpu[:, :, start:, :] = 0
+        o.buf("key_cache")[:] = capi.f16_to_f32(k_cpu.reshape(-1))
+        o.buf("value_cache")[:] = capi.f16_to_f32(v_cpu.reshape(-1))
+        tok = 5
+        for pos in range(start, min(start + 6, shape.seq_len)):
+            print(f"xcd split {name}: pos {pos}", flush=True)
+            nxt = m.forward(tok, pos, 0.0)
+            want = o.forward_logits(tok, pos)
+            got = m.buffer(capi.B_LOGITS)
+            assert np.all(np.isfinite(got)), (start, pos)
+            assert rel_err(got, want) <= LOGIT_TOL, (start, pos)
+            assert nxt == int(np.argmax(want)), (start, pos)
+            tok = nxt
+    m.close()
+    o.close()
+
+
 def test_model_argument_errors():
     shape = SMALL_SHAPES["gqa4_fp16"]
     m = Model(shape)
