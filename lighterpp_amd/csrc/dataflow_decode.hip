@@ -65,18 +65,9 @@ constexpr int kAttScoreFloats = 512;               // half of the sampler's LDS 
 constexpr int kMaxHeadPad = 128;
 constexpr int kShortRounds = 2;                    // cache rows per lane group a one-head work item requests at once
 constexpr int kPacedSteps = 2;                     // next-phase rows a streaming wavefront sends out early after a burst
-constexpr int kMaxAttHeads = 4;                    // query heads of one KV head a work item covers at most
+constexpr int kMaxAttHeads = 4;                    // query heads of one KV head a work item of att_xcd_item covers at most
+constexpr int kItemHeads = 2;                      // the same for the items dealt out over the device (att_group_item)
 constexpr int kRedStride = kMaxHeadPad + 2;        // one wavefront's partial result of one head: values, maximum, sum
-
-// The calling thread's lane, worked out on the spot (two instructions the optimiser can neither hoist nor share).
-// Hides dev::lane_id() in this file on purpose: that one is threadIdx.x & 63, a value that then stays live from the
-// kernel's first instruction to its last and is the first thing to be spilled when registers run short -- and a
-// reload from spill space waits for ALL of the wavefront's outstanding memory operations.
-__device__ __forceinline__ int lane_id() {
-    int lane;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
-    return lane;
-}
 
 typedef unsigned long long u64;
 // Sequence-number base beyond which the host re-zeroes the tagged slots and restarts the count
@@ -178,6 +169,7 @@ struct Blocks {
     int xs_floats;
     int results_floats;
     int gather_floats;
+    int red_floats;   // LDS for the cross-wavefront merge of the attention items
 };
 
 // Hidden units of a workgroup: a contiguous run, gu_a units for each of the first gu_split workgroups, gu for the rest.
@@ -960,6 +952,7 @@ __device__ __forceinline__ int block_rows(int total, int block, int wg) {
 template <int kHs>
 __device__ __forceinline__ void xcd_att_prefetch(const Ctx& c, const Io& io, const Lds& l, int layer);
 
+template <bool kXcd>
 __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) {
 #pragma clang fp contract(off)
     const DecodeArgs& a = c.a;
@@ -985,9 +978,11 @@ __device__ __forceinline__ void io_qkv(Ctx& c, Io& io, const Lds& l, int layer) 
     // is bound by latency, the memory system has room for the bytes, and the attention's inputs are three
     // hand-over steps away.  (Requested a layer ahead, during the gate/up phase, the same bytes make that phase,
     // which is bound by bandwidth, longer by more than they take here.)
-    if (c.t.xa_chunk > 0) {
-        if (hs == 64) xcd_att_prefetch<64>(c, io, l, layer);
-        else xcd_att_prefetch<128>(c, io, l, layer);
+    if constexpr (kXcd) {
+        if (c.t.xa_chunk > 0) {
+            if (hs == 64) xcd_att_prefetch<64>(c, io, l, layer);
+            else xcd_att_prefetch<128>(c, io, l, layer);
+        }
     }
     // (a plain loop, not finished_rows with a closure: a local captured by reference is kept in
     // private memory across the wait, and private memory shares the load counter)
@@ -1184,7 +1179,7 @@ __device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp
 template <int kGroup, int kHeads, int kRounds>
 __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int layer, int h0, int split, int nsplits,
                                                int npos, bool first_item, int hs) {
-    static_assert(kHeads <= kMaxAttHeads, "LDS areas are sized for kMaxAttHeads heads");
+    static_assert(kHeads <= kItemHeads, "LDS areas are sized for kItemHeads heads");
     const DecodeArgs& a = c.a;
     constexpr int ngroups = kIoThreads / kGroup;
     constexpr int kSub = ngroups * kRounds;
@@ -1346,7 +1341,7 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
     if (lane_id() < kGroup) {
 #pragma unroll
         for (int h = 0; h < kHeads; ++h) {
-            float* r = l.red + (io.iw * kMaxAttHeads + h) * kRedStride;
+            float* r = l.red + (io.iw * kItemHeads + h) * kRedStride;
             if (lane_live) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) r[sub * 8 + e] = acc[h][e];
@@ -1366,11 +1361,11 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
         const int h = div_head_size(c, io.it), e = io.it - h * hs;
         float all = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kIoWaves; ++w) all = fmaxf(all, l.red[(w * kMaxAttHeads + h) * kRedStride + kMaxHeadPad]);
+        for (int w = 0; w < kIoWaves; ++w) all = fmaxf(all, l.red[(w * kItemHeads + h) * kRedStride + kMaxHeadPad]);
         float o = 0.0f, ls = 0.0f;
 #pragma unroll
         for (int w = 0; w < kIoWaves; ++w) {
-            const float* r = l.red + (w * kMaxAttHeads + h) * kRedStride;
+            const float* r = l.red + (w * kItemHeads + h) * kRedStride;
             const float f = (r[kMaxHeadPad] == -INFINITY) ? 0.0f : exp_fast(r[kMaxHeadPad] - all);
             o += r[e] * f;
             ls += r[kMaxHeadPad + 1] * f;
@@ -1556,7 +1551,7 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
         mark(c, io, 2);
     }
 
-    float* red = l.red + (io.iw * kMaxAttHeads) * kRedStride;
+    float* red = l.red + (io.iw * kItemHeads) * kRedStride;
     float top = -INFINITY, lsum = 0.0f, o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
     if (wave_live) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows are in
@@ -1667,7 +1662,7 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
         float wtop[kIoWaves], wsum[kIoWaves], wout[kIoWaves];
 #pragma unroll
         for (int w = 0; w < kIoWaves; ++w) {
-            const float* r = l.red + (w * kMaxAttHeads) * kRedStride;
+            const float* r = l.red + (w * kItemHeads) * kRedStride;
             wtop[w] = r[kMaxHeadPad];
             wsum[w] = r[kMaxHeadPad + 1];
             wout[w] = r[e];
@@ -1719,14 +1714,18 @@ struct XcdShare {
     int count;       // positions of the calling wavefront at this context length (0: none)
     bool holds_current;  // the workgroup's share ends with the current position
 };
-__device__ __forceinline__ XcdShare xcd_share(const Ctx& c, int iw) {
+// (rank, xcc, chunk: the workgroup's rank in its XCD, the XCD and xa_chunk, each passed through an empty asm
+// statement by the caller.  Everything here follows from values that do not change from layer to layer; without
+// an opaque input the optimiser works it all out once, ahead of the layer loop, and the results then occupy
+// scalar registers -- and spill -- for the whole token, in every phase.)
+__device__ __forceinline__ XcdShare xcd_share(const Ctx& c, int iw, int rank, int xcc, int chunk) {
     XcdShare x;
     const int shift = c.b.xa_cu_shift;
-    const int j = c.rank_in_xcc >> shift;
-    x.slot = c.rank_in_xcc - (j << shift);
+    const int j = rank >> shift;
+    x.slot = rank - (j << shift);
     x.group0 = j << shift;
-    x.kvh = c.xcc * c.b.qkv_by_xcc + j;
-    const int npos = c.pos + 1, chunk = c.t.xa_chunk, ppw = c.t.xa_ppw;
+    x.kvh = xcc * c.b.qkv_by_xcc + j;
+    const int npos = c.pos + 1, ppw = chunk >> 3;
     const int begin = x.slot * chunk;
     const int end = min(npos, begin + chunk);
     x.t0 = begin + iw * ppw;
@@ -1750,10 +1749,12 @@ __device__ __forceinline__ unsigned xcd_v_offset(int chunk) {
 template <int kHs>
 __device__ __forceinline__ void xcd_att_prefetch(const Ctx& c, const Io& io, const Lds& l, int layer) {
     const DecodeArgs& a = c.a;
-    const XcdShare x = xcd_share(c, io.iw);
+    int rank = c.rank_in_xcc, xcc = c.xcc, chunk = c.t.xa_chunk;
+    asm volatile("" : "+s"(rank), "+s"(xcc), "+s"(chunk));
+    const XcdShare x = xcd_share(c, io.iw, rank, xcc, chunk);
     const int before = min(x.count, c.pos - x.t0);  // rows earlier tokens left in the cache
     if (before <= 0) return;
-    const int chunk = c.t.xa_chunk, ppw = c.t.xa_ppw;
+    const int ppw = chunk >> 3;
     const int lane = fresh_lane();
     const size_t first = ((static_cast<size_t>(layer) * a.n_kv_heads + x.kvh) * a.seq_len + x.t0) * kHs;
     const unsigned k_lds = __builtin_amdgcn_readfirstlane(l.kv_lds + static_cast<unsigned>(io.iw * ppw * 16));
@@ -1777,12 +1778,14 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
     constexpr int kParts = kIoWaves / kG;        // the share's positions in kParts runs of kG wavefronts' worth each
     constexpr int kStreams = kHs == 64 ? 2 : 1;  // positions a wavefront adds up side by side (a V row is 32 or 64 lanes wide)
     const int lane = fresh_lane();
-    const XcdShare x = xcd_share(c, io.iw);
-    const int chunk = c.t.xa_chunk, ppw = c.t.xa_ppw;
+    int rank = c.rank_in_xcc, xcc = c.xcc, chunk = c.t.xa_chunk;
+    asm volatile("" : "+s"(rank), "+s"(xcc), "+s"(chunk));
+    const XcdShare x = xcd_share(c, io.iw, rank, xcc, chunk);
+    const int ppw = chunk >> 3;
     const int share_count = min(c.pos + 1 - x.slot * chunk, chunk);  // positions of the whole share (<= 0: none)
     const bool active = x.slot < c.t.xa_active;  // (uniform over the workgroup)
     const unsigned tag_in = c.seq(layer, kQkv), tag_out = c.seq(layer, kAtt);
-    u64* part_all = c.t.near_part + static_cast<size_t>(c.xcc) * (c.nwg / c.t.n_xcc) * c.t.near_part_stride;
+    u64* part_all = c.t.near_part + static_cast<size_t>(xcc) * (c.nwg / c.t.n_xcc) * c.t.near_part_stride;
     char* kbase = reinterpret_cast<char*>(l.kv);
     char* vbase = kbase + xcd_v_offset<kHs>(chunk);
     float* weights = l.gather;  // [kG][chunk] softmax weights relative to the maximum of the position's part
@@ -1791,7 +1794,7 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
     if (active) {
         // q of the KV head's kG query heads into LDS rows 0 .. kG-1 and, where the share ends with the current
         // position, this token's k and v into that position's rows of the image, rounded as the cache store rounds
-        const u64* near = c.t.near_qkv + static_cast<size_t>(c.xcc) * c.t.near_qkv_stride;
+        const u64* near = c.t.near_qkv + static_cast<size_t>(xcc) * c.t.near_qkv_stride;
         const int wanted = (kG + (x.holds_current ? 2 : 0)) * kHs;  // at most 6 * 128 <= 2 * kIoThreads
         if (io.it < wanted) {
             auto source = [&](int idx) -> const u64* {
@@ -1969,7 +1972,7 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
 #pragma unroll
             for (int w = q * kG; w < (q + 1) * kG; ++w) o += wout[w] * f;  // (a part's wavefronts: q * kG ..)
         }
-        u64* mine = part_all + static_cast<size_t>(c.rank_in_xcc) * c.t.near_part_stride + h * (kHs + 2);
+        u64* mine = part_all + static_cast<size_t>(rank) * c.t.near_part_stride + h * (kHs + 2);
         publish_near(mine + e, o, tag_out);
         if (e == 0) {
             publish_near(mine + kHs, all, tag_out);
@@ -2103,6 +2106,7 @@ __host__ __device__ inline int group_item_splits(int npos, int cap, int n_chunks
     return best;
 }
 
+template <bool kXcd>
 __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int layer) {
     const DecodeArgs& a = c.a;
     const int npos = c.pos + 1;
@@ -2115,7 +2119,8 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
     mark(c, io, 0);
     // Long contexts of grouped-query models: one item covers the heads that share a KV head (four at a
     // time), so that the cache is read once.  Short contexts keep one item per head and no combine pass.
-    if (c.t.xa_chunk > 0) {
+    if constexpr (kXcd) {
+      if (c.t.xa_chunk > 0) {
         io.it = exchange_thread_index(io.iw);
         if (hs == 64) {
             if (a.gqa == 4) att_xcd_item<64, 4>(c, io, l, layer);
@@ -2130,6 +2135,7 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
         mark(c, io, 4);
         ++c.phase_index;
         return;
+      }
     }
     constexpr int heads_per_item = 2;
     if (c.t.att_group_splits > 0) {
@@ -2380,7 +2386,7 @@ __device__ __forceinline__ void io_classify_sample(Ctx& c, Io& io, const Lds& l)
     ++c.phase_index;
 }
 
-template <bool kF16>
+template <bool kF16, bool kXcd>
 __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
     const DecodeArgs& a = c.a;
     // The thread index is made opaque before every phase: per-thread addresses are then formed
@@ -2389,9 +2395,9 @@ __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
     auto fresh = [&]() { io.it = exchange_thread_index(io.iw); };
     for (int layer = 0; layer < a.n_layers; ++layer) {
         fresh();
-        io_qkv(c, io, l, layer);
+        io_qkv<kXcd>(c, io, l, layer);
         fresh();
-        io_attention(c, io, l, layer);
+        io_attention<kXcd>(c, io, l, layer);
         fresh();
         io_proj(c, io, l, 4 * layer + kGO, c.b.o, a.dim, c.b.ns_dim, c.t.xb, nullptr, 0, 0, c.seq(layer, kAtt),
                 c.seq(layer, kOproj));
@@ -2410,7 +2416,9 @@ __device__ __forceinline__ void io_role(Ctx& c, Io& io, const Lds& l) {
 // The kernel
 // ---------------------------------------------------------------------------
 
-template <bool kF16>
+// (kXcd: with the item that splits a context over an XCD, att_xcd_item.  A second instance of the kernel rather than
+// a branch in the one: merely compiled in, that item's registers cost every other plan 5 us per token at the 1B shape.)
+template <bool kF16, bool kXcd>
 __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagged t, Blocks b,
                                                               const uint4* __restrict__ row_lists, int row_list_stride) {
     extern __shared__ __align__(16) float lds[];
@@ -2443,7 +2451,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.sc = l.results + b.results_floats;
     l.qkv = l.sc + 2 * kAttScoreFloats;
     l.red = l.qkv + (kMaxAttHeads + 2) * kMaxHeadPad;
-    l.gather = l.red + kIoWaves * kMaxAttHeads * kRedStride;
+    l.gather = l.red + b.red_floats;
     l.park = l.gather + b.gather_floats;
     l.kv = l.park + b.park_floats;
     // (the LDS address is taken from the array itself, where the address space is plain to the compiler, and the
@@ -2468,7 +2476,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
               token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg, wg % n_xcc, wg / n_xcc};
         Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
         if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
-        io_role<kF16>(c, io, l);
+        io_role<kF16, kXcd>(c, io, l);
     }
 }
 
@@ -2536,9 +2544,7 @@ Plan plan_for(const lpp_model* m, bool parking) {
     if (b.cls * b.ns_dim > slots) slots = b.cls * b.ns_dim;
     b.results_floats = (slots + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
-    // (att_xcd_item keeps its softmax weights and the second merge's table there)
-    const int xcd_att_floats = df::kIoWaves * df::kMaxAttHeads * df::kWave + 32 * (df::kMaxHeadPad / 8 + 2);
-    if (b.gather_floats < xcd_att_floats) b.gather_floats = xcd_att_floats;
+    b.red_floats = df::kIoWaves * df::kItemHeads * df::kRedStride;
     b.xa_cu_shift = 0;
     b.xa_opc = 0;
     b.kv_floats = 0;
@@ -2549,8 +2555,8 @@ Plan plan_for(const lpp_model* m, bool parking) {
     b.park_floats = 0;
     auto lds_floats = [&]() {
         return static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
-                                   (df::kMaxAttHeads + 2) * df::kMaxHeadPad + df::kIoWaves * df::kMaxAttHeads * df::kRedStride +
-                                   b.gather_floats + b.park_floats + b.kv_floats);
+                                   (df::kMaxAttHeads + 2) * df::kMaxHeadPad + b.red_floats + b.gather_floats + b.park_floats +
+                                   b.kv_floats);
     };
     // Parked gate/up rows: whatever LDS is left (binary16 models; the workgroups that hold the attention
     // items of a short context, one per query head, park nothing and own that many fewer hidden units).
@@ -2894,6 +2900,14 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
         const bool wanted = m->head_size == 64 ? npos > lane_cap : (tagged.att_splits > 1 || tagged.att_group_splits > 0);
         if (wanted) xa = xcd_attention_for(m, xcd_plan.blocks, xcd_plan.grid, npos);
         if (xa.chunk > 0) {
+            // (the item's LDS beyond the rows: a merge area for four heads, and the softmax weights in `gather`)
+            df::Blocks& xb = xcd_plan.blocks;
+            const int red_more = df::kIoWaves * df::kMaxAttHeads * df::kRedStride - xb.red_floats;
+            const int gather_more = df::kMaxAttHeads * df::kIoWaves * df::kWave > xb.gather_floats
+                                        ? df::kMaxAttHeads * df::kIoWaves * df::kWave - xb.gather_floats : 0;
+            xb.red_floats += red_more;
+            xb.gather_floats += gather_more;
+            xcd_plan.lds_bytes += static_cast<size_t>(red_more + gather_more) * sizeof(float);
             xcd_plan.blocks.kv_floats = xa.kv_floats;
             xcd_plan.blocks.xa_cu_shift = xa.cu_shift;
             xcd_plan.blocks.xa_opc = xa.opc;
@@ -2928,12 +2942,15 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
         LPP_REQUIRE(m->head_size <= df::kMaxHeadPad, "persistent decode: head_size %d exceeds %d", m->head_size,
                     df::kMaxHeadPad);
         const size_t lds_most = kLdsLimit;  // (every launch brings its own size, up to what a compute unit has)
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&df::k_decode_dataflow<kF16>),
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&df::k_decode_dataflow<kF16, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_most)) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&df::k_decode_dataflow<kF16, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_most)) != hipSuccess)
             return fail(LPP_ERR_UNSUPPORTED, "persistent decode needs %zu bytes of LDS per workgroup", lds_most);
-        int per_cu = 0;
-        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, df::k_decode_dataflow<kF16>, df::kThreads, lds_most));
-        if (per_cu < 1)
+        int per_cu = 0, per_cu_xcd = 0;
+        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, df::k_decode_dataflow<kF16, false>, df::kThreads, lds_most));
+        LPP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_xcd, df::k_decode_dataflow<kF16, true>, df::kThreads, lds_most));
+        if (per_cu < 1 || per_cu_xcd < 1)
             return fail(LPP_ERR_UNSUPPORTED, "persistent decode kernel does not fit a compute unit (LDS %zu bytes)", lds_most);
         m->persist_grid = p.grid;
     }
@@ -2954,8 +2971,12 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     // (test hook: a ticket base one launch behind makes every workgroup's ticket look like one too many for its XCD)
     if (tagged.n_xcc > 1 && take_forced_ticket_failure()) tagged.ticket_base -= static_cast<unsigned>(m->persist_grid / tagged.n_xcc);
     LPP_REQUIRE(p.lds_bytes <= kLdsLimit, "persistent decode: %zu bytes of LDS per workgroup", p.lds_bytes);
-    hipLaunchKernelGGL((df::k_decode_dataflow<kF16>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a, tagged,
-                       p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
+    if (xa.chunk > 0)
+        hipLaunchKernelGGL((df::k_decode_dataflow<kF16, true>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a,
+                           tagged, p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
+    else
+        hipLaunchKernelGGL((df::k_decode_dataflow<kF16, false>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a,
+                           tagged, p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
     LPP_CHECK_LAUNCH("k_decode_dataflow");
     m->df_base += df::phases_per_token(m->cfg.n_layers);
     if (tagged.n_xcc > 1) m->df_ticket_base += static_cast<unsigned>(m->persist_grid / tagged.n_xcc);  // one ticket per workgroup
