@@ -481,7 +481,9 @@ enum lpp_test_option {
     LPP_OPT_PREFILL_WIDE_TILES = 7,     /* [1] 256 x 128 tiles where they fill the device                               */
     LPP_OPT_PREFILL_FUSED_FFN = 8,      /* [1] W1, W3 and SwiGLU in one launch                                          */
     LPP_OPT_PREFILL_MFMA_ATTENTION = 9, /* [1] matrix-core attention; 0: one wavefront per token and KV head            */
-    LPP_OPT_COUNT = 10
+    LPP_OPT_DECODE_CALIBRATE = 10,      /* [1] LPP_PATH_PERSISTENT: before a model's first token, trace two tokens and deal the
+                                               hidden units out by how fast each XCD got through the gate/up phase; 0: evenly  */
+    LPP_OPT_COUNT = 11
 };
 lpp_status lpp_set_test_option(int option, int value);
 lpp_status lpp_get_test_option(int option, int *value);

@@ -37,10 +37,10 @@ GGML_F32, GGML_F16 = 0, 1
 # enum lpp_test_option
 (OPT_DECODE_XCD_HANDOVERS, OPT_DECODE_XCD_QKV, OPT_DECODE_PARKING, OPT_DECODE_LANE_ITEM, OPT_DECODE_FAIL_TICKETS,
  OPT_DECODE_XCD_ATTENTION, OPT_PREFILL_STAGED_GEMM, OPT_PREFILL_WIDE_TILES, OPT_PREFILL_FUSED_FFN,
- OPT_PREFILL_MFMA_ATTENTION, OPT_COUNT) = range(11)
+ OPT_PREFILL_MFMA_ATTENTION, OPT_DECODE_CALIBRATE, OPT_COUNT) = range(12)
 OPT_DEFAULTS = {OPT_DECODE_XCD_HANDOVERS: 1, OPT_DECODE_XCD_QKV: 1, OPT_DECODE_PARKING: 1, OPT_DECODE_LANE_ITEM: 1,
                 OPT_DECODE_FAIL_TICKETS: 0, OPT_DECODE_XCD_ATTENTION: 1, OPT_PREFILL_STAGED_GEMM: 1,
-                OPT_PREFILL_WIDE_TILES: 1, OPT_PREFILL_FUSED_FFN: 1, OPT_PREFILL_MFMA_ATTENTION: 1}
+                OPT_PREFILL_WIDE_TILES: 1, OPT_PREFILL_FUSED_FFN: 1, OPT_PREFILL_MFMA_ATTENTION: 1, OPT_DECODE_CALIBRATE: 1}
 TOKENIZER_SENTENCEPIECE, TOKENIZER_BPE = 0, 1
 
 

@@ -146,14 +146,15 @@ struct Tagged {
     unsigned* abort;  // raised by a wavefront whose poll ran out of patience
     unsigned spin_limit;
     int trace_stride;  // timeline: 0 = workgroup 0 only; else every workgroup writes its own block of this many words
+    const int* gu_first;  // [workgroups + 1] first hidden unit of each workgroup (gu_unit0)
 };
 
 // Rows of each matrix one workgroup owns (a contiguous block), and LDS sizes.
 struct Blocks {
     int qkv;    // rows of the stacked [Wq; Wk; Wv], even
     int o;      // rows of Wo
-    int gu;     // hidden units (one gate row and one up row each) of a workgroup from gu_split on
-    int gu_a;   // hidden units of each of the first gu_split workgroups (those that hold the attention items of a short
+    int gu;     // hidden units (one gate row and one up row each) of a workgroup from gu_split on, before the table's scaling
+    int gu_a;   // the same of each of the first gu_split workgroups (those that hold the attention items of a short
     int gu_split;   // context: they park nothing and own fewer units instead)
     int park_rows;  // gate/up rows a workgroup from gu_split on keeps in LDS instead of streaming them (even; 0: none)
     int park_floats;
@@ -172,15 +173,11 @@ struct Blocks {
     int red_floats;   // LDS for the cross-wavefront merge of the attention items
 };
 
-// Hidden units of a workgroup: a contiguous run, gu_a units for each of the first gu_split workgroups, gu for the rest.
-__host__ __device__ inline int gu_unit0(const Blocks& b, int wg) {
-    return wg < b.gu_split ? wg * b.gu_a : b.gu_split * b.gu_a + (wg - b.gu_split) * b.gu;
-}
-__host__ __device__ inline int gu_units(const Blocks& b, int hidden, int wg) {
-    const int block = wg < b.gu_split ? b.gu_a : b.gu;
-    const int n = hidden - gu_unit0(b, wg);
-    return n < 0 ? 0 : (n > block ? block : n);
-}
+// Hidden units of a workgroup: a contiguous run, units first[wg] .. first[wg + 1] - 1 of a table the host makes
+// (gu_a units for each of the first gu_split workgroups, gu for the rest, each share then scaled by what a traced
+// token says about how fast the workgroup's XCD and kind get through the gate/up phase: calibrate_gateup).
+__host__ __device__ inline int gu_unit0(const int* first, int wg) { return first[wg]; }
+__host__ __device__ inline int gu_units(const int* first, int wg) { return first[wg + 1] - first[wg]; }
 // The last rows of the workgroup's gate/up block are the parked ones.
 __host__ __device__ inline int gu_parked_rows(const Blocks& b, int wg, int units) {
     if (wg < b.gu_split) return 0;
@@ -291,6 +288,7 @@ struct Ctx {
     float temperature, penalty, r;
     int wg, nwg;
     int xcc, rank_in_xcc;  // the XCD this workgroup runs on and its index among that XCD's workgroups
+    int gu0, gun;          // this workgroup's hidden units: first, count
 
     __device__ __forceinline__ unsigned seq(int layer, int phase) const {
         return base + 1u + 5u * static_cast<unsigned>(layer) + static_cast<unsigned>(phase);
@@ -1050,11 +1048,11 @@ __device__ __forceinline__ void io_proj(Ctx& c, Io& io, const Lds& l, int gphase
 // first n_heads workgroups, the host launches with the other plan: no parked rows, uniform blocks.
 __device__ __forceinline__ void park_fetch(Ctx& c, Io& io, const Lds& l, int layer) {
     const DecodeArgs& a = c.a;
-    const int units = gu_units(c.b, a.hidden, c.wg);
+    const int units = c.gun;
     const int parked = gu_parked_rows(c.b, c.wg, units);
     if (parked == 0) return;
     const int first_row = 2 * units - parked;
-    const int unit0 = gu_unit0(c.b, c.wg);
+    const int unit0 = c.gu0;
     const int lane = fresh_lane();
     const int row_bytes = a.dim * 2;
     const int loads_per_row = (row_bytes + 1023) >> 10;  // one wavefront load covers 1 KiB
@@ -1093,7 +1091,7 @@ __device__ __forceinline__ void park_fetch(Ctx& c, Io& io, const Lds& l, int lay
 // (one chain of multiply-adds per 1-KiB chunk, added pairwise, then across the wavefront).
 __device__ __forceinline__ void park_multiply(Ctx& c, Io& io, const Lds& l) {
     const DecodeArgs& a = c.a;
-    const int units = gu_units(c.b, a.hidden, c.wg);
+    const int units = c.gun;
     const int parked = gu_parked_rows(c.b, c.wg, units);
     if (parked == 0) return;
     const int first_row = 2 * units - parked;
@@ -1138,8 +1136,8 @@ __device__ __forceinline__ void io_gateup(Ctx& c, Io& io, const Lds& l, int laye
     const float scale =
         stage_norm(c, io, l, c.t.x, nullptr, a.dim, c.seq(layer, kOproj), a.rms_ffn + static_cast<size_t>(layer) * a.dim);
     mark(c, io, 2);
-    const int unit0 = gu_unit0(c.b, c.wg);
-    const int units = gu_units(c.b, a.hidden, c.wg);
+    const int unit0 = c.gu0;
+    const int units = c.gun;
     const unsigned tag = c.seq(layer, kGateUp);
     if (c.b.park_rows > 0) {
         park_multiply(c, io, l);
@@ -2473,7 +2471,8 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
         if (a.trace != nullptr && (wg == 0 || t.trace_stride > 0)) my_trace = a.trace + static_cast<size_t>(wg) * t.trace_stride;
         const int n_xcc = t.n_xcc > 1 ? t.n_xcc : 1;
         Ctx c{a, t, b, ctl, t.base, my_trace, 0u,
-              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg, wg % n_xcc, wg / n_xcc};
+              token_in, t.pos, t.history_len, t.temperature, t.penalty, t.r, wg, nwg, wg % n_xcc, wg / n_xcc,
+              gu_unit0(t.gu_first, wg), gu_units(t.gu_first, wg)};
         Io io{static_cast<int>(threadIdx.x) - kGemvWaves * kWave, wave - kGemvWaves, 0u, 0, a.step};
         if (c.trace && io.it == 0) c.trace[kTraceMarks * phases_per_token(a.n_layers)] = wall_clock64();
         io_role<kF16, kXcd>(c, io, l);
@@ -2503,7 +2502,33 @@ struct Plan {
     int grid;
     df::Blocks blocks;
     size_t lds_bytes;
+    std::vector<int> gu_first;  // [grid + 1] first hidden unit of every workgroup (df::gu_unit0)
 };
+
+// The hidden units dealt out: workgroup w's share is its block of the plan (gu_a or gu units) times its weight
+// (lpp_model::df_gu_weight, 1 until a traced token has said otherwise), scaled so that the shares add up to
+// hidden_dim, with boundaries rounded on the running sum.  most = the largest share.
+std::vector<int> gateup_table(const lpp_model* m, const df::Blocks& b, int grid, int* most) {
+    std::vector<double> share(grid);
+    double total = 0.0;
+    for (int w = 0; w < grid; ++w) {
+        const double weight = static_cast<size_t>(w) < m->df_gu_weight.size() ? m->df_gu_weight[w] : 1.0;
+        share[w] = (w < b.gu_split ? b.gu_a : b.gu) * weight;
+        total += share[w];
+    }
+    std::vector<int> first(grid + 1, 0);
+    double run = 0.0;
+    *most = 0;
+    for (int w = 0; w < grid; ++w) {
+        run += share[w] * m->cfg.hidden_dim / total;
+        int end = w + 1 == grid ? m->cfg.hidden_dim : static_cast<int>(run + 0.5);
+        if (end < first[w]) end = first[w];
+        if (end > m->cfg.hidden_dim) end = m->cfg.hidden_dim;
+        first[w + 1] = end;
+        if (end - first[w] > *most) *most = end - first[w];
+    }
+    return first;
+}
 
 // parking: keep the last gate/up rows of most workgroups in LDS (short contexts); false: every row streams.
 Plan plan_for(const lpp_model* m, bool parking) {
@@ -2580,6 +2605,14 @@ Plan plan_for(const lpp_model* m, bool parking) {
                 slots = 2 * b.gu * b.ns_dim;
                 b.results_floats = (slots + 7) & ~7;
             }
+        }
+    }
+    {
+        int most = 0;
+        p.gu_first = gateup_table(m, b, p.grid, &most);
+        if (2 * most * b.ns_dim > slots) {
+            slots = 2 * most * b.ns_dim;
+            b.results_floats = (slots + 7) & ~7;
         }
     }
     p.lds_bytes = lds_floats() * sizeof(float);
@@ -2723,7 +2756,7 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
     };
     // gate/up rows of a workgroup that go through the streaming wavefronts: all but the parked ones at the block's end
     auto gu_streamed = [&](int wg) {
-        const int units = df::gu_units(b, hidden, wg);
+        const int units = df::gu_units(p.gu_first.data(), wg);
         return 2 * units - df::gu_parked_rows(b, wg, units);
     };
     int longest = 0;
@@ -2783,7 +2816,7 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
                 // local row 2u = gate row of hidden unit u, 2u + 1 = its up row
                 phase_rows(4 * l + df::kGGateUp, gu_streamed(wg), dim, [&](int r) {
                     return base((r & 1) ? LPP_T_W3 : LPP_T_W1) +
-                           (static_cast<size_t>(l) * hidden + df::gu_unit0(b, wg) + (r >> 1)) * rb_dim;
+                           (static_cast<size_t>(l) * hidden + df::gu_unit0(p.gu_first.data(), wg) + (r >> 1)) * rb_dim;
                 });
                 phase_rows(4 * l + df::kGDown, block_rows(dim, b.down, wg), hidden, [&](int r) {
                     return base(LPP_T_W2) + (static_cast<size_t>(l) * dim + wg * b.down + r) * rb_hidden;
@@ -2799,10 +2832,10 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
         }
     // Every column of every row must be multiplied exactly once per token: by a step, or as a parked row.
     for (int wg = 0; wg < p.grid; ++wg) {
-        const int units = df::gu_units(b, hidden, wg), parked = df::gu_parked_rows(b, wg, units);
+        const int units = df::gu_units(p.gu_first.data(), wg), parked = df::gu_parked_rows(b, wg, units);
         for (int l = 0; l < L; ++l)
             for (int r = 2 * units - parked; r < 2 * units; ++r)
-                covered[base((r & 1) ? LPP_T_W3 : LPP_T_W1) + (static_cast<size_t>(l) * hidden + df::gu_unit0(b, wg) + (r >> 1)) * rb_dim] += dim;
+                covered[base((r & 1) ? LPP_T_W3 : LPP_T_W1) + (static_cast<size_t>(l) * hidden + df::gu_unit0(p.gu_first.data(), wg) + (r >> 1)) * rb_dim] += dim;
     }
     {
         const struct { int tensor; size_t rows; int cols; } all[] = {
@@ -2826,7 +2859,13 @@ lpp_status build_step_lists(lpp_model* m, const Plan& p, int which) {
     }
     lpp_free(m->df_rows[which]);
     m->df_rows[which] = nullptr;
+    lpp_free(m->df_gu_first[which]);
+    m->df_gu_first[which] = nullptr;
     void* d = nullptr;
+    LPP_TRY(lpp_malloc(&d, p.gu_first.size() * sizeof(int)));
+    m->df_gu_first[which] = static_cast<int*>(d);
+    LPP_TRY(lpp_memcpy_h2d(d, p.gu_first.data(), p.gu_first.size() * sizeof(int)));
+    d = nullptr;
     LPP_TRY(lpp_malloc(&d, host.size() * sizeof(df::StepEntry)));
     m->df_rows[which] = d;
     m->df_row_stride[which] = stride;
@@ -2971,6 +3010,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     // (test hook: a ticket base one launch behind makes every workgroup's ticket look like one too many for its XCD)
     if (tagged.n_xcc > 1 && take_forced_ticket_failure()) tagged.ticket_base -= static_cast<unsigned>(m->persist_grid / tagged.n_xcc);
     LPP_REQUIRE(p.lds_bytes <= kLdsLimit, "persistent decode: %zu bytes of LDS per workgroup", p.lds_bytes);
+    tagged.gu_first = m->df_gu_first[which];
     if (xa.chunk > 0)
         hipLaunchKernelGGL((df::k_decode_dataflow<kF16, true>), dim3(m->persist_grid), dim3(df::kThreads), p.lds_bytes, s, a,
                            tagged, p.blocks, static_cast<const uint4*>(m->df_rows[which]), m->df_row_stride[which]);
@@ -3000,11 +3040,32 @@ lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc) {
         lpp_free(m->df_rows[i]);
         m->df_rows[i] = nullptr;
     }
+    if (df_xcc != m->df_xcc) {  // the weights are per XCD: a new numbering starts from even shares
+        m->df_gu_weight.clear();
+        m->df_calibrated = false;
+    }
     m->df_xcc = df_xcc;
     m->persist_grid = 0;
     m->df_ticket_base = 0;
     if (m->sync_words != nullptr) LPP_TRY(lpp_memset(m->sync_words + 96, 0, kMaxXcc * sizeof(unsigned)));
     return LPP_OK;
+}
+
+// The step lists alone (the partition of the hidden units changed): rebuilt at the next launch.
+lpp_status dataflow_forget_lists(lpp_model* m, hipStream_t s) {
+    LPP_HIP(hipStreamSynchronize(s));
+    for (int i = 0; i < 2; ++i) {
+        lpp_free(m->df_rows[i]);
+        m->df_rows[i] = nullptr;
+    }
+    return LPP_OK;
+}
+// Workgroups that hold the attention items of a short context (they own fewer hidden units and park no rows); the
+// XCDs the workgroups are numbered by (1: not numbered by XCD).
+void dataflow_partition_classes(const lpp_model* m, int* item_workgroups, int* n_xcc) {
+    const Plan p = plan_for(m, test_option(LPP_OPT_DECODE_PARKING) != 0);
+    *item_workgroups = p.blocks.gu_split;
+    *n_xcc = m->df_xcc > 1 ? m->df_xcc : 1;
 }
 
 // After a launch that left a code in StepParams::error (the stream is idle, the step record is as the launch found it:

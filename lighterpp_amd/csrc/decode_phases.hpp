@@ -869,6 +869,8 @@ lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s)
 unsigned dataflow_phases_per_token(int n_layers);
 unsigned dataflow_trace_marks();
 lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc);
+lpp_status dataflow_forget_lists(lpp_model* m, hipStream_t s);
+void dataflow_partition_classes(const lpp_model* m, int* item_workgroups, int* n_xcc);
 lpp_status dataflow_after_error(lpp_model* m, int code, bool* relaunch);
 
 }  // namespace lpp

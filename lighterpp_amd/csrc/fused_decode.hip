@@ -15,9 +15,13 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <vector>
 
 #include "decode_phases.hpp"
+
+// (defined with the timeline code at the end of the file)
+static lpp_status calibrate_gateup(lpp_model* m);
 
 namespace lpp {
 namespace {
@@ -349,6 +353,8 @@ lpp_status fused_release(lpp_model* m) {
     lpp_free(m->tagged);
     lpp_free(m->df_rows[0]);
     lpp_free(m->df_rows[1]);
+    lpp_free(m->df_gu_first[0]);
+    lpp_free(m->df_gu_first[1]);
     lpp_free(m->gen_uniforms);
     return LPP_OK;
 }
@@ -377,6 +383,7 @@ static lpp_status begin_run(lpp_model* m, const StepParams& init, hipStream_t s)
 lpp_status fused_forward(lpp_model* m, int token, int pos, float temperature, float penalty, const int* history,
                          int history_len, float r, int* next_token) {
     LPP_TRY(require_fused(m));
+    LPP_TRY(calibrate_gateup(m));
     hipStream_t s = stream();
     const bool use_history = penalty > 1.0f && history != nullptr && history_len > 0;
     if (use_history)
@@ -415,6 +422,7 @@ lpp_status fused_generate(lpp_model* m, int first_token, int start_pos, int n_st
                           int* out_tokens, lpp_gen_stats* stats) {
     LPP_TRY(require_fused(m));
     if (n_steps == 0) return LPP_OK;
+    LPP_TRY(calibrate_gateup(m));
     hipStream_t s = stream();
     LPP_TRY(ensure_gen_capacity(m, n_steps));
     StepParams sp{};
@@ -627,6 +635,7 @@ extern "C" lpp_status lpp_profile_kernels(lpp_model* m, int pos, int reps, lpp_k
         if (!m->w_loaded[t]) return fail(LPP_ERR_STATE, "weight tensor %d has not been uploaded", t);
     if (m->path == LPP_PATH_OPS) return ops_profile(m, pos, reps, out, capacity, count);
     if (!m->fused_ok) return fail(LPP_ERR_UNSUPPORTED, "fused path unavailable: %s", m->fused_why);
+    LPP_TRY(calibrate_gateup(m));
     StepParams sp{};
     sp.pos = pos;
     sp.temperature = 0.8f;
@@ -698,13 +707,121 @@ static lpp_status trace_impl(lpp_model* m, int pos, unsigned long long* out, int
     return LPP_OK;
 }
 
+// The gate/up phase moves two thirds of a layer's bytes and ends when its slowest workgroup publishes.  How fast
+// a workgroup gets through it depends on the XCD it runs on (the same XCDs finish late layer after layer, up to 2 us
+// of a 31 us phase at the 8B shape) and on whether it holds an attention item.  Before a model's first token on the
+// persistent path, two tokens are therefore traced at position 256 (a few hundred positions of context, whatever
+// the cache holds there: what a short run sees on average) and the hidden units dealt out anew: a class of
+// workgroups (those of one XCD that hold no attention item) that published d later than the median of a phase that
+// took T gets 1 - d / T of its share, and so does the rest of its XCD.  Results do not change (a hidden unit's value does not depend on who forms it); the cache rows the
+// traced tokens write at that position are put back.
+static lpp_status calibrate_gateup(lpp_model* m) {
+    using namespace lpp;
+    if (m->df_calibrated || m->path != LPP_PATH_PERSISTENT) return LPP_OK;
+    m->df_calibrated = true;
+    if (test_option(LPP_OPT_DECODE_CALIBRATE) == 0) return LPP_OK;
+    for (int t = 0; t < LPP_T_COUNT; ++t)
+        if (!m->w_loaded[t]) return LPP_OK;
+    const lpp_config& c = m->cfg;
+    const int L = c.n_layers, hs = m->head_size, rows = L * c.n_kv_heads;
+    if (L < 2) return LPP_OK;
+    hipStream_t s = stream();
+    // the traced position's row of every layer and KV head, as it is now
+    const int at_pos = c.seq_len > 256 ? 256 : c.seq_len - 1;
+    const size_t row_bytes = static_cast<size_t>(hs) * sizeof(uint16_t), pitch = static_cast<size_t>(c.seq_len) * row_bytes;
+    uint16_t* k_rows = m->key_cache + static_cast<size_t>(at_pos) * hs;
+    uint16_t* v_rows = m->value_cache + static_cast<size_t>(at_pos) * hs;
+    std::vector<uint16_t> keep_k(static_cast<size_t>(rows) * hs), keep_v(keep_k.size());
+    LPP_HIP(hipStreamSynchronize(s));
+    LPP_HIP(hipMemcpy2D(keep_k.data(), row_bytes, k_rows, pitch, row_bytes, rows, hipMemcpyDeviceToHost));
+    LPP_HIP(hipMemcpy2D(keep_v.data(), row_bytes, v_rows, pitch, row_bytes, rows, hipMemcpyDeviceToHost));
+    const int nwg = compute_units();
+    const int marks = static_cast<int>(dataflow_trace_marks());
+    const int n = marks * static_cast<int>(dataflow_phases_per_token(L));
+    std::vector<unsigned long long> t(static_cast<size_t>(n) * nwg);
+    lpp_status st = LPP_OK;
+    for (int pass = 0; pass < 2 && st == LPP_OK; ++pass) {
+        int count = 0, per_phase = 0, workgroups = 0;
+        st = trace_impl(m, at_pos, t.data(), static_cast<int>(t.size()), &count, &per_phase, &workgroups, true);
+        if (st != LPP_OK || workgroups != nwg) break;
+        int item_wgs = 0, n_xcc = 1;
+        dataflow_partition_classes(m, &item_wgs, &n_xcc);
+        if (n_xcc <= 1) break;  // (workgroups not numbered by XCD: nothing to tell them apart by)
+        if (m->df_gu_weight.size() != static_cast<size_t>(nwg)) m->df_gu_weight.assign(nwg, 1.0f);
+        const int classes = 2 * n_xcc;
+        std::vector<double> late(classes, 0.0);
+        std::vector<int> members(classes, 0);
+        double phase_time = 0.0;
+        int phases = 0;
+        std::vector<double> pub(nwg), len(nwg), sorted(nwg);
+        auto median = [&](const std::vector<double>& v) {
+            sorted = v;
+            std::nth_element(sorted.begin(), sorted.begin() + nwg / 2, sorted.end());
+            return sorted[nwg / 2];
+        };
+        bool complete = true;
+        for (int layer = 1; layer < L; ++layer) {
+            const size_t at = static_cast<size_t>(marks) * (5 * layer + 3);  // the gate/up phase of the layer
+            for (int w = 0; w < nwg; ++w) {
+                const unsigned long long staged = t[static_cast<size_t>(w) * n + at + 2], published = t[static_cast<size_t>(w) * n + at + 4];
+                complete = complete && staged != 0 && published >= staged;
+                pub[w] = static_cast<double>(published);
+                len[w] = static_cast<double>(published) - static_cast<double>(staged);
+            }
+            const double mid = median(pub);
+            phase_time += median(len);
+            ++phases;
+            for (int w = 0; w < nwg; ++w) {
+                const int cls = (w % n_xcc) + (w < item_wgs ? n_xcc : 0);
+                late[cls] += pub[w] - mid;
+                if (layer == 1) members[cls] += 1;
+            }
+        }
+        if (!complete || phases == 0 || phase_time <= 0.0) break;
+        phase_time /= phases;
+        // class means; the classes of the item holders are folded into one factor on top of their XCD's
+        std::vector<double> factor(classes, 1.0);
+        for (int k = 0; k < classes; ++k)
+            if (members[k] > 0) {
+                const double d = late[k] / (static_cast<double>(members[k]) * phases);
+                double f = 1.0 - d / phase_time;
+                f = f < 0.85 ? 0.85 : (f > 1.15 ? 1.15 : f);
+                factor[k] = f;
+            }
+        // (The workgroups that hold a short context's attention items publish early or late as a class too -- 1.6 us
+        // early at the TinyLlama shape -- but shifting units to or from them made every shape tried slower: their
+        // lead is spent on the next layer's items.  Only the XCDs' factors are applied.)
+        if (n_xcc > 1)
+            for (int w = 0; w < nwg; ++w) m->df_gu_weight[w] *= static_cast<float>(factor[w % n_xcc]);
+        st = dataflow_forget_lists(m, s);
+    }
+    LPP_HIP(hipStreamSynchronize(s));
+    LPP_HIP(hipMemcpy2D(k_rows, pitch, keep_k.data(), row_bytes, row_bytes, rows, hipMemcpyHostToDevice));
+    LPP_HIP(hipMemcpy2D(v_rows, pitch, keep_v.data(), row_bytes, row_bytes, rows, hipMemcpyHostToDevice));
+    return st;
+}
+
 extern "C" lpp_status lpp_trace_token(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count,
                                       int* marks_per_phase) {
+    if (m != nullptr && m->fused_ok) {  // (the timeline is that of the partition the decode loop runs with)
+        const int saved_path = m->path;
+        m->path = LPP_PATH_PERSISTENT;
+        const lpp_status st = calibrate_gateup(m);
+        m->path = saved_path;
+        LPP_TRY(st);
+    }
     return trace_impl(m, pos, out, capacity, count, marks_per_phase, nullptr, false);
 }
 
 extern "C" lpp_status lpp_trace_token_all(lpp_model* m, int pos, unsigned long long* out, int capacity, int* count,
                                           int* marks_per_phase, int* workgroups) {
     LPP_REQUIRE(workgroups != nullptr, "lpp_trace_token_all: null argument");
+    if (m != nullptr && m->fused_ok) {
+        const int saved_path = m->path;
+        m->path = LPP_PATH_PERSISTENT;
+        const lpp_status st = calibrate_gateup(m);
+        m->path = saved_path;
+        LPP_TRY(st);
+    }
     return trace_impl(m, pos, out, capacity, count, marks_per_phase, workgroups, true);
 }

@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <vector>
+
 #include "lpp_internal.hpp"
 
 // Everything forward() touches, resident in HBM.  Field names follow
@@ -57,6 +59,9 @@ struct lpp_model {
     void* df_rows[2] = {nullptr, nullptr};   // row lists of the persistent kernel's streaming wavefronts: [0] every row
     int df_row_stride[2] = {0, 0};           // streamed, [1] with parked gate/up rows left out (short contexts)
     const void* df_rows_key[12] = {};        // weight addresses the lists were built from
+    int* df_gu_first[2] = {nullptr, nullptr};  // device tables of the gate/up partition the lists were built for
+    std::vector<float> df_gu_weight;         // per workgroup: its share of the hidden units relative to an even deal
+    bool df_calibrated = false;              // a traced token has set df_gu_weight (or could not)
     // Host's own count of the step record for the persistent path: everything but the token id
     // is known before a launch and travels as kernel arguments.
     int df_pos = 0, df_history_len = 0, df_history_cap = 0, df_step_index = 0, df_freeze = 0;

@@ -34,7 +34,7 @@ struct RopeTable {
 std::map<std::tuple<int, int, uint32_t>, RopeTable> g_rope;  // key: device, head_size, base bits
 
 // Test hooks (lpp_set_test_option): which of its alternatives the library may pick by itself.
-int g_test_options[LPP_OPT_COUNT] = {1, 1, 1, 1, 0, 1, 1, 1, 1, 1};
+int g_test_options[LPP_OPT_COUNT] = {1, 1, 1, 1, 0, 1, 1, 1, 1, 1, 1};
 unsigned g_test_epoch = 1;  // advanced by every change a model has to act on
 
 }  // namespace

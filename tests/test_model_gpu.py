@@ -338,6 +338,36 @@ def test_persistent_alternatives_the_library_selects_by_itself(variant, test_opt
     o.close()
 
 
+def test_gateup_partition_weighted_by_xcd_changes_no_bit(test_options):
+    """Before its first token a model on the persistent path traces two tokens and deals the hidden units out by how
+    fast each XCD got through the gate/up phase.  Who forms a hidden unit does not change its value, and the cache row
+    the traced tokens wrote is put back: a model set up with the hook off (even shares) gives the same logits and
+    cache, bit for bit, from a cache pre-filled up to the traced position and beyond."""
+    shape = Shape(2048, 4096, 3, 32, 8, 500, 640, 500000.0, fp16=True, tied=True)  # (the trace needs layers to average over)
+    runs = []
+    fill = capi.synth_normal_f16(shape.n_layers * shape.n_kv_heads * shape.seq_len * shape.head_size, 801, 1.0)
+    for calibrate in (1, 0):
+        test_options(capi.OPT_DECODE_CALIBRATE, calibrate)
+        m = Model(shape)
+        m.load_synthetic(41)
+        m.set_path(capi.PATH_PERSISTENT)
+        m.write_buffer(capi.B_KEY_CACHE, fill)
+        m.write_buffer(capi.B_VALUE_CACHE, fill[::-1].copy())
+        out, tok = [], 5
+        for pos in range(300, 304):
+            tok = m.forward(tok, pos, 0.0)
+            out.append(m.buffer(capi.B_LOGITS).view(np.uint32).copy())
+        runs.append((out, m.buffer(capi.B_KEY_CACHE).copy(), m.buffer(capi.B_VALUE_CACHE).copy()))
+        m.close()
+    (la, ka, va), (lb, kb, vb) = runs
+    assert all(np.array_equal(x, y) for x, y in zip(la, lb))
+    assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+    # the traced position's rows are the pre-filled ones again (positions 300..303 alone were written)
+    k = ka.reshape(shape.n_layers, shape.n_kv_heads, shape.seq_len, shape.head_size)
+    want = fill.reshape(k.shape)
+    assert np.array_equal(k[:, :, :300, :], want[:, :, :300, :]) and np.array_equal(k[:, :, 304:, :], want[:, :, 304:, :])
+
+
 def test_persistent_relaunches_a_token_when_an_xcd_is_dealt_unevenly(test_options):
     """A launch in which an XCD draws more tickets than its share ends with every workgroup leaving the kernel
     normally and no token delivered; the library switches the per-XCD hand-overs off and launches the same token
