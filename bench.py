@@ -166,6 +166,8 @@ def bench_prefill(args, model, shape, name, cus) -> int:
         print("bench.py: the batched prefill does not take this model", file=sys.stderr)
         return 2
     ids = capi.synth_token_ids(n, SEED + 1, shape.vocab_size)
+    fast = args.prefill_mode == "fast"
+    model.set_prefill_mode(capi.PREFILL_FAST if fast else capi.PREFILL_EXACT)
     reps = args.steps if args.steps is not None else 30
     for _ in range(max(args.warmup if args.warmup != 16 else 3, 1)):
         model.prefill(ids, 0)
@@ -183,13 +185,15 @@ def bench_prefill(args, model, shape, name, cus) -> int:
     tflops = (gemm_flops + att_flops) / sec / 1e12
     out = dict(metric="batched prefill, prompt ids/s, " + args.config, value=round(n / sec, 1), unit="tok/s", n_gpus=1,
                steps=reps, warmup=max(args.warmup if args.warmup != 16 else 3, 1), ms_per_step=round(sec * 1e3, 3), higher_is_better=True, scaling="weak",
-               vs_baseline=None, dtype="f32 accumulate over f16 weights, activations split hi+lo", data="synthetic",
-               config=dict(workload=args.config, prompt_ids=n, chunk=512),
+               vs_baseline=None,
+               dtype="f32 accumulate over f16 weights, activations rounded to f16 at each GEMM input" if fast
+               else "f32 accumulate over f16 weights, activations split hi+lo", data="synthetic",
+               config=dict(workload=args.config, prompt_ids=n, chunk=512, prefill_mode=args.prefill_mode),
                roofline=dict(bound="mfma", achieved=round(tflops, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
                              frac=round(tflops / MFMA_F16_PEAK_TFLOPS, 4), traffic=None,
                              note="algorithmic flops of what the cache depends on (the last layer stops at its K/V "
-                                  "rows); each product counted once: the kernel issues two MFMAs per product, for "
-                                  "the activation's head and remainder"),
+                                  "rows); each product counted once" + ("" if fast else ": the kernel issues two MFMAs "
+                                  "per product, for the activation's head and remainder")),
                cpu_baseline=None,
                device=dict(name=name.value.decode(), compute_units=cus.value))
     print(json.dumps(out))
@@ -207,6 +211,8 @@ def main() -> int:
     ap.add_argument("--parity-steps", type=int, default=3)
     ap.add_argument("--profile-reps", type=int, default=20)
     ap.add_argument("--no-timeline", action="store_true", help="skip the traced token behind the `timeline` object")
+    ap.add_argument("--prefill-mode", default="exact", choices=["exact", "fast"],
+                    help="with --prefill: activations as binary16 head + remainder (exact) or the head alone (fast)")
     ap.add_argument("--prefill", type=int, default=0, metavar="N",
                     help="time the batched prefill of N prompt ids instead of the decode loop (a second, separate line)")
     args = ap.parse_args()

@@ -365,6 +365,14 @@ lpp_status lpp_run(lpp_model *m, const int *prompt, int n_prompt, int steps, flo
  * (LPP_ERR_UNSUPPORTED and the reason in lpp_last_error otherwise).  `tokens` is host
  * memory.  Synchronous. */
 lpp_status lpp_prefill_supported(const lpp_model *m);
+/* What a prefill GEMM takes as its input.  LPP_PREFILL_EXACT (default): the fp32 activations as a binary16 head plus a
+ * binary16 remainder, two matrix-core products per weight tile: every cache entry lands within one binary16 step of
+ * what prefill-by-decode writes.  LPP_PREFILL_FAST: the head alone -- the activations rounded to binary16 where a
+ * GEMM reads them, which is what the reference's own GPU GEMV does to x (matmul.cu:85-98), accumulation still fp32:
+ * a quarter fewer matrix-core cycles and a third fewer bytes through LDS; the steps that follow stay inside the
+ * logits bar of 2e-3 against the CPU path, cache entries drift by a few binary16 steps over the layers. */
+enum { LPP_PREFILL_EXACT = 0, LPP_PREFILL_FAST = 1 };
+lpp_status lpp_model_set_prefill_mode(lpp_model *m, int mode);
 lpp_status lpp_prefill(lpp_model *m, const int *tokens, int n_tokens, int start_pos);
 /* lpp_run with the prompt (all ids but the last) prefilled by lpp_prefill instead of
  * by decode steps; everything else, the uniforms' indexing by position included, as

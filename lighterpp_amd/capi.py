@@ -34,6 +34,7 @@ TENSOR_NAMES = ["token_embedding", "rms_att", "wq", "wk", "wv", "wo", "rms_ffn",
 
 PATH_OPS, PATH_FUSED, PATH_PERSISTENT = 0, 1, 2
 GGML_F32, GGML_F16 = 0, 1
+PREFILL_EXACT, PREFILL_FAST = 0, 1
 # enum lpp_test_option
 (OPT_DECODE_XCD_HANDOVERS, OPT_DECODE_XCD_QKV, OPT_DECODE_PARKING, OPT_DECODE_LANE_ITEM, OPT_DECODE_FAIL_TICKETS,
  OPT_DECODE_XCD_ATTENTION, OPT_PREFILL_STAGED_GEMM, OPT_PREFILL_WIDE_TILES, OPT_PREFILL_FUSED_FFN,
@@ -119,6 +120,7 @@ SIGNATURES = {
     "lpp_run": (_i, [_vp, _vp, _i, _i, _f, _f, _vp, _vp, _i, C.POINTER(LppRunResult)]),
     "lpp_run_batched_prefill": (_i, [_vp, _vp, _i, _i, _f, _f, _vp, _vp, _i, C.POINTER(LppRunResult)]),
     "lpp_prefill_supported": (_i, [_vp]),
+    "lpp_model_set_prefill_mode": (_i, [_vp, _i]),
     "lpp_prefill": (_i, [_vp, _vp, _i, _i]),
     "lpp_prefill_gemm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "lpp_prefill_gemm_noalloc": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),

@@ -81,6 +81,7 @@ struct lpp_model {
 
     void* pf_buf[12] = {};                   // batched prefill: activations of a chunk of tokens (prefill.hip)
     int pf_cap = 0;                          // tokens those buffers hold
+    int pf_mode = 0;                         // LPP_PREFILL_EXACT / LPP_PREFILL_FAST
 
     hipGraphExec_t graph_exec[2] = {nullptr, nullptr};  // [0] without, [1] with uniforms/out arrays
     hipEvent_t ev_a = nullptr, ev_b = nullptr;

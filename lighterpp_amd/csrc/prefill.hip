@@ -382,10 +382,11 @@ struct PipeJob {
 
 constexpr int kPipeTripK = 64;  // columns per trip of the narrow tiles; K must be a multiple
 
-template <int kFi, int kTj, int kTripK>
+// (kLo: the activations' remainder tile travels and is multiplied too; without it a stage is a third smaller)
+template <int kFi, int kTj, int kTripK, bool kLo = true>
 struct PipeShape {
     static constexpr int kRowBytes = 2 * kTripK;
-    static constexpr int kRowsA = 64 * kFi, kRowsB = 64 * kTj, kRows = kRowsA + 2 * kRowsB;
+    static constexpr int kRowsA = 64 * kFi, kRowsB = 64 * kTj, kRows = kRowsA + (kLo ? 2 : 1) * kRowsB;
     static constexpr int kStageBytes = kRows * kRowBytes;
     static constexpr int kStages = (160 * 1024) / kStageBytes > 5 ? 5 : (160 * 1024) / kStageBytes;
     static constexpr int kLoads = kStageBytes / 4096;  // requests of 1 KiB per wavefront and stage
@@ -411,9 +412,9 @@ __device__ __forceinline__ void swiglu_split4(half4_pf_t& hi, half4_pf_t& lo, co
     }
 }
 
-template <int kFi, int kTj, int kMode, int kTripK>
+template <int kFi, int kTj, int kMode, int kTripK, bool kLo>
 __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
-    typedef PipeShape<kFi, kTj, kTripK> Shape;
+    typedef PipeShape<kFi, kTj, kTripK, kLo> Shape;
     constexpr int kRowsA = Shape::kRowsA, kRowsB = Shape::kRowsB, kStages = Shape::kStages, kLoads = Shape::kLoads;
     constexpr int kStageBytes = Shape::kStageBytes, kRowBytes = Shape::kRowBytes;
     constexpr int kSteps = kTripK / 16;      // k-steps per trip
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
             } else {
                 from = w + static_cast<size_t>(f_base + row) * K;
             }
-        } else if (row < kRowsA + kRowsB) {
+        } else if (!kLo || row < kRowsA + kRowsB) {
             from = job.xh + static_cast<size_t>(t_base + row - kRowsA) * K;
         } else {
             from = job.xl + static_cast<size_t>(t_base + row - kRowsA - kRowsB) * K;
@@ -501,7 +502,7 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
 #pragma unroll
         for (int j = 0; j < kTj; ++j) {
             f.bh[j] = *reinterpret_cast<const half8_t*>(stage + b_off[s] + j * 32 * kRowBytes);
-            f.bl[j] = *reinterpret_cast<const half8_t*>(stage + b_off[s] + (kRowsB + j * 32) * kRowBytes);
+            if constexpr (kLo) f.bl[j] = *reinterpret_cast<const half8_t*>(stage + b_off[s] + (kRowsB + j * 32) * kRowBytes);
         }
     };
     // (one half of a k-step's MFMAs: the weight tiles [kFi / 2 * half, kFi / 2 * (half + 1)))
@@ -511,7 +512,7 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
 #pragma unroll
             for (int j = 0; j < kTj; ++j) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[i], f.bh[j], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[i], f.bl[j], acc[i][j], 0, 0, 0);
+                if constexpr (kLo) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[i], f.bl[j], acc[i][j], 0, 0, 0);
             }
     };
     // (requesting wavefronts) wait until the requests of `trip` have landed: those of later trips, at
@@ -1042,27 +1043,32 @@ struct Product {
 };
 
 // The kernel's LDS need, told to the runtime once per device (the attribute belongs to the device's copy of the kernel).
-template <int kFi, int kTj, int kMode, int kTripK>
+template <int kFi, int kTj, int kMode, int kTripK, bool kLo = true>
 lpp_status size_pipe() {
     static bool sized[64] = {};
     int device = 0;
     LPP_HIP(hipGetDevice(&device));
     if (device < 0 || device >= 64 || !sized[device]) {
-        LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, pf::PipeShape<kFi, kTj, kTripK>::kLdsBytes));
+        LPP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&pf::k_gemm_pipe<kFi, kTj, kMode, kTripK, kLo>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, pf::PipeShape<kFi, kTj, kTripK, kLo>::kLdsBytes));
         if (device >= 0 && device < 64) sized[device] = true;
     }
     return LPP_OK;
 }
 
-template <int kFi, int kTj, int kMode, int kTripK = pf::kPipeTripK>
-lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
-    typedef pf::PipeShape<kFi, kTj, kTripK> Shape;
-    LPP_TRY((size_pipe<kFi, kTj, kMode, kTripK>()));
+template <int kFi, int kTj, int kMode, int kTripK, bool kLo>
+lpp_status launch_pipe_as(const pf::PipeJob& job, hipStream_t s) {
+    typedef pf::PipeShape<kFi, kTj, kTripK, kLo> Shape;
+    LPP_TRY((size_pipe<kFi, kTj, kMode, kTripK, kLo>()));
     const int per_die = (job.groups + 7) / 8;
-    hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode, kTripK>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
+    hipLaunchKernelGGL((pf::k_gemm_pipe<kFi, kTj, kMode, kTripK, kLo>), dim3(per_die * 8 * job.token_tiles), dim3(512), Shape::kLdsBytes, s, job);
     LPP_CHECK_LAUNCH("k_gemm_pipe");
     return LPP_OK;
+}
+// (a job without a remainder array takes the kernels that neither fetch nor multiply one)
+template <int kFi, int kTj, int kMode, int kTripK = pf::kPipeTripK>
+lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
+    return job.xl != nullptr ? launch_pipe_as<kFi, kTj, kMode, kTripK, true>(job, s) : launch_pipe_as<kFi, kTj, kMode, kTripK, false>(job, s);
 }
 
 // `partials` (optional, partial_floats long): room for the partial products of a split K.  A product
@@ -1072,7 +1078,8 @@ lpp_status launch_pipe(const pf::PipeJob& job, hipStream_t s) {
 // ranges itself (in order, in the kernel that reads the product next) and gets their number there;
 // without it they are added to y here, in order.
 lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad, bool accumulate,
-                hipStream_t s, float* partials = nullptr, size_t partial_floats = 0, int* left_split = nullptr) {
+                hipStream_t s, float* partials = nullptr, size_t partial_floats = 0, int* left_split = nullptr,
+                bool remainder = true) {
     LPP_REQUIRE(count >= 1 && count <= 3 && t_pad % pf::kTileTokens == 0 && K % 32 == 0, "prefill GEMM: %d products, K %d, T %d",
                 count, K, t_pad);
     if (left_split != nullptr) *left_split = 1;
@@ -1111,7 +1118,7 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
             }
         }
         job.xh = xh;
-        job.xl = xl;
+        job.xl = remainder ? xl : nullptr;  // (without: the kernels that neither fetch nor multiply the remainder)
         job.K = K;
         job.k_len = K / splits;
         job.split_stride = stride;
@@ -1190,7 +1197,7 @@ lpp_status norm_split(float* x, const float* gain, pf::half_t* hi, pf::half_t* l
 // (hi, lo)[t][u] = SwiGLU(W1 x[t], W3 x[t])[u] in one launch: the gate and the up projection of a
 // feature share a workgroup, and the activation is applied to the accumulators.
 lpp_status gate_up_swiglu(const void* w1, const void* w3, int hidden, const pf::half_t* xh, const pf::half_t* xl, int K, int t_pad,
-                          pf::half_t* out_hi, pf::half_t* out_lo, hipStream_t s) {
+                          pf::half_t* out_hi, pf::half_t* out_lo, hipStream_t s, bool remainder) {
     pf::PipeJob job = {};
     job.w[0] = static_cast<const pf::half_t*>(w1);
     job.w[1] = static_cast<const pf::half_t*>(w3);
@@ -1198,7 +1205,7 @@ lpp_status gate_up_swiglu(const void* w1, const void* w3, int hidden, const pf::
     job.first_tile[0] = 0;
     job.first_tile[1] = job.first_tile[2] = 0x7fffffff;
     job.xh = xh;
-    job.xl = xl;
+    job.xl = remainder ? xl : nullptr;
     job.K = K;
     job.k_len = K;
     job.feature_tiles = hidden / 128;  // 128 features a tile: 128 rows of W1 and the same 128 of W3
@@ -1239,6 +1246,10 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
     // The fp32 gate and up buffers double as room for the partial products of the GEMMs whose K is
     // split (each is t_pad * hidden floats): up for Wq/Wk/Wv, gate for Wo and then for W2.
     const size_t room = static_cast<size_t>(t_pad) * hidden;
+    // LPP_PREFILL_EXACT: every product takes the activations as binary16 head + remainder.  LPP_PREFILL_FAST: the head
+    // alone, in the staged kernels (what a GEMM sees of its input is then what the reference's own GPU GEMV sees,
+    // matmul.cu:85-98; accumulation stays fp32).
+    const bool exact = m->pf_mode != LPP_PREFILL_FAST;
     const bool fused_ffn = dim % pf::kPipeTripK == 0 && hidden % 128 == 0 && test_option(LPP_OPT_PREFILL_STAGED_GEMM) != 0 &&
                            test_option(LPP_OPT_PREFILL_FUSED_FFN) != 0;
     int pending = 0;  // ranges of the product before (W2's, then Wo's) still to be added to x
@@ -1253,7 +1264,7 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
                                 {layer_of(LPP_T_WV, l, kv, dim), v, kv}};
         const int q_dim = last_layer ? 0 : dim;
         int qkv_split = 1;
-        LPP_TRY(gemm(qkv + (last_layer ? 1 : 0), last_layer ? 2 : 3, hi, lo, dim, t_pad, false, s, up, room, &qkv_split));
+        LPP_TRY(gemm(qkv + (last_layer ? 1 : 0), last_layer ? 2 : 3, hi, lo, dim, t_pad, false, s, up, room, &qkv_split, exact));
         const size_t qkv_stride = static_cast<size_t>(t_pad) * (q_dim + 2 * kv);
         const float* qs = qkv_split > 1 ? up : q;
         const float* ks = qkv_split > 1 ? up + static_cast<size_t>(t_pad) * q_dim : k;
@@ -1282,21 +1293,21 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
                                m->value_cache, hi, lo, l, pos0, dim, kv, hs, m->gqa, c.seq_len, n);
         LPP_CHECK_LAUNCH("k_attention");
         const Product wo = {layer_of(LPP_T_WO, l, dim, dim), x, dim};
-        LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s, gate, room, &pending));
+        LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s, gate, room, &pending, exact));
         // feed-forward block, model.cpp:221-226
         LPP_TRY(norm_split(x, static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, t_pad, gate,
                            pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s));
         if (fused_ffn) {
             LPP_TRY(gate_up_swiglu(layer_of(LPP_T_W1, l, hidden, dim), layer_of(LPP_T_W3, l, hidden, dim), hidden, hi, lo, dim, t_pad,
-                                   hi2, lo2, s));
+                                   hi2, lo2, s, exact));
         } else {
             const Product gate_up[2] = {{layer_of(LPP_T_W1, l, hidden, dim), gate, hidden}, {layer_of(LPP_T_W3, l, hidden, dim), up, hidden}};
-            LPP_TRY(gemm(gate_up, 2, hi, lo, dim, t_pad, false, s));
+            LPP_TRY(gemm(gate_up, 2, hi, lo, dim, t_pad, false, s, nullptr, 0, nullptr, exact));
             hipLaunchKernelGGL(pf::k_swiglu_split, dim3((hidden + 255) / 256, t_pad), dim3(256), 0, s, gate, up, hi2, lo2, hidden, n);
             LPP_CHECK_LAUNCH("k_swiglu_split");
         }
         const Product w2 = {layer_of(LPP_T_W2, l, dim, hidden), x, dim};
-        LPP_TRY(gemm(&w2, 1, hi2, lo2, hidden, t_pad, true, s, gate, room, &pending));
+        LPP_TRY(gemm(&w2, 1, hi2, lo2, hidden, t_pad, true, s, gate, room, &pending, exact));
     }
     LPP_HIP(hipStreamSynchronize(s));
     return LPP_OK;
@@ -1315,6 +1326,12 @@ void prefill_release(lpp_model* m) {
 }  // namespace lpp
 
 extern "C" {
+
+lpp_status lpp_model_set_prefill_mode(lpp_model* m, int mode) {
+    LPP_REQUIRE(m != nullptr && (mode == LPP_PREFILL_EXACT || mode == LPP_PREFILL_FAST), "lpp_model_set_prefill_mode: mode %d", mode);
+    m->pf_mode = mode;
+    return LPP_OK;
+}
 
 lpp_status lpp_prefill_supported(const lpp_model* m) {
     LPP_REQUIRE(m != nullptr, "lpp_prefill_supported: null model");

@@ -345,6 +345,10 @@ class Model:
         """Whether lpp_prefill (batched prefill on the matrix cores) takes this model."""
         return self.lib.lpp_prefill_supported(self.handle) == capi.LPP_OK
 
+    def set_prefill_mode(self, mode: int) -> None:
+        """capi.PREFILL_EXACT (binary16 head + remainder of the activations) or capi.PREFILL_FAST (head alone)."""
+        capi.check(self.lib.lpp_model_set_prefill_mode(self.handle, mode))
+
     def prefill(self, tokens, start_pos: int = 0) -> None:
         """lpp_prefill: the KV cache entries of `tokens` at positions start_pos.., all layers, in one batch."""
         t = np.ascontiguousarray(tokens, dtype=np.int32)

@@ -204,6 +204,79 @@ def test_run_with_batched_prefill_matches_run(temperature):
     m.close()
 
 
+@pytest.mark.parametrize("name", list(SHAPES))
+def test_fast_prefill_stays_inside_the_logits_bar(name):
+    """LPP_PREFILL_FAST: every GEMM of the prefill sees its input rounded to binary16 (the head of the activation
+    alone, no remainder product), accumulation in fp32.  The contract that is left is the decode loop's own: the
+    steps after the prompt within 2e-3 of the CPU path's logits and the same greedy ids; cache entries may sit a few
+    binary16 steps from the oracle's (bounded here at 2^-6 of the largest entry)."""
+    shape = SHAPES[name]
+    b = Model(shape)
+    w = b.load_synthetic(7, keep=True)
+    o = ob.OracleModel(shape, w, fp16=True, kv_round_f16=True)
+    b.set_path(capi.PATH_PERSISTENT)
+    b.set_prefill_mode(capi.PREFILL_FAST)
+    n = 37
+    prompt = capi.synth_token_ids(n, 11, shape.vocab_size)
+    b.prefill(prompt, 0)
+    for i, tok in enumerate(prompt):
+        o.forward_logits(int(tok), i)
+    kb, vb, _, _ = caches(b, shape, n)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    for got, name_ in ((kb, "key_cache"), (vb, "value_cache")):
+        want = o.buf(name_).reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :]
+        assert np.max(np.abs(got - want)) <= 2.0 ** -6 * np.abs(want).max()
+    tok, worst, agree, steps = int(prompt[-1]), 0.0, 0, 24
+    for pos in range(n, n + steps):
+        nxt = b.forward(tok, pos, 0.0)
+        want = o.forward_logits(tok, pos)
+        worst = max(worst, rel_err(b.buffer(capi.B_LOGITS), want))
+        agree += int(nxt == int(np.argmax(want)))
+        tok = int(np.argmax(want))
+    assert worst <= LOGIT_TOL, f"max relative logit error after a fast prefill {worst}"
+    assert agree >= steps - 1
+    b.close()
+    o.close()
+
+
+def test_prefill_at_full_size_against_the_oracle():
+    """The 1B shape straight against the CPU oracle (no decode run in between): 24 prompt ids prefilled in either
+    mode, then 4 decode steps -- cache entries of all 16 layers and the steps' logits and greedy ids."""
+    shape = CONFIGS["c3_llama32_1b_fp16"]
+    b = Model(shape)
+    w = b.load_synthetic(3, keep=True)
+    o = ob.OracleModel(shape, w, fp16=True, kv_round_f16=True)
+    b.set_path(capi.PATH_PERSISTENT)
+    n, steps = 24, 4
+    prompt = capi.synth_token_ids(n, 9, shape.vocab_size)
+    for i, tok in enumerate(prompt):
+        print(f"oracle prompt position {i}", flush=True)
+        o.forward_logits(int(tok), i)
+    hs, nkv, L = shape.head_size, shape.n_kv_heads, shape.n_layers
+    want_k = o.buf("key_cache").reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :].copy()
+    want_v = o.buf("value_cache").reshape(L, nkv, shape.seq_len, hs)[:, :, :n, :].copy()
+    wants, tok = [], int(prompt[-1])
+    for pos in range(n, n + steps):
+        wants.append(o.forward_logits(tok, pos))
+        tok = int(np.argmax(wants[-1]))
+    o.close()
+    for mode, cache_bar in ((capi.PREFILL_EXACT, 2.0 ** -9), (capi.PREFILL_FAST, 2.0 ** -6)):
+        b.reset()
+        b.set_prefill_mode(mode)
+        b.prefill(prompt, 0)
+        kb, vb, _, _ = caches(b, shape, n)
+        for got, want in ((kb, want_k), (vb, want_v)):
+            scale = np.abs(want).max()
+            assert np.all(np.abs(got - want) <= np.maximum(np.abs(want) * cache_bar, scale * cache_bar / 4)), (mode, np.max(np.abs(got - want)), scale)
+        tok = int(prompt[-1])
+        for pos, want in zip(range(n, n + steps), wants):
+            nxt = b.forward(tok, pos, 0.0)
+            assert rel_err(b.buffer(capi.B_LOGITS), want) <= LOGIT_TOL, (mode, pos)
+            assert nxt == int(np.argmax(want)), (mode, pos)
+            tok = nxt
+    b.close()
+
+
 @pytest.mark.parametrize("config,n", [("c3_llama32_1b_fp16", 300), ("c2_tinyllama_1b_fp16", 200), ("c5_llama3_8b_fp16", 140)])
 def test_prefill_at_full_size_against_decode(config, n):
     """The benchmark shapes (1B: 300 prompt ids; TinyLlama: 44 feature tiles of the fused gate/up launch, not a
