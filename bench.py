@@ -43,10 +43,14 @@ HBM_PEAK_GBS = 8000.0
 # the kernel's source file when the two counter runs were made).  Hardware counters cannot be read in-process, so
 # the figure is a constant; it is quoted only while the kernel's source is the one that was measured, and is null
 # (with a note) from the moment the file changes until the two runs are repeated
-# (profiles/persistent_decode_c3_llama32_1b_pmc_hbm_traffic.txt gives the commands).
+# (profiles/persistent_decode_<workload>_pmc_hbm_traffic.txt give the commands, one file per configuration).
 KERNEL_SOURCES = {"k_decode_dataflow": ROOT / "lighterpp_amd" / "csrc" / "dataflow_decode.hip"}
+_MEASURED_SOURCE = "6ec79e5b081d39f11103ba536d70baf5987ac251ae91b677d1f3661a01f3f601"
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    ("c3_llama32_1b_fp16", "k_decode_dataflow"): (2.5132e9, "41546cc7fdb11b399048d99761b05c1972f0491d54f14515337f71cce6592be8"),
+    ("c2_tinyllama_1b_fp16", "k_decode_dataflow"): (2.1265e9, _MEASURED_SOURCE),
+    ("c3_llama32_1b_fp16", "k_decode_dataflow"): (2.5143e9, _MEASURED_SOURCE),
+    ("c4_llama32_1b_longctx_fp16", "k_decode_dataflow"): (2.8024e9, _MEASURED_SOURCE),
+    ("c5_llama3_8b_fp16", "k_decode_dataflow"): (1.5185e10, _MEASURED_SOURCE),
 }
 
 
