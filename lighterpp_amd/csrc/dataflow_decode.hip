@@ -161,7 +161,8 @@ struct Blocks {
     int qkv_by_xcc; // > 0: the stacked [Wq; Wk; Wv] rows are dealt out per XCD, this many KV heads (with their query heads) to each
     int xa_cu_shift;  // att_xcd_item: log2 of the workgroups that share a KV head
     int xa_opc;       // att_xcd_item: attention outputs each of them combines
-    int kv_floats;    // LDS for the K and V rows of a workgroup's share of a context
+    int kv_floats;    // LDS for the K and V rows of a workgroup's share of a context, where they have an area of their own
+    int kv_offset;    // where those rows start, in floats from the start of LDS (their own area, or inside xs: see plan_for)
     int slice_dim;  // columns per slice of a dim-column row (slice_width)
     int down;   // rows of W2
     int cls;    // rows of the classifier
@@ -2129,6 +2130,10 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
             else if (a.gqa == 2) att_xcd_item<128, 2>(c, io, l, layer);
             else att_xcd_item<128, 1>(c, io, l, layer);
         }
+        // (after the item, through registers.  Requested straight into LDS as soon as the item's inputs are in, the
+        // rows would travel while the scores are formed -- but such a request holds its wavefront until the memory
+        // pipeline has taken it, a microsecond or two for a wavefront's rows, and that is on the item's path: 677 us
+        // per token against 649 at the 1B shape and 600 positions.)
         park_fetch(c, io, l, layer);
         mark(c, io, 4);
         ++c.phase_index;
@@ -2451,7 +2456,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.red = l.qkv + (kMaxAttHeads + 2) * kMaxHeadPad;
     l.gather = l.red + b.red_floats;
     l.park = l.gather + b.gather_floats;
-    l.kv = l.park + b.park_floats;
+    l.kv = lds + b.kv_offset;
     // (the LDS address is taken from the array itself, where the address space is plain to the compiler, and the
     // area's offset added as a number: a pointer that has been through a structure is not reliably traced back)
     l.kv_lds = static_cast<unsigned>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds)) +
@@ -2530,8 +2535,43 @@ std::vector<int> gateup_table(const lpp_model* m, const df::Blocks& b, int grid,
     return first;
 }
 
+constexpr int kMaxXcc = 8;
+constexpr int kMaxPerXcc = 32;  // workgroups of one XCD the XCD-wide attention split is laid out for
+
+// The split of a KV head's context over the workgroups of its XCD (att_xcd_item) at npos positions, for a plan whose
+// Wq/Wk/Wv rows are dealt out per XCD; chunk 0 where it does not apply.
+struct XcdAttention {
+    int chunk, active, ppw, cu_shift, opc, kv_floats;
+};
+XcdAttention xcd_attention_for(const lpp_model* m, const df::Blocks& b, int grid, int npos) {
+    XcdAttention x = {};
+    if (test_option(LPP_OPT_DECODE_XCD_ATTENTION) == 0 || b.qkv_by_xcc <= 0 || m->df_xcc <= 1) return x;
+    const int hs = m->head_size, g = m->gqa;
+    if ((hs != 64 && hs != 128) || (g != 1 && g != 2 && g != 4)) return x;
+    const int per_xcc = grid / m->df_xcc;
+    if (per_xcc > kMaxPerXcc || per_xcc % b.qkv_by_xcc != 0) return x;
+    const int n_cu = per_xcc / b.qkv_by_xcc;  // workgroups that share a KV head
+    if ((n_cu & (n_cu - 1)) != 0 || (g * hs) % n_cu != 0) return x;
+    const int opc = g * hs / n_cu;            // outputs each of them combines: all of one head, at most 16
+    if (opc > hs || hs % opc != 0 || opc > df::kMaxHeadPad / 8) return x;
+    const int chunk = ((npos + n_cu - 1) / n_cu + 7) & ~7;
+    if (chunk > df::kIoWaves * df::kWave) return x;
+    while ((1 << x.cu_shift) < n_cu) ++x.cu_shift;
+    x.chunk = chunk;
+    x.active = (npos + chunk - 1) / chunk;
+    x.ppw = chunk / df::kIoWaves;
+    x.opc = opc;
+    x.kv_floats = chunk * hs;  // eight wavefronts x ppw positions x (K row + V row) of binary16
+    return x;
+}
+
 // parking: keep the last gate/up rows of most workgroups in LDS (short contexts); false: every row streams.
-Plan plan_for(const lpp_model* m, bool parking) {
+// xa (chunk > 0): the plan of att_xcd_item -- every workgroup holds a share of a KV head's context, with room for
+// four heads in the merge areas.  Where the share's rows fit the part of xs that only the down phase uses (beyond
+// the first dim floats: between two down phases nothing else is staged there), they live there and every workgroup
+// parks gate/up rows in what LDS is left; where they do not, they get an area of their own and nothing is parked.
+// Either way the rows parked do not depend on the position, so a growing context keeps its step lists.
+Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr) {
     const lpp_config& c = m->cfg;
     Plan p;
     p.grid = compute_units();
@@ -2573,6 +2613,18 @@ Plan plan_for(const lpp_model* m, bool parking) {
     b.xa_cu_shift = 0;
     b.xa_opc = 0;
     b.kv_floats = 0;
+    b.kv_offset = 0;
+    const bool xcd = xa != nullptr && xa->chunk > 0;
+    bool kv_in_xs = false;
+    if (xcd) {
+        b.red_floats = df::kIoWaves * df::kMaxAttHeads * df::kRedStride;
+        if (df::kMaxAttHeads * df::kIoWaves * df::kWave > b.gather_floats) b.gather_floats = df::kMaxAttHeads * df::kIoWaves * df::kWave;
+        b.xa_cu_shift = xa->cu_shift;
+        b.xa_opc = xa->opc;
+        kv_in_xs = xa->kv_floats <= b.xs_floats - dim_pad;
+        if (kv_in_xs) b.kv_offset = 2 * dim_pad;  // xraw, then the first dim floats of xs
+        else b.kv_floats = xa->kv_floats;
+    }
     b.slice_dim = df::slice_width(c.dim, chunk_cols);
     b.gu_a = b.gu;
     b.gu_split = 0;
@@ -2585,7 +2637,7 @@ Plan plan_for(const lpp_model* m, bool parking) {
     };
     // Parked gate/up rows: whatever LDS is left (binary16 models; the workgroups that hold the attention
     // items of a short context, one per query head, park nothing and own that many fewer hidden units).
-    if (parking && c.weight_precision == LPP_WEIGHT_FP16 && c.n_heads < p.grid) {
+    if (parking && c.weight_precision == LPP_WEIGHT_FP16 && c.n_heads < p.grid && (!xcd || kv_in_xs)) {
         constexpr size_t kLdsBytes = 160 * 1024, kReserve = 2048;  // the rest is for the kernel's static LDS
         const size_t used = lds_floats() * sizeof(float);
         const size_t row_bytes = static_cast<size_t>(c.dim) * 2;
@@ -2593,12 +2645,12 @@ Plan plan_for(const lpp_model* m, bool parking) {
         rows &= ~1;                                 // whole hidden units
         const int cap = 4 * df::kIoWaves;  // a handful of rows per exchange wavefront is plenty
         if (rows > cap) rows = cap;
-        // units of an ordinary workgroup if the first n_heads own rows / 2 fewer
-        const int gu = (c.hidden_dim + c.n_heads * (rows / 2) + p.grid - 1) / p.grid;
+        // units of an ordinary workgroup if the first n_heads own rows / 2 fewer (att_xcd_item: all workgroups alike)
+        const int gu = xcd ? b.gu : (c.hidden_dim + c.n_heads * (rows / 2) + p.grid - 1) / p.grid;
         if (rows >= 2 && gu - rows / 2 >= 1 && 2 * gu - rows >= df::kGemvWaves) {
             b.gu = gu;
-            b.gu_a = gu - rows / 2;
-            b.gu_split = c.n_heads;
+            b.gu_a = xcd ? gu : gu - rows / 2;
+            b.gu_split = xcd ? 0 : c.n_heads;
             b.park_rows = rows;
             b.park_floats = static_cast<int>((static_cast<size_t>(rows) * row_bytes + 31) / 32 * 8);
             if (2 * b.gu * b.ns_dim > slots) {
@@ -2615,13 +2667,13 @@ Plan plan_for(const lpp_model* m, bool parking) {
             b.results_floats = (slots + 7) & ~7;
         }
     }
+    if (xcd && !kv_in_xs)
+        b.kv_offset = static_cast<int>(lds_floats()) - b.kv_floats;  // the last area
     p.lds_bytes = lds_floats() * sizeof(float);
     return p;
 }
 
 constexpr int kGridCap = 1024;  // workgroups the statistics table has room for
-constexpr int kMaxXcc = 8;
-constexpr int kMaxPerXcc = 32;  // workgroups of one XCD the XCD-wide attention split is laid out for
 // Tagged values of one XCD's copy of an n-value vector: whole 128-byte lines.
 size_t near_stride(int n) { return (static_cast<size_t>(n) + 15) / 16 * 16; }
 
@@ -2644,33 +2696,6 @@ int lane_item_positions(const lpp_model* m, const Plan& p) {
     if (cap > df::kLaneItemPositions) cap = df::kLaneItemPositions;
     const int in_cache = m->cfg.seq_len / df::kWave * df::kWave;
     return cap < in_cache ? cap : in_cache;
-}
-
-// The split of a KV head's context over the workgroups of its XCD (att_xcd_item) at npos positions, for a plan whose
-// Wq/Wk/Wv rows are dealt out per XCD; chunk 0 where it does not apply.
-struct XcdAttention {
-    int chunk, active, ppw, cu_shift, opc, kv_floats;
-};
-XcdAttention xcd_attention_for(const lpp_model* m, const df::Blocks& b, int grid, int npos) {
-    XcdAttention x = {};
-    if (test_option(LPP_OPT_DECODE_XCD_ATTENTION) == 0 || b.qkv_by_xcc <= 0 || m->df_xcc <= 1) return x;
-    const int hs = m->head_size, g = m->gqa;
-    if ((hs != 64 && hs != 128) || (g != 1 && g != 2 && g != 4)) return x;
-    const int per_xcc = grid / m->df_xcc;
-    if (per_xcc > kMaxPerXcc || per_xcc % b.qkv_by_xcc != 0) return x;
-    const int n_cu = per_xcc / b.qkv_by_xcc;  // workgroups that share a KV head
-    if ((n_cu & (n_cu - 1)) != 0 || (g * hs) % n_cu != 0) return x;
-    const int opc = g * hs / n_cu;            // outputs each of them combines: all of one head, at most 16
-    if (opc > hs || hs % opc != 0 || opc > df::kMaxHeadPad / 8) return x;
-    const int chunk = ((npos + n_cu - 1) / n_cu + 7) & ~7;
-    if (chunk > df::kIoWaves * df::kWave) return x;
-    while ((1 << x.cu_shift) < n_cu) ++x.cu_shift;
-    x.chunk = chunk;
-    x.active = (npos + chunk - 1) / chunk;
-    x.ppw = chunk / df::kIoWaves;
-    x.opc = opc;
-    x.kv_floats = chunk * hs;  // eight wavefronts x ppw positions x (K row + V row) of binary16
-    return x;
 }
 
 df::Tagged tagged_of(const lpp_model* m, bool generating, int lane_item_cap) {
@@ -2890,14 +2915,12 @@ const char* dataflow_unsupported_reason(const lpp_model* m) {
     return nullptr;
 }
 
+lpp_status dataflow_take_options(lpp_model* m, hipStream_t s);
+
 template <bool kF16>
 static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s) {
     if (const char* why = dataflow_unsupported_reason(m)) return fail(LPP_ERR_UNSUPPORTED, "%s", why);
-    if (m->df_options_epoch != test_options_epoch()) {
-        // A test hook changed what the plans may use: forget what was derived under the old settings.
-        LPP_TRY(dataflow_forget_plans(m, s, 0));
-        m->df_options_epoch = test_options_epoch();
-    }
+    LPP_TRY(dataflow_take_options(m, s));
     if (m->df_xcc == 0) {
         // Workgroups are handed to the XCDs in turn.  The per-XCD hand-overs rely on every XCD getting an equal share
         // of them, so it is measured, not assumed: anything but workgroup w on XCD (first + w) % n switches them off.
@@ -2939,18 +2962,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
         const bool wanted = m->head_size == 64 ? npos > lane_cap : (tagged.att_splits > 1 || tagged.att_group_splits > 0);
         if (wanted) xa = xcd_attention_for(m, xcd_plan.blocks, xcd_plan.grid, npos);
         if (xa.chunk > 0) {
-            // (the item's LDS beyond the rows: a merge area for four heads, and the softmax weights in `gather`)
-            df::Blocks& xb = xcd_plan.blocks;
-            const int red_more = df::kIoWaves * df::kMaxAttHeads * df::kRedStride - xb.red_floats;
-            const int gather_more = df::kMaxAttHeads * df::kIoWaves * df::kWave > xb.gather_floats
-                                        ? df::kMaxAttHeads * df::kIoWaves * df::kWave - xb.gather_floats : 0;
-            xb.red_floats += red_more;
-            xb.gather_floats += gather_more;
-            xcd_plan.lds_bytes += static_cast<size_t>(red_more + gather_more) * sizeof(float);
-            xcd_plan.blocks.kv_floats = xa.kv_floats;
-            xcd_plan.blocks.xa_cu_shift = xa.cu_shift;
-            xcd_plan.blocks.xa_opc = xa.opc;
-            xcd_plan.lds_bytes += static_cast<size_t>(xa.kv_floats) * sizeof(float);
+            xcd_plan = plan_for(m, parking_allowed, &xa);
             if (xcd_plan.lds_bytes > kLdsLimit) xa.chunk = 0;
         }
     }
@@ -2963,7 +2975,8 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     }
     const bool use_parked = xa.chunk == 0 && parked_plan.blocks.park_rows > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0;
     const Plan p = xa.chunk > 0 ? xcd_plan : (use_parked ? parked_plan : plan_for(m, false));
-    const int which = use_parked ? 1 : 0;
+    // (step lists: [0] every row streamed, [1] the parked plan's, [2] those of att_xcd_item's plan with parked rows)
+    const int which = xa.chunk > 0 ? (xcd_plan.blocks.park_rows > 0 ? 2 : 0) : (use_parked ? 1 : 0);
     // q, k and v stay inside the XCD that formed them while every head's item sits on that XCD: one item per head
     tagged.local_qkv = (p.blocks.qkv_by_xcc > 0 && tagged.att_splits == 1 && tagged.att_group_splits == 0) ? 1 : 0;
     // Sequence numbers are compared for equality, so they must not come round to values that slots
@@ -2997,7 +3010,7 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     for (int t = 0; t < LPP_T_COUNT && !moved; ++t) moved = m->df_rows_key[t] != m->w[t];
     if (moved) {
         LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the old lists
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 3; ++i) {
             lpp_free(m->df_rows[i]);
             m->df_rows[i] = nullptr;
         }
@@ -3005,8 +3018,17 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     }
     // (both lists at once: a generation loop that grows past the short contexts must not stop to build the other one)
     if (m->df_rows[which] == nullptr) LPP_TRY(build_step_lists(m, p, which));
-    if (parked_plan.blocks.park_rows > 0 && m->df_rows[1 - which] == nullptr)
+    if (which < 2 && parked_plan.blocks.park_rows > 0 && m->df_rows[1 - which] == nullptr)
         LPP_TRY(build_step_lists(m, use_parked ? plan_for(m, false) : parked_plan, 1 - which));
+    if (which != 2 && m->df_rows[2] == nullptr && parking_allowed) {
+        // (the third as well, where a context of a thousand positions would take att_xcd_item's plan with parked rows)
+        const Plan plain = plan_for(m, false);
+        const XcdAttention probe = xcd_attention_for(m, plain.blocks, plain.grid, m->cfg.seq_len < 1024 ? m->cfg.seq_len : 1024);
+        if (probe.chunk > 0) {
+            const Plan later = plan_for(m, true, &probe);
+            if (later.blocks.park_rows > 0 && later.lds_bytes <= kLdsLimit) LPP_TRY(build_step_lists(m, later, 2));
+        }
+    }
     // (test hook: a ticket base one launch behind makes every workgroup's ticket look like one too many for its XCD)
     if (tagged.n_xcc > 1 && take_forced_ticket_failure()) tagged.ticket_base -= static_cast<unsigned>(m->persist_grid / tagged.n_xcc);
     LPP_REQUIRE(p.lds_bytes <= kLdsLimit, "persistent decode: %zu bytes of LDS per workgroup", p.lds_bytes);
@@ -3036,7 +3058,7 @@ lpp_status dataflow_launch(lpp_model* m, const ph::DecodeArgs& a, hipStream_t s)
 // device again, 1 leaves the per-XCD hand-overs off for this model.
 lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc) {
     LPP_HIP(hipStreamSynchronize(s));  // a launch still running may be reading the lists and drawing tickets
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 3; ++i) {
         lpp_free(m->df_rows[i]);
         m->df_rows[i] = nullptr;
     }
@@ -3051,10 +3073,18 @@ lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc) {
     return LPP_OK;
 }
 
+// A test hook changed what the plans may use: forget what was derived under the old settings (calibration included).
+lpp_status dataflow_take_options(lpp_model* m, hipStream_t s) {
+    if (m->df_options_epoch == test_options_epoch()) return LPP_OK;
+    LPP_TRY(dataflow_forget_plans(m, s, 0));
+    m->df_options_epoch = test_options_epoch();
+    return LPP_OK;
+}
+
 // The step lists alone (the partition of the hidden units changed): rebuilt at the next launch.
 lpp_status dataflow_forget_lists(lpp_model* m, hipStream_t s) {
     LPP_HIP(hipStreamSynchronize(s));
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 3; ++i) {
         lpp_free(m->df_rows[i]);
         m->df_rows[i] = nullptr;
     }

@@ -872,5 +872,6 @@ lpp_status dataflow_forget_plans(lpp_model* m, hipStream_t s, int df_xcc);
 lpp_status dataflow_forget_lists(lpp_model* m, hipStream_t s);
 void dataflow_partition_classes(const lpp_model* m, int* item_workgroups, int* n_xcc);
 lpp_status dataflow_after_error(lpp_model* m, int code, bool* relaunch);
+lpp_status dataflow_take_options(lpp_model* m, hipStream_t s);
 
 }  // namespace lpp

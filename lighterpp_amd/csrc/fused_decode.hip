@@ -351,10 +351,10 @@ lpp_status fused_release(lpp_model* m) {
     lpp_free(m->sync_words);
     lpp_free(m->sample_scratch);
     lpp_free(m->tagged);
-    lpp_free(m->df_rows[0]);
-    lpp_free(m->df_rows[1]);
-    lpp_free(m->df_gu_first[0]);
-    lpp_free(m->df_gu_first[1]);
+    for (int i = 0; i < 3; ++i) {
+        lpp_free(m->df_rows[i]);
+        lpp_free(m->df_gu_first[i]);
+    }
     lpp_free(m->gen_uniforms);
     return LPP_OK;
 }
@@ -717,7 +717,9 @@ static lpp_status trace_impl(lpp_model* m, int pos, unsigned long long* out, int
 // traced tokens write at that position are put back.
 static lpp_status calibrate_gateup(lpp_model* m) {
     using namespace lpp;
-    if (m->df_calibrated || m->path != LPP_PATH_PERSISTENT) return LPP_OK;
+    if (m->path != LPP_PATH_PERSISTENT) return LPP_OK;
+    LPP_TRY(dataflow_take_options(m, stream()));  // (a changed test option drops the calibration with the plans)
+    if (m->df_calibrated) return LPP_OK;
     m->df_calibrated = true;
     if (test_option(LPP_OPT_DECODE_CALIBRATE) == 0) return LPP_OK;
     for (int t = 0; t < LPP_T_COUNT; ++t)

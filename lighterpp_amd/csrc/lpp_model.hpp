@@ -56,10 +56,11 @@ struct lpp_model {
     float* gen_uniforms = nullptr;           // device copy of the per-step draws
     int gen_cap = 0;
     void* tagged = nullptr;                  // value+sequence-number vectors of the persistent kernel
-    void* df_rows[2] = {nullptr, nullptr};   // row lists of the persistent kernel's streaming wavefronts: [0] every row
-    int df_row_stride[2] = {0, 0};           // streamed, [1] with parked gate/up rows left out (short contexts)
+    void* df_rows[3] = {nullptr, nullptr, nullptr};  // row lists of the persistent kernel's streaming wavefronts: [0] every row
+    int df_row_stride[3] = {0, 0, 0};        // streamed, [1] with parked gate/up rows left out (short contexts), [2] the
+                                             // same for the plan that splits a context over an XCD
     const void* df_rows_key[12] = {};        // weight addresses the lists were built from
-    int* df_gu_first[2] = {nullptr, nullptr};  // device tables of the gate/up partition the lists were built for
+    int* df_gu_first[3] = {nullptr, nullptr, nullptr};  // device tables of the gate/up partition the lists were built for
     std::vector<float> df_gu_weight;         // per workgroup: its share of the hidden units relative to an even deal
     bool df_calibrated = false;              // a traced token has set df_gu_weight (or could not)
     // Host's own count of the step record for the persistent path: everything but the token id

@@ -775,7 +775,7 @@ __global__ __launch_bounds__(256) void k_attention(const float* __restrict__ q, 
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
-template <int kHs>
+template <int kHs, bool kLo>
 __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict__ q, const uint16_t* __restrict__ key_cache,
                                                         const uint16_t* __restrict__ value_cache, half_t* __restrict__ out_hi,
                                                         half_t* __restrict__ out_lo, int layer, int pos0, int dim, int kv_dim,
@@ -784,7 +784,9 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     const int lane = lane_id(), wave = wave_index();
     const int r = lane & 31, g = lane >> 5;
     const int tokens_per_tile = 32 / gqa;
-    const int t0 = static_cast<int>(blockIdx.x) * tokens_per_tile;
+    // (the tiles with the longest contexts are dispatched first: where not all workgroups are resident at once, the
+    // short ones fill the gaps at the end instead of the long ones starting last)
+    const int t0 = static_cast<int>(gridDim.x - 1 - blockIdx.x) * tokens_per_tile;
     if (t0 >= n_tokens) return;  // (the whole workgroup)
     const int kvh = blockIdx.y;
     const int my_tok = t0 + r / gqa, my_head = r % gqa;
@@ -795,9 +797,11 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     const int my_limit = pos0 + tok_c + 1;    // positions this lane's row attends to: [0, my_limit)
     const uint16_t* kbase = key_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * kHs;
     const uint16_t* vbase = value_cache + static_cast<size_t>(layer) * kv_dim * seq_len + static_cast<size_t>(kvh) * seq_len * kHs;
-    // this wavefront's tile of V^T: [d][32 positions], rows 72 bytes apart (8-byte reads, few shared banks)
-    constexpr int kTileRow = 36;  // binary16 per row
-    __shared__ __align__(16) uint16_t vt_tiles[4][kHs * kTileRow];
+    // this wavefront's tile of the block's V rows, as the cache holds them: [32 positions][kHs], rows 16 bytes
+    // longer than a cache row, so that the rows four positions apart, which the two halves of the wavefront read
+    // side by side, start 16 banks apart
+    constexpr int kTileRow = kHs + 8;  // binary16 per row
+    __shared__ __align__(16) uint16_t vt_tiles[4][32 * kTileRow];
     uint16_t* vt_tile = vt_tiles[wave];
     constexpr int kVChunks = kHs / 16;  // 16-byte pieces of the block's V rows per lane
     const float scale = 1.0f / sqrtf(static_cast<float>(kHs));  // model.cpp:188
@@ -862,7 +866,7 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
 #pragma unroll
         for (int s = 0; s < kKSteps; ++s) {
             st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], qh[s], st, 0, 0, 0);
-            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], ql[s], st, 0, 0, 0);
+            if constexpr (kLo) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], ql[s], st, 0, 0, 0);
         }
         float sv[16];
         float block_top = -INFINITY;
@@ -888,14 +892,13 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         block_sum += __shfl_xor(block_sum, 32);
         lsum = lsum * corr + block_sum;
         top = grown;
-        // V rows into the tile, a position's 8 dimensions down a column; the LDS serves a wavefront's accesses
-        // in order, so the fragment reads below see them (and the next block's writes come after these reads)
+        // V rows into the tile, 16 bytes a lane (no two lanes of a quarter wavefront on one bank); the LDS serves a
+        // wavefront's accesses in order, so the fragment reads below see them (and the next block's writes come
+        // after these reads)
 #pragma unroll
         for (int i = 0; i < kVChunks; ++i) {
             const int c = lane + 64 * i, p = c / (kHs / 8), d0 = (c % (kHs / 8)) * 8;
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                vt_tile[(d0 + e) * kTileRow + p] = static_cast<uint16_t>(vrows[i][e >> 1] >> (16 * (e & 1)));
+            *reinterpret_cast<uintx4*>(vt_tile + p * kTileRow + d0) = vrows[i];
         }
 #pragma unroll
         for (int dt = 0; dt < kDTiles; ++dt) {
@@ -903,12 +906,14 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
             for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-                const uint16_t* vrow = vt_tile + (32 * dt + r) * kTileRow + 16 * s2 + 4 * g;
-                const half4_t a0 = *reinterpret_cast<const half4_t*>(vrow);
-                const half4_t a1 = *reinterpret_cast<const half4_t*>(vrow + 8);
-                const half8_t vf = half8_t{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                // the fragment: dimension 32 dt + r at the eight positions this lane supplies, one 2-byte read each
+                // (32 lanes read 64 consecutive bytes: every bank once per half wavefront)
+                const half_t* vcol = reinterpret_cast<const half_t*>(vt_tile) + (16 * s2 + 4 * g) * kTileRow + 32 * dt + r;
+                half8_t vf;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) vf[j] = vcol[((j & 3) + 8 * (j >> 2)) * kTileRow];
                 o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, ph[s2], o[dt], 0, 0, 0);
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pl[s2], o[dt], 0, 0, 0);
+                if constexpr (kLo) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pl[s2], o[dt], 0, 0, 0);
             }
         }
     }
@@ -958,7 +963,7 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
                     l[u] = static_cast<half_t>(v - static_cast<float>(h[u]));
                 }
                 *reinterpret_cast<half4_t*>(out_hi + base + 32 * dt + 8 * e4 + 4 * g) = h;
-                *reinterpret_cast<half4_t*>(out_lo + base + 32 * dt + 8 * e4 + 4 * g) = l;
+                if constexpr (kLo) *reinterpret_cast<half4_t*>(out_lo + base + 32 * dt + 8 * e4 + 4 * g) = l;
             }
     }
 }
@@ -1278,12 +1283,18 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         if (matrix_cores) {
             const int tiles = (n + 32 / m->gqa - 1) / (32 / m->gqa);
             const dim3 grid(tiles, c.n_kv_heads);
-            if (hs == 64)
-                hipLaunchKernelGGL(pf::k_attention_mfma<64>, grid, dim3(256), 0, s, q, m->key_cache, m->value_cache, hi, lo, l, pos0,
-                                   dim, kv, m->gqa, c.seq_len, n);
-            else
-                hipLaunchKernelGGL(pf::k_attention_mfma<128>, grid, dim3(256), 0, s, q, m->key_cache, m->value_cache, hi, lo, l, pos0,
-                                   dim, kv, m->gqa, c.seq_len, n);
+#define LPP_PF_ATTENTION(HS, LO)                                                                                          \
+    hipLaunchKernelGGL((pf::k_attention_mfma<HS, LO>), grid, dim3(256), 0, s, q, m->key_cache, m->value_cache, hi, lo, l, pos0, \
+                       dim, kv, m->gqa, c.seq_len, n)
+            // (the fast mode rounds q and the softmax weights to binary16 as it rounds every GEMM input)
+            if (hs == 64) {
+                if (exact) LPP_PF_ATTENTION(64, true);
+                else LPP_PF_ATTENTION(64, false);
+            } else {
+                if (exact) LPP_PF_ATTENTION(128, true);
+                else LPP_PF_ATTENTION(128, false);
+            }
+#undef LPP_PF_ATTENTION
             LPP_CHECK_LAUNCH("k_attention_mfma");
         } else if (hs == 64)
             hipLaunchKernelGGL(pf::k_attention<8>, dim3((n + 3) / 4, c.n_kv_heads), dim3(256), 0, s, q, m->key_cache,

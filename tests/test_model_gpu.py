@@ -412,6 +412,11 @@ XCD_SPLIT = {
     "hs128_mha_8kv": (Shape(1024, 512, 1, 8, 8, 500, 700, 10000.0, fp16=True, tied=True), (120, 640)),
     "hs64_mha_32kv": (Shape(2048, 512, 1, 32, 32, 500, 4200, 10000.0, fp16=True, tied=True), (520, 4090)),
     "hs64_gqa2_16kv": (Shape(2048, 512, 1, 32, 16, 500, 1100, 500000.0, fp16=True, tied=False), (515, 1000)),
+    # hidden_dim well above dim: the share's rows live in the part of the staged-activation area that only the down
+    # phase uses, and every workgroup parks gate/up rows beside the item (two layers: the down phase overwrites the
+    # rows in between); the last start of the first shape is past what that area holds (3072 positions)
+    "hs64_gqa4_8kv_parked": (Shape(2048, 8192, 2, 32, 8, 500, 3300, 500000.0, fp16=True, tied=True), (520, 3066, 3090)),
+    "hs128_gqa4_8kv_parked": (Shape(4096, 14336, 2, 32, 8, 500, 1300, 500000.0, fp16=True, tied=False), (620, 1050)),
 }
 
 
