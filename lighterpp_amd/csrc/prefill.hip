@@ -870,20 +870,38 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         }
         float sv[16];
         float block_top = -INFINITY;
+        if (p0 + 32 <= pos0 + t0 + 1) {  // (uniform) every row of the tile attends to the whole block: nothing to mask
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int pos = p0 + 8 * (e >> 2) + 4 * g + (e & 3);
-            sv[e] = (pos < my_limit) ? st[e] * scale : -INFINITY;
-            block_top = fmaxf(block_top, sv[e]);
+            for (int e = 0; e < 16; ++e) {
+                sv[e] = st[e] * scale;
+                block_top = fmaxf(block_top, sv[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int pos = p0 + 8 * (e >> 2) + 4 * g + (e & 3);
+                sv[e] = (pos < my_limit) ? st[e] * scale : -INFINITY;
+                block_top = fmaxf(block_top, sv[e]);
+            }
         }
         block_top = fmaxf(block_top, __shfl_xor(block_top, 32));
-        const float grown = fmaxf(top, block_top);  // finite from the first block on: position 0 is in every row's range
-        const float corr = (top == -INFINITY) ? 0.0f : exp_fast(top - grown);
+        // The reference the exponentials are taken against follows the row's maximum lazily: it moves only when a
+        // block's maximum exceeds it by more than kSlack (weights then stay below e^kSlack, far inside binary16, and
+        // any reference gives the same quotient in the end).  After a row's first blocks it hardly ever moves, and a
+        // block in which no row's reference moved skips the rescaling of the running sums and outputs altogether.
+        constexpr float kSlack = 4.0f;
+        const bool moves = block_top > top + kSlack;  // (true for the first block: top is -inf; finite from then on: position 0 is in every row's range)
+        const float grown = moves ? block_top : top;
+        const float corr = (top == -INFINITY) ? 0.0f : (moves ? exp_fast(top - grown) : 1.0f);
+        const bool rescale = __builtin_amdgcn_ballot_w64(moves && top != -INFINITY) != 0ull;  // (uniform; outputs are still zero before the first block)
         half8_t ph[2], pl[2];
         float block_sum = 0.0f;
+        // (a row that has seen nothing but masked positions so far keeps -inf as its reference: its weights are
+        // exp(-inf - 0) = 0 instead of exp(-inf + inf))
+        const float against = (grown == -INFINITY) ? 0.0f : grown;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float pw = (sv[e] == -INFINITY) ? 0.0f : exp_fast(sv[e] - grown);
+            const float pw = exp_fast(sv[e] - against);
             block_sum += pw;
             const half_t h = static_cast<half_t>(pw);
             ph[e >> 3][e & 7] = h;
@@ -902,8 +920,10 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
         }
 #pragma unroll
         for (int dt = 0; dt < kDTiles; ++dt) {
+            if (rescale) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
+                for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
+            }
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
                 // the fragment: dimension 32 dt + r at the eight positions this lane supplies, one 2-byte read each
@@ -951,6 +971,7 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
     }
     if (valid) {
         const size_t base = static_cast<size_t>(my_tok) * dim + (kvh * gqa + my_head) * kHs;
+        const float inv_sum = 1.0f / lsum;
 #pragma unroll
         for (int dt = 0; dt < kDTiles; ++dt)
 #pragma unroll
@@ -958,7 +979,7 @@ __global__ __launch_bounds__(256) void k_attention_mfma(const float* __restrict_
                 half4_t h, l;
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const float v = o[dt][4 * e4 + u] / lsum;
+                    const float v = o[dt][4 * e4 + u] * inv_sum;
                     h[u] = static_cast<half_t>(v);
                     l[u] = static_cast<half_t>(v - static_cast<float>(h[u]));
                 }
