@@ -90,11 +90,44 @@ __global__ __launch_bounds__(kAttThreads) void scale_kernel(float* att, float sc
 
 // ops.cpp:56-75 per head: max, expf(x - max) with a tree sum, true division.
 constexpr int kSoftmaxThreads = 1024;
+// kSoftmaxKept: values a thread keeps in registers (1, 4 or 16: rows of up to 16384 positions, the context cap of
+// loader.cpp:310); 0: any length, the row re-read from memory in every pass.
+template <int kSoftmaxKept>
 __global__ __launch_bounds__(kSoftmaxThreads) void softmax_kernel(float* out, const float* x,
                                                                   int npos, int att_stride) {
     __shared__ float scratch[16];
     const float* row = x + static_cast<size_t>(blockIdx.x) * att_stride;
     float* orow = out + static_cast<size_t>(blockIdx.x) * att_stride;
+    if constexpr (kSoftmaxKept > 0) {
+        // The row stays in registers between the three passes (one read, one write; the same values meet the same
+        // reductions in the same order as below, so the result is the same bit for bit).
+        float v[kSoftmaxKept > 0 ? kSoftmaxKept : 1];
+        float top = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < kSoftmaxKept; ++k) {
+            const int t = static_cast<int>(threadIdx.x) + k * kSoftmaxThreads;
+            v[k] = t < npos ? row[t] : -INFINITY;
+        }
+#pragma unroll
+        for (int k = 0; k < kSoftmaxKept; ++k) top = fmaxf(top, v[k]);
+        top = block_max(top, scratch);
+        float total = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kSoftmaxKept; ++k) {
+            const int t = static_cast<int>(threadIdx.x) + k * kSoftmaxThreads;
+            if (t < npos) {
+                v[k] = expf(v[k] - top);
+                total += v[k];
+            }
+        }
+        total = block_sum(total, scratch);
+#pragma unroll
+        for (int k = 0; k < kSoftmaxKept; ++k) {
+            const int t = static_cast<int>(threadIdx.x) + k * kSoftmaxThreads;
+            if (t < npos) orow[t] = v[k] / total;
+        }
+        return;
+    }
     float top = -INFINITY;
     for (int t = threadIdx.x; t < npos; t += kSoftmaxThreads) top = fmaxf(top, row[t]);
     top = block_max(top, scratch);
@@ -148,14 +181,14 @@ __global__ __launch_bounds__(kAggThreads) void aggregate_kernel(float* __restric
         out[static_cast<size_t>(h) * head_size + e] = part[e];
 }
 
-// Long contexts: kSplit workgroups per query head, each over a contiguous run of positions, so that the launch has
+// Long contexts: several workgroups per query head, each over a contiguous run of positions, so that the launch has
 // work for every compute unit (one workgroup per head leaves most of them idle and takes 29 us for 8193 positions
 // of the 1B shape).  A workgroup leaves its partial sums in a scratch area that lives in the library's device image
 // (the operator allocates nothing and takes no workspace argument); the workgroup of a head that finishes last adds
 // the partials up, always in split order, so the result does not depend on who finished when.  Calls on different
 // streams would share the scratch: like the reference's operators, these are for one stream.
 constexpr int kAggSplitThreads = 512;
-constexpr int kAggMaxHeads = 256, kAggMaxSplits = 16, kAggPad = 128;
+constexpr int kAggMaxHeads = 256, kAggMaxSplits = 8, kAggPad = 128;
 static __device__ float agg_partials[kAggMaxHeads * kAggMaxSplits * kAggPad];
 static __device__ unsigned agg_tickets[kAggMaxHeads];  // back at zero after every launch
 
@@ -165,10 +198,10 @@ __global__ __launch_bounds__(kAggSplitThreads) void aggregate_split_kernel(float
                                                                            const float* __restrict__ att, int npos,
                                                                            int head_size, int gqa, int att_stride,
                                                                            float* partials, unsigned* tickets) {
-    extern __shared__ __align__(16) float part[];  // [ngroups][hs_pad]
+    constexpr int kWaves = kAggSplitThreads / kWave;
+    __shared__ float part[kWaves][kAggPad];  // a wavefront's sums, one row each
     __shared__ int is_last;
     constexpr int kGroups = kAggSplitThreads / kGroup;
-    constexpr int hs_pad = kGroup * 8;
     const int h = blockIdx.x, split = blockIdx.y, nsplits = gridDim.y;
     const int sub = static_cast<int>(threadIdx.x) % kGroup;
     const int grp = static_cast<int>(threadIdx.x) / kGroup;
@@ -178,7 +211,7 @@ __global__ __launch_bounds__(kAggSplitThreads) void aggregate_split_kernel(float
     const float* ah = att + static_cast<size_t>(h) * att_stride;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (sub * 8 < head_size) {
-        constexpr int kUnroll = 4;  // rows requested before the first is used
+        constexpr int kUnroll = 8;  // rows requested before the first is used: 512 positions a trip (heads of 64)
         for (int t0 = t_begin + grp; t0 < t_end; t0 += kUnroll * kGroups) {
             uintx4 rows[kUnroll];
             float w[kUnroll];
@@ -200,15 +233,25 @@ __global__ __launch_bounds__(kAggSplitThreads) void aggregate_split_kernel(float
             }
         }
     }
+    // The groups of a wavefront meet by lane exchange (group g with g ^ 1, then ^ 2, ...), the wavefronts through LDS,
+    // added in wavefront order: always the same order, so a call repeats bit for bit.
 #pragma unroll
-    for (int e = 0; e < 8; ++e) part[grp * hs_pad + sub * 8 + e] = acc[e];
-    __syncthreads();
-    for (int width = kGroups / 2; width >= 1; width >>= 1) {
-        for (int i = threadIdx.x; i < width * hs_pad; i += kAggSplitThreads) part[i] += part[i + width * hs_pad];
-        __syncthreads();
+    for (int off = kGroup; off < kWave; off <<= 1)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], off);
+    const int wave = static_cast<int>(threadIdx.x) / kWave;
+    if (lane_id() < kGroup) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part[wave][sub * 8 + e] = acc[e];
     }
+    __syncthreads();
     float* mine = partials + (static_cast<size_t>(h) * kAggMaxSplits + split) * kAggPad;
-    for (int e = threadIdx.x; e < head_size; e += kAggSplitThreads) Mem<true>::st(mine + e, part[e]);
+    for (int e = threadIdx.x; e < head_size; e += kAggSplitThreads) {
+        float s = part[0][e];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) s += part[w][e];
+        Mem<true>::st(mine + e, s);
+    }
     // (the barrier waits for this workgroup's stores; the ticket is drawn after it)
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -218,10 +261,18 @@ __global__ __launch_bounds__(kAggSplitThreads) void aggregate_split_kernel(float
     }
     __syncthreads();
     if (!is_last) return;
+    // the last range to arrive adds the ranges' sums in range order, eight of them requested at a time
     const float* all = partials + static_cast<size_t>(h) * kAggMaxSplits * kAggPad;
     for (int e = threadIdx.x; e < head_size; e += kAggSplitThreads) {
-        float s = Mem<true>::ld(all + e);
-        for (int k = 1; k < nsplits; ++k) s += Mem<true>::ld(all + k * kAggPad + e);
+        float s = 0.0f;
+        for (int k0 = 0; k0 < nsplits; k0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = k0 + u < nsplits ? Mem<true>::ld(all + (k0 + u) * kAggPad + e) : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (k0 + u < nsplits) s = (k0 + u == 0) ? v[u] : s + v[u];
+        }
         out[static_cast<size_t>(h) * head_size + e] = s;
     }
 }
@@ -332,8 +383,14 @@ lpp_status lpp_softmax_multihead(float* d_out, const float* d_x, int n_heads, in
     LPP_REQUIRE(d_out && d_x, "lpp_softmax_multihead: null pointer");
     LPP_REQUIRE(n_heads > 0 && seq_len > 0 && att_stride >= seq_len,
                 "lpp_softmax_multihead: n_heads = %d, seq_len = %d, att_stride = %d", n_heads, seq_len, att_stride);
-    hipLaunchKernelGGL(softmax_kernel, dim3(n_heads), dim3(kSoftmaxThreads), 0, stream(), d_out, d_x,
-                       seq_len, att_stride);
+#define LPP_SOFTMAX(KEPT)                                                                                    \
+    hipLaunchKernelGGL((softmax_kernel<KEPT>), dim3(n_heads), dim3(kSoftmaxThreads), 0, stream(), d_out, d_x, \
+                       seq_len, att_stride)
+    if (seq_len <= kSoftmaxThreads) LPP_SOFTMAX(1);
+    else if (seq_len <= 4 * kSoftmaxThreads) LPP_SOFTMAX(4);
+    else if (seq_len <= 16 * kSoftmaxThreads) LPP_SOFTMAX(16);
+    else LPP_SOFTMAX(0);
+#undef LPP_SOFTMAX
     LPP_CHECK_LAUNCH("softmax_kernel");
     return LPP_OK;
 }
@@ -353,15 +410,18 @@ lpp_status lpp_aggregation_multihead(float* d_out, const lpp_half* d_v, const fl
         LPP_CHECK_LAUNCH("aggregate_generic_kernel");
         return LPP_OK;
     }
-    // Enough workgroups for the device once a head's context is long (two per compute unit, a few hundred positions each).
-    int splits = (2 * compute_units() + n_heads - 1) / n_heads;
+    // Work for every compute unit once a head's context is long: a workgroup per head and range of a few hundred
+    // positions.  No more than eight ranges: the ranges of a head meet at one counter, and read-modify-writes of one
+    // address at device scope are served one at a time, 0.1 us each (8193 positions, 32 heads: 13.2 us with 32 ranges,
+    // 10.3 with 16, 9.6 with 8, of which an empty launch of the same grid takes 3.9).
+    int splits = (compute_units() + n_heads - 1) / n_heads;
     if (splits > kAggMaxSplits) splits = kAggMaxSplits;
     if (splits > seq_len / 256) splits = seq_len / 256;
     if (splits > 1 && n_heads <= kAggMaxHeads && g >= 1) {
         float* partials = nullptr;
         unsigned* tickets = nullptr;
         LPP_TRY(agg_scratch(&partials, &tickets));
-        const size_t lds_split = static_cast<size_t>(kAggSplitThreads) * 8 * sizeof(float);
+        const size_t lds_split = 0;
 #define LPP_AGG_SPLIT(G)                                                                                              \
     hipLaunchKernelGGL((aggregate_split_kernel<G>), dim3(n_heads, splits), dim3(kAggSplitThreads), lds_split, stream(), \
                        d_out, d_v, d_att, seq_len, head_size, gqa_factor, att_stride, partials, tickets)

@@ -338,6 +338,25 @@ def test_persistent_alternatives_the_library_selects_by_itself(variant, test_opt
     o.close()
 
 
+def test_generate_grows_from_the_parked_rows_plan_into_the_xcd_split():
+    """One generation call that starts inside the one-pass item's 512 positions and ends past them: the launches
+    change plan, step lists and kernel instance in mid-flight (the next token's launch is queued before the last
+    one's id is back).  Teacher-forced against the oracle; the cache before the start holds zeros on both sides."""
+    shape = SELF_SELECTED
+    m, o = build(shape, 33)
+    m.set_path(capi.PATH_PERSISTENT)
+    start, steps = 505, 14
+    toks, _, _ = m.generate(5, start, steps, temperature=0.0)
+    tok = 5
+    for i in range(steps):
+        want = o.forward_logits(tok, start + i)
+        assert int(toks[i]) == int(np.argmax(want)), (start + i, toks.tolist())
+        tok = int(toks[i])
+    assert rel_err(m.buffer(capi.B_LOGITS), want) <= LOGIT_TOL
+    m.close()
+    o.close()
+
+
 def test_gateup_partition_weighted_by_xcd_changes_no_bit(test_options):
     """Before its first token a model on the persistent path traces two tokens and deals the hidden units out by how
     fast each XCD got through the gate/up phase.  Who forms a hidden unit does not change its value, and the cache row

@@ -307,7 +307,10 @@ def test_scale_multihead_bit_exact(lib):  # runtests.cpp:696-748
     assert np.array_equal(bits(got[:, n:]), bits(att[:, n:]))
 
 
-@pytest.mark.parametrize("nh,n,stride", [(4, 32, 64), (32, 512, 2048), (32, 8448, 16384), (6, 1, 256), (3, 1025, 1030)])
+# (rows of up to 1024, 4096 and 16384 values take a kernel that keeps them in registers, longer ones the general kernel)
+@pytest.mark.parametrize("nh,n,stride", [(4, 32, 64), (32, 512, 2048), (32, 8448, 16384), (6, 1, 256), (3, 1025, 1030),
+                                         (2, 1024, 1024), (2, 4096, 4100), (2, 4097, 4100), (2, 16384, 16384),
+                                         (2, 16385, 16400), (1, 40000, 40000)])
 def test_softmax_multihead(lib, nh, n, stride):  # runtests.cpp:633-694
     if (nh, n, stride) == (4, 32, 64):
         x = np.zeros((nh, stride), F)
