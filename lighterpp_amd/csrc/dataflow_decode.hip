@@ -1059,7 +1059,7 @@ __device__ __forceinline__ void park_fetch(Ctx& c, Io& io, const Lds& l, int lay
     const int loads_per_row = (row_bytes + 1023) >> 10;  // one wavefront load covers 1 KiB
     const int mine = (parked - io.iw + kIoWaves - 1) / kIoWaves;
     const int total = mine * loads_per_row;
-    constexpr int kBatch = 12;
+    constexpr int kBatch = 16;
     char* park = reinterpret_cast<char*>(l.park);
     for (int base = 0; base < total; base += kBatch) {
         uintx4 v[kBatch];

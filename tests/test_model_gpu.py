@@ -251,6 +251,11 @@ ONE_PASS = {
     # KV-head boundaries and an XCD's first workgroups hold the items of two KV heads.
     "mha_16kv": Shape(1024, 512, 1, 16, 16, 500, 640, 10000.0, fp16=True, tied=True),
     "gqa2_16kv": Shape(2048, 512, 1, 32, 16, 500, 640, 500000.0, fp16=True, tied=False),
+    # Fewer KV heads than XCDs: two (four, eight) XCDs share a KV head, each with part of its query heads and its own
+    # copy of the k and v rows ("gqa2_4kv" above is one of these too: a single query head per XCD).
+    "gqa8_4kv": Shape(2048, 1024, 2, 32, 4, 500, 640, 10000.0, fp16=True, tied=False),
+    "gqa8_2kv": Shape(1024, 512, 1, 16, 2, 500, 640, 500000.0, fp16=True, tied=True),
+    "gqa8_1kv": Shape(512, 512, 2, 8, 1, 500, 640, 10000.0, fp16=True, tied=True),
 }
 
 
