@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void k_norm_split_wide(float* __restrict__ x, 
 #pragma unroll
         for (int c = 0; c < kPer; ++c) {
             *reinterpret_cast<half4_t*>(hi + row + 1024 * c + first) = zero;
-            *reinterpret_cast<half4_t*>(lo + row + 1024 * c + first) = zero;
+            if (lo != nullptr) *reinterpret_cast<half4_t*>(lo + row + 1024 * c + first) = zero;
         }
         return;
     }
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256) void k_norm_split_wide(float* __restrict__ x, 
             l[e] = static_cast<half_t>(y - static_cast<float>(h[e]));
         }
         *reinterpret_cast<half4_t*>(hi + row + 1024 * c + first) = h;
-        *reinterpret_cast<half4_t*>(lo + row + 1024 * c + first) = l;
+        if (lo != nullptr) *reinterpret_cast<half4_t*>(lo + row + 1024 * c + first) = l;  // (null: nobody reads the remainders)
     }
 }
 
@@ -590,7 +590,7 @@ __global__ __launch_bounds__(512) void k_gemm_pipe(PipeJob job) {
                 }
             const size_t at = static_cast<size_t>(t_base + wt * 32 * kTj + 32 * j) * job.out_ld + f_base + wf * 64 + 8 * part8;
 #pragma unroll
-            for (int part = 0; part < 2; ++part) {
+            for (int part = 0; part < (kLo ? 2 : 1); ++part) {  // (without kLo the next GEMM reads no remainders either)
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -1192,10 +1192,12 @@ lpp_status gemm(const Product* prods, int count, const pf::half_t* xh, const pf:
     return LPP_OK;
 }
 
+// (remainders false: nobody reads lo after this norm, and the wide kernel leaves it unwritten)
 lpp_status norm_split(float* x, const float* gain, pf::half_t* hi, pf::half_t* lo, int dim, int n, int t_pad, const float* partials,
-                      int splits, size_t split_stride, hipStream_t s) {
+                      int splits, size_t split_stride, hipStream_t s, bool remainders = true) {
+    pf::half_t* lo_wide = remainders ? lo : nullptr;
 #define LPP_NORM_WIDE(PER, SPLITS) \
-    hipLaunchKernelGGL((pf::k_norm_split_wide<PER, SPLITS>), dim3(t_pad), dim3(256), 0, s, x, gain, hi, lo, n, partials, split_stride)
+    hipLaunchKernelGGL((pf::k_norm_split_wide<PER, SPLITS>), dim3(t_pad), dim3(256), 0, s, x, gain, hi, lo_wide, n, partials, split_stride)
 #define LPP_NORM_WIDE_DIM(PER)          \
     switch (splits) {                   \
         case 0: LPP_NORM_WIDE(PER, 0); break; \
@@ -1278,11 +1280,14 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
     const bool exact = m->pf_mode != LPP_PREFILL_FAST;
     const bool fused_ffn = dim % pf::kPipeTripK == 0 && hidden % 128 == 0 && test_option(LPP_OPT_PREFILL_STAGED_GEMM) != 0 &&
                            test_option(LPP_OPT_PREFILL_FUSED_FFN) != 0;
+    // Nobody reads a remainder when every GEMM of the chain is a staged one in the fast mode: the kernels that produce
+    // activations then leave the remainders unwritten.  (The direct GEMM, taken for other shapes, always reads them.)
+    const bool lean = !exact && fused_ffn;
     int pending = 0;  // ranges of the product before (W2's, then Wo's) still to be added to x
     for (int l = 0; l < c.n_layers; ++l) {
         // attention block, model.cpp:216-218
         LPP_TRY(norm_split(x, static_cast<const float*>(m->w[LPP_T_RMS_ATT]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, t_pad, gate,
-                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s));
+                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s, !lean));
         // What a prefill leaves behind is the cache: the last layer needs its K and V rows only, and
         // nothing reads what the rest of that layer would compute.
         const bool last_layer = l == c.n_layers - 1;
@@ -1309,10 +1314,10 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
                        dim, kv, m->gqa, c.seq_len, n)
             // (the fast mode rounds q and the softmax weights to binary16 as it rounds every GEMM input)
             if (hs == 64) {
-                if (exact) LPP_PF_ATTENTION(64, true);
+                if (!lean) LPP_PF_ATTENTION(64, true);
                 else LPP_PF_ATTENTION(64, false);
             } else {
-                if (exact) LPP_PF_ATTENTION(128, true);
+                if (!lean) LPP_PF_ATTENTION(128, true);
                 else LPP_PF_ATTENTION(128, false);
             }
 #undef LPP_PF_ATTENTION
@@ -1328,7 +1333,7 @@ lpp_status prefill_chunk(lpp_model* m, const int* tokens, int n, int pos0) {
         LPP_TRY(gemm(&wo, 1, hi, lo, dim, t_pad, true, s, gate, room, &pending, exact));
         // feed-forward block, model.cpp:221-226
         LPP_TRY(norm_split(x, static_cast<const float*>(m->w[LPP_T_RMS_FFN]) + static_cast<size_t>(l) * dim, hi, lo, dim, n, t_pad, gate,
-                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s));
+                           pending > 1 ? pending : 0, static_cast<size_t>(t_pad) * dim, s, !lean));
         if (fused_ffn) {
             LPP_TRY(gate_up_swiglu(layer_of(LPP_T_W1, l, hidden, dim), layer_of(LPP_T_W3, l, hidden, dim), hidden, hi, lo, dim, t_pad,
                                    hi2, lo2, s, exact));

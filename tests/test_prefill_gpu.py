@@ -204,13 +204,16 @@ def test_run_with_batched_prefill_matches_run(temperature):
     m.close()
 
 
+@pytest.mark.parametrize("direct_gemm", [False, True], ids=["staged", "direct_gemm"])
 @pytest.mark.parametrize("name", list(SHAPES))
-def test_fast_prefill_stays_inside_the_logits_bar(name):
+def test_fast_prefill_stays_inside_the_logits_bar(name, direct_gemm, test_options):
     """LPP_PREFILL_FAST: every GEMM of the prefill sees its input rounded to binary16 (the head of the activation
     alone, no remainder product), accumulation in fp32.  The contract that is left is the decode loop's own: the
     steps after the prompt within 2e-3 of the CPU path's logits and the same greedy ids; cache entries may sit a few
     binary16 steps from the oracle's (bounded here at 2^-6 of the largest entry)."""
     shape = SHAPES[name]
+    if direct_gemm:  # (the GEMM without LDS stages always reads the remainders: the kernels before it must still write them)
+        test_options(capi.OPT_PREFILL_STAGED_GEMM, 0)
     b = Model(shape)
     w = b.load_synthetic(7, keep=True)
     o = ob.OracleModel(shape, w, fp16=True, kv_round_f16=True)
