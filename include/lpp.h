@@ -369,8 +369,11 @@ lpp_status lpp_prefill_supported(const lpp_model *m);
  * binary16 remainder, two matrix-core products per weight tile: every cache entry lands within one binary16 step of
  * what prefill-by-decode writes.  LPP_PREFILL_FAST: the head alone -- the activations rounded to binary16 where a
  * GEMM reads them, which is what the reference's own GPU GEMV does to x (matmul.cu:85-98), accumulation still fp32:
- * a quarter fewer matrix-core cycles and a third fewer bytes through LDS; the steps that follow stay inside the
- * logits bar of 2e-3 against the CPU path, cache entries drift by a few binary16 steps over the layers. */
+ * half the matrix-core products and a third fewer bytes through LDS, at a price in accuracy that grows with the
+ * depth of the model: every rounded GEMM input adds about 3e-4 of the output's size.  The logits of the steps that
+ * follow are then 1.5e-3 to 1.7e-3 from the CPU path's at 16 and 22 layers (inside the decode loop's bar of 2e-3,
+ * not by much) and 5e-3 at 32 layers (outside it); cache entries drift by a few binary16 steps.  Opt-in for that
+ * reason: the exact mode is the one whose results are held to the decode loop's bar at every shape. */
 enum { LPP_PREFILL_EXACT = 0, LPP_PREFILL_FAST = 1 };
 lpp_status lpp_model_set_prefill_mode(lpp_model *m, int mode);
 lpp_status lpp_prefill(lpp_model *m, const int *tokens, int n_tokens, int start_pos);
