@@ -162,6 +162,7 @@ struct Blocks {
     int xa_cu_shift;  // att_xcd_item: log2 of the workgroups that share a KV head
     int xa_opc;       // att_xcd_item: attention outputs each of them combines
     int kv_floats;    // LDS for the K and V rows of a workgroup's share of a context, where they have an area of their own
+    int qkv_floats;   // LDS for this token's q (a row per head of an item), k and v rows
     int kv_offset;    // where those rows start, in floats from the start of LDS (their own area, or inside xs: see plan_for)
     int slice_dim;  // columns per slice of a dim-column row (slice_width)
     int down;   // rows of W2
@@ -1340,7 +1341,7 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
     if (lane_id() < kGroup) {
 #pragma unroll
         for (int h = 0; h < kHeads; ++h) {
-            float* r = l.red + (io.iw * kItemHeads + h) * kRedStride;
+            float* r = l.red + (io.iw * kHeads + h) * kRedStride;  // (as many heads per wavefront as the item covers)
             if (lane_live) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) r[sub * 8 + e] = acc[h][e];
@@ -1360,11 +1361,11 @@ __device__ __forceinline__ void att_group_item(Ctx& c, Io& io, const Lds& l, int
         const int h = div_head_size(c, io.it), e = io.it - h * hs;
         float all = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kIoWaves; ++w) all = fmaxf(all, l.red[(w * kItemHeads + h) * kRedStride + kMaxHeadPad]);
+        for (int w = 0; w < kIoWaves; ++w) all = fmaxf(all, l.red[(w * kHeads + h) * kRedStride + kMaxHeadPad]);
         float o = 0.0f, ls = 0.0f;
 #pragma unroll
         for (int w = 0; w < kIoWaves; ++w) {
-            const float* r = l.red + (w * kItemHeads + h) * kRedStride;
+            const float* r = l.red + (w * kHeads + h) * kRedStride;
             const float f = (r[kMaxHeadPad] == -INFINITY) ? 0.0f : exp_fast(r[kMaxHeadPad] - all);
             o += r[e] * f;
             ls += r[kMaxHeadPad + 1] * f;
@@ -1550,7 +1551,7 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
         mark(c, io, 2);
     }
 
-    float* red = l.red + (io.iw * kItemHeads) * kRedStride;
+    float* red = l.red + io.iw * kRedStride;  // (one head)
     float top = -INFINITY, lsum = 0.0f, o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
     if (wave_live) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows are in
@@ -1661,7 +1662,7 @@ __device__ __forceinline__ void att_lane_item(Ctx& c, Io& io, const Lds& l, int 
         float wtop[kIoWaves], wsum[kIoWaves], wout[kIoWaves];
 #pragma unroll
         for (int w = 0; w < kIoWaves; ++w) {
-            const float* r = l.red + (w * kItemHeads) * kRedStride;
+            const float* r = l.red + w * kRedStride;
             wtop[w] = r[kMaxHeadPad];
             wsum[w] = r[kMaxHeadPad + 1];
             wout[w] = r[e];
@@ -2453,7 +2454,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     l.results = l.xs + b.xs_floats;
     l.sc = l.results + b.results_floats;
     l.qkv = l.sc + 2 * kAttScoreFloats;
-    l.red = l.qkv + (kMaxAttHeads + 2) * kMaxHeadPad;
+    l.red = l.qkv + b.qkv_floats;
     l.gather = l.red + b.red_floats;
     l.park = l.gather + b.gather_floats;
     l.kv = lds + b.kv_offset;
@@ -2610,6 +2611,7 @@ Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr
     b.results_floats = (slots + 7) & ~7;
     b.gather_floats = (splits_cap_for(m) * (m->head_size + 2) + 7) & ~7;
     b.red_floats = df::kIoWaves * df::kItemHeads * df::kRedStride;
+    b.qkv_floats = (df::kMaxAttHeads + 2) * df::kMaxHeadPad;
     b.xa_cu_shift = 0;
     b.xa_opc = 0;
     b.kv_floats = 0;
@@ -2632,13 +2634,18 @@ Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr
     b.park_floats = 0;
     auto lds_floats = [&]() {
         return static_cast<size_t>(dim_pad + b.xs_floats + b.results_floats + 2 * df::kAttScoreFloats +
-                                   (df::kMaxAttHeads + 2) * df::kMaxHeadPad + b.red_floats + b.gather_floats + b.park_floats +
+                                   b.qkv_floats + b.red_floats + b.gather_floats + b.park_floats +
                                    b.kv_floats);
     };
     // Parked gate/up rows: whatever LDS is left (binary16 models; the workgroups that hold the attention
     // items of a short context, one per query head, park nothing and own that many fewer hidden units).
     if (parking && c.weight_precision == LPP_WEIGHT_FP16 && c.n_heads < p.grid && (!xcd || kv_in_xs)) {
         constexpr size_t kLdsBytes = 160 * 1024, kReserve = 2048;  // the rest is for the kernel's static LDS
+        // (the plan with parked rows only ever runs items of one head: a wavefront's partial result of one head each)
+        if (!xcd) {
+            b.red_floats = df::kIoWaves * df::kRedStride;
+            b.qkv_floats = 3 * df::kMaxHeadPad;
+        }
         const size_t used = lds_floats() * sizeof(float);
         const size_t row_bytes = static_cast<size_t>(c.dim) * 2;
         int rows = used + kReserve < kLdsBytes ? static_cast<int>((kLdsBytes - kReserve - used) / row_bytes) : 0;
