@@ -45,12 +45,12 @@ HBM_PEAK_GBS = 8000.0
 # (with a note) from the moment the file changes until the two runs are repeated
 # (profiles/persistent_decode_<workload>_pmc_hbm_traffic.txt give the commands, one file per configuration).
 KERNEL_SOURCES = {"k_decode_dataflow": ROOT / "lighterpp_amd" / "csrc" / "dataflow_decode.hip"}
-_MEASURED_SOURCE = "697831f89dc5cb0ef3267e1222f8d13bf41900f3389641bfd269005670210caf"
+_MEASURED_SOURCE = "67451771cb3b70cf8ae783ab64095801eef69448e63cc034229614cbb111aa20"
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    ("c2_tinyllama_1b_fp16", "k_decode_dataflow"): (2.1257e9, _MEASURED_SOURCE),
-    ("c3_llama32_1b_fp16", "k_decode_dataflow"): (2.5144e9, _MEASURED_SOURCE),
-    ("c4_llama32_1b_longctx_fp16", "k_decode_dataflow"): (2.8030e9, _MEASURED_SOURCE),
-    ("c5_llama3_8b_fp16", "k_decode_dataflow"): (1.5186e10, _MEASURED_SOURCE),
+    ("c2_tinyllama_1b_fp16", "k_decode_dataflow"): (2.1260e9, _MEASURED_SOURCE),
+    ("c3_llama32_1b_fp16", "k_decode_dataflow"): (2.5143e9, _MEASURED_SOURCE),
+    ("c4_llama32_1b_longctx_fp16", "k_decode_dataflow"): (2.8022e9, _MEASURED_SOURCE),
+    ("c5_llama3_8b_fp16", "k_decode_dataflow"): (1.5185e10, _MEASURED_SOURCE),
 }
 
 
