@@ -161,9 +161,9 @@ struct Blocks {
     int qkv_by_xcc; // > 0: the stacked [Wq; Wk; Wv] rows are dealt out per XCD, this many KV heads (with their query heads) to each
     int xa_cu_shift;  // att_xcd_item: log2 of the workgroups that share a KV head
     int xa_opc;       // att_xcd_item: attention outputs each of them combines
-    int kv_floats;    // LDS for the K and V rows of a workgroup's share of a context, where they have an area of their own
+    int kv_floats;    // LDS behind the parked rows for what the K and V rows of a workgroup's share of a context need beyond them
     int qkv_floats;   // LDS for this token's q (a row per head of an item), k and v rows
-    int kv_offset;    // where those rows start, in floats from the start of LDS (their own area, or inside xs: see plan_for)
+    int kv_offset;    // where those rows start, in floats from the start of LDS (inside xs: see plan_for)
     int slice_dim;  // columns per slice of a dim-column row (slice_width)
     int down;   // rows of W2
     int cls;    // rows of the classifier
@@ -2131,10 +2131,14 @@ __device__ __forceinline__ void io_attention(Ctx& c, Io& io, const Lds& l, int l
             else if (a.gqa == 2) att_xcd_item<128, 2>(c, io, l, layer);
             else att_xcd_item<128, 1>(c, io, l, layer);
         }
-        // (after the item, through registers.  Requested straight into LDS as soon as the item's inputs are in, the
-        // rows would travel while the scores are formed -- but such a request holds its wavefront until the memory
-        // pipeline has taken it, a microsecond or two for a wavefront's rows, and that is on the item's path: 677 us
-        // per token against 649 at the 1B shape and 600 positions.)
+        // (after the item, through registers: the fetch then runs beside the hand-over to the next phase.  Between the
+        // item's two merges it delays what every other workgroup of the XCD waits for: 770 against 702 us per token
+        // at 8300 positions of the 1B shape.  Requested before the item walks its share and kept in registers until
+        // nothing reads the share any more, which may lie where the rows go: 732-744 us there, 3065 against 3020 at
+        // the 8B shape and 600 positions.  Requested straight into LDS as soon as the item's inputs are in, where the
+        // share leaves the rows' area alone: such a request holds its wavefront until the memory pipeline has taken
+        // it, a microsecond or two for a wavefront's rows, and that is on the item's path: 677 us per token against
+        // 649 at the 1B shape and 600 positions.)
         park_fetch(c, io, l, layer);
         mark(c, io, 4);
         ++c.phase_index;
@@ -2451,12 +2455,16 @@ __global__ __launch_bounds__(kThreads) void k_decode_dataflow(DecodeArgs a, Tagg
     Lds l;
     l.xraw = lds;
     l.xs = l.xraw + dim_pad;
-    l.results = l.xs + b.xs_floats;
+    // (a share of a context whose rows run on beyond xs has the parked rows' area next, then what it needs beyond
+    // that: plan_for)
+    bool share_runs_on = false;
+    if constexpr (kXcd) share_runs_on = t.xa_chunk * a.head_size > b.xs_floats - dim_pad;
+    l.results = l.xs + b.xs_floats + (share_runs_on ? b.park_floats + b.kv_floats : 0);
     l.sc = l.results + b.results_floats;
     l.qkv = l.sc + 2 * kAttScoreFloats;
     l.red = l.qkv + b.qkv_floats;
     l.gather = l.red + b.red_floats;
-    l.park = l.gather + b.gather_floats;
+    l.park = share_runs_on ? l.xs + b.xs_floats : l.gather + b.gather_floats;
     l.kv = lds + b.kv_offset;
     // (the LDS address is taken from the array itself, where the address space is plain to the compiler, and the
     // area's offset added as a number: a pointer that has been through a structure is not reliably traced back)
@@ -2568,10 +2576,12 @@ XcdAttention xcd_attention_for(const lpp_model* m, const df::Blocks& b, int grid
 
 // parking: keep the last gate/up rows of most workgroups in LDS (short contexts); false: every row streams.
 // xa (chunk > 0): the plan of att_xcd_item -- every workgroup holds a share of a KV head's context, with room for
-// four heads in the merge areas.  Where the share's rows fit the part of xs that only the down phase uses (beyond
-// the first dim floats: between two down phases nothing else is staged there), they live there and every workgroup
-// parks gate/up rows in what LDS is left; where they do not, they get an area of their own and nothing is parked.
-// Either way the rows parked do not depend on the position, so a growing context keeps its step lists.
+// four heads in the merge areas, and every workgroup parks gate/up rows in what LDS is left.  The share's rows take
+// LDS that nothing else uses while the item runs: the part of xs that only the down phase uses (beyond the first
+// dim floats: between two down phases nothing else is staged there), then the parked rows' area, which follows xs
+// (the rows of a layer are multiplied before the next layer's share is requested, and fetched after the item has
+// read the share for the last time), then an area of their own for what is still missing.  The rows parked do
+// not depend on the position, so a growing context keeps its step lists until the share no longer fits at all.
 Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr) {
     const lpp_config& c = m->cfg;
     Plan p;
@@ -2617,15 +2627,12 @@ Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr
     b.kv_floats = 0;
     b.kv_offset = 0;
     const bool xcd = xa != nullptr && xa->chunk > 0;
-    bool kv_in_xs = false;
     if (xcd) {
         b.red_floats = df::kIoWaves * df::kMaxAttHeads * df::kRedStride;
-        if (df::kMaxAttHeads * df::kIoWaves * df::kWave > b.gather_floats) b.gather_floats = df::kMaxAttHeads * df::kIoWaves * df::kWave;
+        b.gather_floats = df::kMaxAttHeads * df::kIoWaves * df::kWave;  // (the weights of a share; nothing is gathered)
         b.xa_cu_shift = xa->cu_shift;
         b.xa_opc = xa->opc;
-        kv_in_xs = xa->kv_floats <= b.xs_floats - dim_pad;
-        if (kv_in_xs) b.kv_offset = 2 * dim_pad;  // xraw, then the first dim floats of xs
-        else b.kv_floats = xa->kv_floats;
+        b.kv_offset = 2 * dim_pad;  // xraw, then the first dim floats of xs
     }
     b.slice_dim = df::slice_width(c.dim, chunk_cols);
     b.gu_a = b.gu;
@@ -2639,7 +2646,7 @@ Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr
     };
     // Parked gate/up rows: whatever LDS is left (binary16 models; the workgroups that hold the attention
     // items of a short context, one per query head, park nothing and own that many fewer hidden units).
-    if (parking && c.weight_precision == LPP_WEIGHT_FP16 && c.n_heads < p.grid && (!xcd || kv_in_xs)) {
+    if (parking && c.weight_precision == LPP_WEIGHT_FP16 && c.n_heads < p.grid) {
         constexpr size_t kLdsBytes = 160 * 1024, kReserve = 2048;  // the rest is for the kernel's static LDS
         // (the plan with parked rows only ever runs items of one head: a wavefront's partial result of one head each)
         if (!xcd) {
@@ -2674,8 +2681,13 @@ Plan plan_for(const lpp_model* m, bool parking, const XcdAttention* xa = nullptr
             b.results_floats = (slots + 7) & ~7;
         }
     }
-    if (xcd && !kv_in_xs)
-        b.kv_offset = static_cast<int>(lds_floats()) - b.kv_floats;  // the last area
+    // Order of the areas: xraw, xs, partial sums, scores, q/k/v, merge, gather, parked rows -- unless a share's rows run
+    // on beyond xs: then the parked rows follow xs, whatever the share needs beyond them comes next, and the rest after.
+    // (the kernel tells the two orders apart by the same comparison: chunk positions x head_size floats)
+    if (xcd && xa->kv_floats > b.xs_floats - dim_pad) {
+        const int in_place = b.xs_floats - dim_pad + b.park_floats;
+        b.kv_floats = xa->kv_floats > in_place ? xa->kv_floats - in_place : 0;
+    }
     p.lds_bytes = lds_floats() * sizeof(float);
     return p;
 }
@@ -2958,9 +2970,9 @@ static lpp_status launch_impl(lpp_model* m, const ph::DecodeArgs& a, hipStream_t
     df::Tagged tagged = tagged_of(m, a.uniforms != nullptr, lane_cap);
     // Contexts beyond what the plan with parked gate/up rows covers (one work item per head: the one-pass item's
     // reach for heads of size 64, the cost model's choice otherwise): a KV head's context is split over the
-    // workgroups of its XCD, if the shape allows and the rows fit LDS.  That plan parks no gate/up rows (the rows'
-    // LDS holds the context instead: at the 8B shape the parked rows are worth more than the faster attention, 3087
-    // against 2844 us per token at 100 positions) and shares the step lists of the plan without parking.
+    // workgroups of its XCD, if the shape allows and the rows fit LDS.  That plan parks gate/up rows as well, fewer
+    // of them (its merge areas hold four heads), and has step lists of its own (without parking it shares those of
+    // the plan without).
     constexpr size_t kLdsLimit = 160 * 1024 - 2048;
     Plan xcd_plan = plan_for(m, false);
     XcdAttention xa = {};

@@ -438,9 +438,14 @@ XCD_SPLIT = {
     "hs64_gqa2_16kv": (Shape(2048, 512, 1, 32, 16, 500, 1100, 500000.0, fp16=True, tied=False), (515, 1000)),
     # hidden_dim well above dim: the share's rows live in the part of the staged-activation area that only the down
     # phase uses, and every workgroup parks gate/up rows beside the item (two layers: the down phase overwrites the
-    # rows in between); the last start of the first shape is past what that area holds (3072 positions)
+    # rows in between); the last start of the first shape is past what that area holds (3072 positions): the rows run on
+    # into the parked rows' area
     "hs64_gqa4_8kv_parked": (Shape(2048, 8192, 2, 32, 8, 500, 3300, 500000.0, fp16=True, tied=True), (520, 3066, 3090)),
     "hs128_gqa4_8kv_parked": (Shape(4096, 14336, 2, 32, 8, 500, 1300, 500000.0, fp16=True, tied=False), (620, 1050)),
+    # long contexts with parked rows: the share's rows run on from that area into the parked rows' own (overwritten
+    # by this layer's rows once the item is done, and by the next layer's share after those are multiplied) and, at
+    # the third start, into an area behind them; the last start is past what LDS takes: the plain split
+    "hs64_gqa4_8kv_parked_long": (Shape(2048, 8192, 2, 32, 8, 500, 14100, 500000.0, fp16=True, tied=True), (4100, 8441, 14050, 14090)),
 }
 
 
