@@ -1775,7 +1775,11 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
     const DecodeArgs& a = c.a;
     static_assert(kG <= kMaxAttHeads && kG * kHs <= kIoThreads && kIoWaves % kG == 0, "one thread per (head, dimension) in the merge");
     constexpr int kPieces = kHs / 8;
-    constexpr int kParts = kIoWaves / kG;        // the share's positions in kParts runs of kG wavefronts' worth each
+    // Heads of 64: the scores are MFMA products, every wavefront scores the positions whose values it adds up
+    // and is a part of its own.  Heads of 128: wavefront (head, part) scores a part's positions for one head.
+    constexpr bool kMatrixScores = kHs == 64;
+    constexpr int kPartWaves = kMatrixScores ? 1 : kG;  // wavefronts whose positions make up a part
+    constexpr int kParts = kIoWaves / kPartWaves;       // the share's positions in kParts runs
     constexpr int kStreams = kHs == 64 ? 2 : 1;  // positions a wavefront adds up side by side (a V row is 32 or 64 lanes wide)
     const int lane = fresh_lane();
     int rank = c.rank_in_xcc, xcc = c.xcc, chunk = c.t.xa_chunk;
@@ -1811,6 +1815,14 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
                 const int which = idx / kHs, e = idx - which * kHs;
                 if (which < kG) {
                     l.qkv[which * kMaxHeadPad + e] = in[j];
+                    if constexpr (kMatrixScores) {
+                        // q as a binary16 head and a binary16 remainder (rows kMaxAttHeads.. of the area: heads, then
+                        // remainders): products with the binary16 K rows are then exact, the sums fp32
+                        half_t* q16 = reinterpret_cast<half_t*>(l.qkv + kMaxAttHeads * kMaxHeadPad);
+                        const half_t head = static_cast<half_t>(in[j]);
+                        q16[which * kHs + e] = head;
+                        q16[(kMaxAttHeads + which) * kHs + e] = static_cast<half_t>(in[j] - static_cast<float>(head));
+                    }
                 } else {
                     const uint16_t bits = f32_to_f16_bits(in[j]);
                     char* at = which == kG ? kbase + (e >> 3) * chunk * 16 + lc * 16 + (e & 7) * 2 : vbase + lc * (kHs * 2) + e * 2;
@@ -1828,71 +1840,166 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
     mark(c, io, 2);
 
     if (active) {
-        // Scores: wavefront (h, part) takes head h over the part's positions, a LANE per position: the lane reads
-        // its position's K row (pieces side by side in LDS) and forms the dot product alone; q is read once per
-        // wavefront, four pieces at a time, and kept while the part's passes of 64 positions go by.
-        {
-            const int h = io.iw % kG, part = io.iw / kG;
-            const int first = part * kG * ppw;
-            const int n = min(share_count - first, kG * ppw);  // positions of the part (<= 0: none)
-            float sc[kG];
+        if constexpr (kMatrixScores) {
+            // Scores of the wavefront's own positions for all heads at once: sixteen 4 x 4 products per MFMA, K rows
+            // (a LANE per position, as it reads them below) times q columns (lane & 3: the head), four dimensions
+            // a step; lane 4 b + j ends up with head j's scores of positions 4 b .. 4 b + 3.  Every K row is read
+            // once, whatever the number of heads.
+            typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+            union Piece {
+                uintx4 u;
+                half4_t h[2];
+            };
+            const int w0 = io.iw * ppw;
+            const int hd = lane & 3, p0 = lane & ~3;
+            floatx4 acc_head = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, acc_rest = acc_head;
+            if (x.count > 0) {  // (uniform)
+                const int my = w0 + (lane < x.count ? lane : 0);  // (lanes past the wavefront's positions read its first row; their scores are dropped)
+                const char* q_head = reinterpret_cast<const char*>(l.qkv + kMaxAttHeads * kMaxHeadPad) + hd * (kHs * 2);
+                const char* q_rest = q_head + kMaxAttHeads * kHs * 2;
 #pragma unroll
-            for (int j = 0; j < kG; ++j) sc[j] = 0.0f;
-            if (n > 0) {  // (uniform)
+                for (int i = 0; i < kPieces; ++i) {
+                    Piece kp, qh, qr;
+                    kp.u = *reinterpret_cast<const uintx4*>(kbase + i * chunk * 16 + my * 16);
+                    qh.u = *reinterpret_cast<const uintx4*>(q_head + 16 * i);
+                    qr.u = *reinterpret_cast<const uintx4*>(q_rest + 16 * i);
+                    acc_head = __builtin_amdgcn_mfma_f32_4x4x4f16(kp.h[0], qh.h[0], acc_head, 0, 0, 0);
+                    acc_rest = __builtin_amdgcn_mfma_f32_4x4x4f16(kp.h[0], qr.h[0], acc_rest, 0, 0, 0);
+                    acc_head = __builtin_amdgcn_mfma_f32_4x4x4f16(kp.h[1], qh.h[1], acc_head, 0, 0, 0);
+                    acc_rest = __builtin_amdgcn_mfma_f32_4x4x4f16(kp.h[1], qr.h[1], acc_rest, 0, 0, 0);
+                }
+            }
+            // (over the lanes of a head: 4 apart inside a row of 16, then across the rows)
+            auto over_head = [&](float v, auto op) {
+                v = op(v, dpp_move<0x124>(v));  // row_ror:4
+                v = op(v, dpp_move<0x128>(v));  // row_ror:8
+                v = op(v, lane_xor(v, 16, lane));
+                return op(v, lane_xor(v, 32, lane));
+            };
+            float sc[4];
+            float top = -INFINITY;
 #pragma unroll
-                for (int r = 0; r < kPieces / 4; ++r) {
-                    compiler_fence();
-                    __builtin_amdgcn_sched_barrier(0);
-                    floatx4 qa[4], qb[4];
+            for (int r = 0; r < 4; ++r) {
+                const bool live = hd < kG && p0 + r < x.count;
+                sc[r] = live ? (acc_head[r] + acc_rest[r]) * c.t.inv_sqrt_head : -INFINITY;  // model.cpp:188
+                top = fmaxf(top, sc[r]);
+            }
+            top = over_head(top, [](float a, float b) { return fmaxf(a, b); });
+            // Weights as a binary16 head plus a binary16 remainder, by head, wavefront and position within the
+            // wavefront's 64 (zero past its positions): the values below are MFMA products too.
+            float sum = 0.0f;
+            half4_t w_head, w_rest;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        qa[i] = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + 8 * (4 * r + i));
-                        qb[i] = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + 8 * (4 * r + i) + 4);
-                    }
+            for (int r = 0; r < 4; ++r) {
+                const float w = (sc[r] == -INFINITY) ? 0.0f : exp_fast(sc[r] - top);
+                sum += w;
+                w_head[r] = static_cast<_Float16>(w);
+                w_rest[r] = static_cast<_Float16>(w - static_cast<float>(w_head[r]));
+            }
+            if (hd < kG) {
+                half4_t* w16 = reinterpret_cast<half4_t*>(weights) + ((hd * kIoWaves + io.iw) * kWave + p0) / 4;
+                w16[0] = w_head;
+                w16[kMaxAttHeads * kIoWaves * kWave / 4] = w_rest;
+            }
+            sum = over_head(sum, [](float a, float b) { return a + b; });
+            if (lane < kG) {  // (lane = head)
+                stats[(lane * kParts + io.iw) * 2] = top;
+                stats[(lane * kParts + io.iw) * 2 + 1] = sum;
+            }
+            compiler_fence();  // (the weights are read back by this wavefront alone)
+        } else {
+            // Scores: wavefront (h, part) takes head h over the part's positions, a LANE per position: the lane reads
+            // its position's K row (pieces side by side in LDS) and forms the dot product alone; q is read once per
+            // wavefront, four pieces at a time, and kept while the part's passes of 64 positions go by.
+            {
+                const int h = io.iw % kG, part = io.iw / kG;
+                const int first = part * kG * ppw;
+                const int n = min(share_count - first, kG * ppw);  // positions of the part (<= 0: none)
+                float sc[kG];
 #pragma unroll
-                    for (int j = 0; j < kG; ++j) {
-                        if (j * kWave < n) {  // (uniform)
-                            const int p = j * kWave + lane;
-                            const int my = first + (p < n ? p : 0);  // (lanes past the part read its first row; their scores are dropped)
-                            uintx4 kbits[4];
+                for (int j = 0; j < kG; ++j) sc[j] = 0.0f;
+                if (n > 0) {  // (uniform)
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) kbits[i] = *reinterpret_cast<const uintx4*>(kbase + (4 * r + i) * chunk * 16 + my * 16);
-                            __builtin_amdgcn_sched_barrier(0);  // (left alone, the scheduler pairs every read with its use)
-                            float part4[4];
+                    for (int r = 0; r < kPieces / 4; ++r) {
+                        compiler_fence();
+                        __builtin_amdgcn_sched_barrier(0);
+                        floatx4 qa[4], qb[4];
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) part4[i] = dot8(kbits[i], qa[i], qb[i], 0.0f);
-                            sc[j] += (part4[0] + part4[1]) + (part4[2] + part4[3]);
-                            // (the sum is wanted HERE: without a use in place the multiply-adds are sunk to where the
-                            // score is first needed, behind every other round's reads, and all the rows wait in registers)
-                            asm volatile("" : "+v"(sc[j]));
+                        for (int i = 0; i < 4; ++i) {
+                            qa[i] = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + 8 * (4 * r + i));
+                            qb[i] = *reinterpret_cast<const floatx4*>(l.qkv + h * kMaxHeadPad + 8 * (4 * r + i) + 4);
+                        }
+#pragma unroll
+                        for (int j = 0; j < kG; ++j) {
+                            if (j * kWave < n) {  // (uniform)
+                                const int p = j * kWave + lane;
+                                const int my = first + (p < n ? p : 0);  // (lanes past the part read its first row; their scores are dropped)
+                                uintx4 kbits[4];
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) kbits[i] = *reinterpret_cast<const uintx4*>(kbase + (4 * r + i) * chunk * 16 + my * 16);
+                                __builtin_amdgcn_sched_barrier(0);  // (left alone, the scheduler pairs every read with its use)
+                                float part4[4];
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) part4[i] = dot8(kbits[i], qa[i], qb[i], 0.0f);
+                                sc[j] += (part4[0] + part4[1]) + (part4[2] + part4[3]);
+                                // (the sum is wanted HERE: without a use in place the multiply-adds are sunk to where the
+                                // score is first needed, behind every other round's reads, and all the rows wait in registers)
+                                asm volatile("" : "+v"(sc[j]));
+                            }
                         }
                     }
                 }
-            }
-            float top = -INFINITY;
+                float top = -INFINITY;
 #pragma unroll
-            for (int j = 0; j < kG; ++j) {
-                sc[j] = (j * kWave + lane < n) ? sc[j] * c.t.inv_sqrt_head : -INFINITY;  // model.cpp:188
-                top = fmaxf(top, sc[j]);
-            }
-            top = wave_max(top);
-            float sum = 0.0f;
+                for (int j = 0; j < kG; ++j) {
+                    sc[j] = (j * kWave + lane < n) ? sc[j] * c.t.inv_sqrt_head : -INFINITY;  // model.cpp:188
+                    top = fmaxf(top, sc[j]);
+                }
+                top = wave_max(top);
+                float sum = 0.0f;
 #pragma unroll
-            for (int j = 0; j < kG; ++j) {
-                const float w = (sc[j] == -INFINITY) ? 0.0f : exp_fast(sc[j] - top);
-                sum += w;
-                if (j * kWave + lane < kG * ppw) weights[h * chunk + first + j * kWave + lane] = w;
+                for (int j = 0; j < kG; ++j) {
+                    const float w = (sc[j] == -INFINITY) ? 0.0f : exp_fast(sc[j] - top);
+                    sum += w;
+                    if (j * kWave + lane < kG * ppw) weights[h * chunk + first + j * kWave + lane] = w;
+                }
+                sum = wave_sum(sum);
+                if (lane == 0) {
+                    stats[(h * kParts + part) * 2] = top;
+                    stats[(h * kParts + part) * 2 + 1] = sum;
+                }
             }
-            sum = wave_sum(sum);
-            if (lane == 0) {
-                stats[(h * kParts + part) * 2] = top;
-                stats[(h * kParts + part) * 2 + 1] = sum;
-            }
+            io_sync(c.ctl, io);
         }
-        io_sync(c.ctl, io);
         // Values: wavefront w takes its own xa_ppw positions for all heads; lane (stream, pair) adds up dimensions
         // 2 pair, 2 pair + 1 over positions stream, stream + kStreams, ...: four positions' values and weights are
         // requested before the first is used.
+        if constexpr (kMatrixScores) {
+            // Values: out[head][dimension] = sum over the wavefront's positions of weight x V, four positions a step:
+            // weight rows (lane & 3: the head, the same in all sixteen products) times V columns (a LANE per
+            // dimension, which reads its 2 bytes of four rows); lane d ends up with dimension d of every head.
+            typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+            const int w0 = io.iw * ppw;
+            floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            const half4_t* w16 = reinterpret_cast<const half4_t*>(weights) + (((lane & 3) * kIoWaves + io.iw) * kWave) / 4;
+            const char* vcol = vbase + lane * 2;
+#pragma unroll 4
+            for (int k0 = 0; k0 < x.count; k0 += 4) {  // (uniform)
+                half4_t v;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    // (what lies past the wavefront's positions may be anything, NaN included: its weight is zero, and
+                    // the value is taken from a row that has one)
+                    const int at = w0 + (k0 + k < x.count ? k0 + k : 0);
+                    v[k] = *reinterpret_cast<const _Float16*>(vcol + at * (kHs * 2));
+                }
+                const half4_t wh = w16[k0 / 4], wr = w16[kMaxAttHeads * kIoWaves * kWave / 4 + k0 / 4];
+                acc = __builtin_amdgcn_mfma_f32_4x4x4f16(wh, v, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_4x4x4f16(wr, v, acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int h = 0; h < kG; ++h) l.red[(io.iw * kMaxAttHeads + h) * kRedStride + lane] = acc[h];
+        } else {
         float out[kG][2];
 #pragma unroll
         for (int h = 0; h < kG; ++h) out[h][0] = out[h][1] = 0.0f;
@@ -1946,6 +2053,7 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
                 }
             }
         }
+        }
     }
     mark(c, io, 7);
     io_sync(c.ctl, io);
@@ -1970,7 +2078,7 @@ __device__ __forceinline__ void att_xcd_item(Ctx& c, Io& io, const Lds& l, int l
             const float f = (ptop[q] == -INFINITY) ? 0.0f : exp_fast(ptop[q] - all);
             ls += psum[q] * f;
 #pragma unroll
-            for (int w = q * kG; w < (q + 1) * kG; ++w) o += wout[w] * f;  // (a part's wavefronts: q * kG ..)
+            for (int w = q * kPartWaves; w < (q + 1) * kPartWaves; ++w) o += wout[w] * f;  // (a part's wavefronts)
         }
         u64* mine = part_all + static_cast<size_t>(rank) * c.t.near_part_stride + h * (kHs + 2);
         publish_near(mine + e, o, tag_out);
